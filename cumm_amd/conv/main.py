@@ -1,0 +1,190 @@
+"""``ConvMainUnitTest``: the sparse-convolution operator surface (implicit_gemm2).
+
+Host prelude of the reference's generated ``implicit_gemm2``
+(cumm/conv/main.py:483-745 with cumm/conv/nvrtc_code.py:20-197): validation,
+m/n/k, operand permutation by op type, source-pointer rules and workspace; the
+launch goes through the C ABI (``cumm_hip_sparse_conv``).  Only mask-based
+sparse convolution (``mask_sparse``) is built; dense NHWC convolution is not.
+"""
+import ctypes
+from typing import List, Tuple
+
+from .. import _capi
+from ..gemm.main import (INT_MAX, _check_device, _check_shape, _enum_int, _ptr, desp_from_c,
+                         desp_to_c)
+from ..tensorview import Tensor, empty, uint8
+from ..tensorview.gemm import (ConvAlgoDesp, ConvOpType, ConvParams, gemm_abc_012_to_iwo,
+                               implicit_gemm_mnk)
+
+
+def conv_desp_to_c(desp: ConvAlgoDesp) -> _capi.ConvDesc:
+    c = _capi.ConvDesc()
+    c.gemm = desp_to_c(desp)
+    c.ndim = desp.ndim
+    c.op_type = _enum_int(desp.op_type)
+    c.mask_sparse = int(desp.mask_sparse)
+    c.increment_k_first = int(desp.increment_k_first)
+    c.dynamic_mask = int(desp.dynamic_mask)
+    c.is_int8_inference = int(desp.is_int8_inference)
+    return c
+
+
+class ConvMainUnitTest:
+    """Static operator functions, as the reference's pybind class."""
+
+    @staticmethod
+    def get_all_conv_algo_desp() -> List[ConvAlgoDesp]:
+        """cumm/conv/main.py:983-1050 of the reference."""
+        L = _capi.lib()
+        n = L.cumm_hip_list_conv_algos(None, 0)
+        arr = (_capi.ConvDesc * n)()
+        L.cumm_hip_list_conv_algos(arr, n)
+        out = []
+        for i in range(n):
+            d = ConvAlgoDesp(arr[i].ndim, ConvOpType(arr[i].op_type))
+            desp_from_c(arr[i].gemm, d)
+            d.mask_sparse = bool(arr[i].mask_sparse)
+            d.increment_k_first = bool(arr[i].increment_k_first)
+            d.dynamic_mask = bool(arr[i].dynamic_mask)
+            d.is_int8_inference = bool(arr[i].is_int8_inference)
+            out.append(d)
+        return out
+
+    @staticmethod
+    def extract_mnk(op_type, N: int, C: int, K: int, kernel_volume: int, in_prod: int,
+                    out_prod: int, mask_sparse: bool) -> Tuple[int, int, int]:
+        """cumm/conv/main.py:467-481 of the reference."""
+        return tuple(implicit_gemm_mnk(op_type, N, C, K, kernel_volume, in_prod, out_prod,
+                                       mask_sparse))
+
+    @staticmethod
+    def implicit_gemm2(params: ConvParams) -> None:
+        desp = params.conv_algo_desp
+        if not desp.mask_sparse:
+            raise RuntimeError("can't find any suitable algo for your parameters. "
+                               "(dense convolution is not built)")
+        op_type = ConvOpType(desp.op_type)
+        inp, weight, output = params.input, params.weight, params.output
+        bias, scale, output_add = params.bias, params.scale, params.output_add
+        indices, mask, mask_argsort = params.indices, params.mask, params.mask_argsort
+        mask_output, mask_width = params.mask_output, params.mask_width
+        split_k_slices = params.split_k_slices
+        if inp.ndim != 2:
+            raise RuntimeError("error")
+        if weight.ndim != 3:
+            raise RuntimeError("error")
+        if output.ndim != 2:
+            raise RuntimeError("error")
+        if not (desp.split_k_serial or desp.split_k_parallel) and split_k_slices > 1:
+            raise RuntimeError("algo don't support splitk but you provide split_k_slices > 1.")
+        K = weight.dim(0)
+        C = inp.dim(1)
+        if output.dim(1) != K:
+            raise RuntimeError("error")
+        _check_device(inp, weight, output, bias, scale, output_add, indices, mask, mask_argsort,
+                      mask_output)
+        inv = gemm_abc_012_to_iwo(op_type)
+        iwo = [inp, weight, output]
+        a_ten, b_ten, c_ten = iwo[inv[0]], iwo[inv[1]], iwo[inv[2]]
+        if not desp.is_int8_inference:
+            if not output_add.empty():
+                raise ValueError("only int8 inference support output_add not empty ")
+        else:
+            if bias.empty() or scale.empty():
+                raise RuntimeError("int8 inference must have both scale and bias")
+        if output_add.empty():
+            if desp.is_int8_inference or bias.empty():
+                d_ten = c_ten
+            else:
+                d_ten = bias
+        else:
+            if output_add.dtype != output.dtype or output_add.shape != output.shape:
+                raise RuntimeError("output and output_add must have same dtype and shape")
+            d_ten = output_add
+        if op_type == ConvOpType.BackwardWeight:
+            if not (mask_width > 0 and mask_width % desp.tile_shape[2] == 0):
+                raise RuntimeError("error")
+        if indices.empty() or mask.empty() or mask_argsort.empty():
+            raise RuntimeError("error")
+        kernel_volume = weight.dim(1)
+        _check_shape(indices, [kernel_volume, -1])
+        N = indices.dim(1)
+        if weight.dim(2) != C:
+            raise RuntimeError("error")
+        if op_type == ConvOpType.BackwardWeight:
+            if N != output.dim(0):
+                raise RuntimeError("error")
+            if N * C * b_ten.itemsize >= INT_MAX or N * K * a_ten.itemsize >= INT_MAX:
+                raise RuntimeError("your data exceed int32 range.")
+        elif op_type == ConvOpType.Forward:
+            if N != output.dim(0):
+                raise RuntimeError("error")
+            if N * C * a_ten.itemsize >= INT_MAX:
+                raise RuntimeError("your data exceed int32 range.")
+        else:
+            if N * K * a_ten.itemsize >= INT_MAX:
+                raise RuntimeError("your data exceed int32 range.")
+            if N != inp.dim(0):
+                raise RuntimeError("error")
+        mnk = implicit_gemm_mnk(op_type, N, C, K, kernel_volume, -1, -1, True)
+        if not desp.supported(mnk[0], mnk[1], mnk[2], C, K, mask_width):
+            raise RuntimeError("error")
+        if mask_argsort.dim(0) < N:
+            raise RuntimeError("error")
+        if op_type == ConvOpType.BackwardWeight:
+            if mask.dim(0) < (N + mask_width - 1) // mask_width:
+                raise RuntimeError("error")
+        elif mask.dim(0) < N:
+            raise RuntimeError("error")
+        for t in (inp, weight, output):
+            if not t.is_contiguous():
+                raise ValueError("input, weight and output must be contiguous")
+        if (not bias.empty() and bias.dim(0) != K) or (not scale.empty() and scale.dim(0) != K):
+            raise RuntimeError("bias and scale must have one entry per output channel")
+
+        workspace_size = desp.query_conv_workspace_size(mnk[0], mnk[1], mnk[2], split_k_slices,
+                                                        kernel_volume)
+        if workspace_size > 0:
+            if not params.workspace.empty():
+                if params.workspace.nbytes < workspace_size:
+                    raise RuntimeError("workspace at least %d bytes." % workspace_size)
+            else:
+                # as in the reference the allocation stays in the caller's params object
+                params.workspace = empty([workspace_size], uint8, 0)
+        workspace = params.workspace
+
+        args = _capi.SparseConvArgs()
+        args.ptr_A, args.ptr_B, args.ptr_C = _ptr(a_ten), _ptr(b_ten), _ptr(c_ten)
+        args.ptr_D = _ptr(d_ten)
+        args.alpha, args.beta = params.alpha, params.beta
+        args.act_alpha, args.act_beta = params.act_alpha, params.act_beta
+        args.act_type = _enum_int(params.act_type)
+        args.split_k_slices = split_k_slices
+        args.workspace = _ptr(workspace)
+        args.workspace_bytes = 0 if workspace.empty() else workspace.nbytes
+        args.mask_ptr = _ptr(mask)
+        if op_type == ConvOpType.Forward and not mask_output.empty():
+            tiles = (N + desp.tile_shape[0] - 1) // desp.tile_shape[0]
+            if mask_output.dim(0) < tiles:
+                raise RuntimeError("mask_output needs one word per tile of tile_shape[0] positions")
+            args.mask_out_ptr = _ptr(mask_output)
+        args.indice_ptr = _ptr(indices)
+        args.mask_argsort_ptr = _ptr(mask_argsort)
+        args.mask_filter = params.mask_filter & 0xFFFFFFFF
+        args.reverse_mask = int(bool(params.reverse_mask))
+        args.mask_width = mask_width
+        args.ndim, args.N, args.C, args.K = desp.ndim, N, C, K
+        args.kernel_volume = kernel_volume
+        args.d_is_bias = int(not bias.empty())
+        args.bias_pointer = _ptr(bias)
+        args.scale_pointer = _ptr(scale)
+        args.rows_in, args.rows_out = inp.dim(0), output.dim(0)
+        cdesc = conv_desp_to_c(desp)
+        name = repr(desp) if params.timer.enable else ""
+        if name:
+            params.timer.record(name, params.stream)
+        status = _capi.lib().cumm_hip_sparse_conv(ctypes.byref(cdesc), ctypes.byref(args),
+                                                  params.stream)
+        if name:
+            params.timer.record(name, params.stream)
+        _capi.check(status)

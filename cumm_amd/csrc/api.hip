@@ -1,0 +1,543 @@
+// C ABI of libcummhip.so: argument checks, kernel selection and launches.
+#include "../../include/cumm_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "launch.h"
+
+using namespace cummhip;
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char *fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+  return fail(CUMM_HIP_ERUNTIME, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                   \
+  do {                                                  \
+    hipError_t e_ = (expr);                             \
+    if (e_ != hipSuccess) return hip_fail(e_, #expr);   \
+  } while (0)
+
+bool is_float16_like(int dt) { return dt == CUMM_HIP_F16 || dt == CUMM_HIP_BF16; }
+int elem_bytes(int dt) { return dt == CUMM_HIP_S8 ? 1 : (is_float16_like(dt) ? 2 : 4); }
+int per_vec(int dt) { return 16 / elem_bytes(dt); }
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// fragments per lane per channel chunk for a contraction of c_in elements
+int pick_ks(int c_in, int dt) {
+  const int row_bytes = c_in * elem_bytes(dt);
+  if (row_bytes <= 64) return 1;
+  if (row_bytes <= 128) return 2;
+  return 4;
+}
+
+bool same_dtype3(const CummHipGemmDesc &d) {
+  return d.dtype_a == d.dtype_b && d.dtype_a == d.dtype_c &&
+         (is_float16_like(d.dtype_a) || d.dtype_a == CUMM_HIP_S8);
+}
+
+bool acc_ok(const CummHipGemmDesc &d) {
+  if (d.dtype_a == CUMM_HIP_S8) return d.dacc == CUMM_HIP_S32 && d.dcomp == CUMM_HIP_F32;
+  return d.dacc == CUMM_HIP_F32 && d.dcomp == CUMM_HIP_F32;
+}
+
+hipError_t launch_rowgemm(int dt, int tm, int tn, int ks, bool wt, const RowGemmParams &p,
+                          hipStream_t s) {
+  switch (dt) {
+  case CUMM_HIP_F16: return launch_rowgemm_f16(tm, tn, ks, wt, p, s);
+  case CUMM_HIP_BF16: return launch_rowgemm_bf16(tm, tn, ks, wt, p, s);
+  case CUMM_HIP_S8: return launch_rowgemm_s8(tm, tn, ks, wt, p, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_tilegemm(int dt, int tm, int tn, bool xk, bool yk, const TileGemmParams &p,
+                           dim3 grid, hipStream_t s) {
+  switch (dt) {
+  case CUMM_HIP_F16: return launch_tilegemm_f16(tm, tn, xk, yk, p, grid, s);
+  case CUMM_HIP_BF16: return launch_tilegemm_bf16(tm, tn, xk, yk, p, grid, s);
+  case CUMM_HIP_S8: return launch_tilegemm_s8(tm, tn, xk, yk, p, grid, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+constexpr int kSpinLimit = 1 << 24;
+
+// which kernel family serves a GEMM descriptor: 1 rowgemm, 2 tilegemm, 0 none
+int gemm_family(const CummHipGemmDesc &d) {
+  if (!same_dtype3(d) || !acc_ok(d)) return 0;
+  const int tm = d.tile_shape[0], tn = d.tile_shape[1], tk = d.tile_shape[2];
+  const int mk = d.dtype_a == CUMM_HIP_S8 ? 64 : 32;
+  if (tk != mk) return 0;
+  if (d.split_k_parallel) return 0;
+  if (d.shuffle_type == CUMM_HIP_SHUFFLE_AC) {
+    if (d.trans_a || d.trans_c || d.split_k_serial) return 0;
+    return rowgemm_has_tile(tm, tn) ? 1 : 0;
+  }
+  if (d.shuffle_type == CUMM_HIP_SHUFFLE_AB) {
+    if (!d.trans_a || d.trans_b || d.trans_c) return 0;
+    return tilegemm_has_tile(tm, tn) ? 2 : 0;
+  }
+  if (d.shuffle_type == CUMM_HIP_NO_SHUFFLE) return tilegemm_has_tile(tm, tn) ? 2 : 0;
+  return 0;
+}
+
+int conv_family(const CummHipConvDesc &c) {
+  const CummHipGemmDesc &d = c.gemm;
+  if (!c.mask_sparse || c.dynamic_mask) return 0;
+  if (!same_dtype3(d) || !acc_ok(d)) return 0;
+  if (d.split_k_parallel) return 0;
+  const int tm = d.tile_shape[0], tn = d.tile_shape[1], tk = d.tile_shape[2];
+  const int mk = d.dtype_a == CUMM_HIP_S8 ? 64 : 32;
+  if (tk != mk) return 0;
+  if (c.is_int8_inference && (d.dtype_a != CUMM_HIP_S8 || c.op_type != CUMM_HIP_OP_FORWARD)) return 0;
+  if (c.op_type == CUMM_HIP_OP_FORWARD || c.op_type == CUMM_HIP_OP_BACKWARD_INPUT) {
+    if (d.split_k_serial) return 0;
+    return rowgemm_has_tile(tm, tn) ? 1 : 0;
+  }
+  if (c.op_type == CUMM_HIP_OP_BACKWARD_WEIGHT) {
+    if (d.dtype_a == CUMM_HIP_S8) return 0;
+    return tilegemm_has_tile(tm, tn) ? 2 : 0;
+  }
+  return 0;
+}
+
+void fill_gemm_desc(CummHipGemmDesc &d, int dt, int ta, int tb, int tc, int tm, int tn, int shuffle,
+                    int splitk) {
+  std::memset(&d, 0, sizeof(d));
+  d.dtype_a = d.dtype_b = d.dtype_c = dt;
+  d.dacc = dt == CUMM_HIP_S8 ? CUMM_HIP_S32 : CUMM_HIP_F32;
+  d.dcomp = CUMM_HIP_F32;
+  d.trans_a = ta; d.trans_b = tb; d.trans_c = tc;
+  const int tk = dt == CUMM_HIP_S8 ? 64 : 32;
+  d.tile_shape[0] = tm; d.tile_shape[1] = tn; d.tile_shape[2] = tk;
+  d.num_stage = 2;
+  d.shuffle_type = shuffle;
+  d.split_k_serial = splitk;
+  d.split_k_parallel = 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *cumm_hip_last_error(void) { return g_err.c_str(); }
+
+int cumm_hip_gemm_supported(const CummHipGemmDesc *desc) { return desc && gemm_family(*desc) != 0; }
+int cumm_hip_conv_supported(const CummHipConvDesc *desc) { return desc && conv_family(*desc) != 0; }
+
+int cumm_hip_list_gemm_algos(CummHipGemmDesc *out, int cap) {
+  std::vector<CummHipGemmDesc> v;
+  const int dts[3] = {CUMM_HIP_F16, CUMM_HIP_BF16, CUMM_HIP_S8};
+  const int row_tiles[4][2] = {{64, 64}, {128, 64}, {64, 128}, {128, 128}};
+  const int sq_tiles[2][2] = {{64, 64}, {128, 128}};
+  for (int dt : dts) {
+    for (auto &t : row_tiles)
+      for (int tb = 0; tb < 2; ++tb) {
+        CummHipGemmDesc d;
+        fill_gemm_desc(d, dt, 0, tb, 0, t[0], t[1], CUMM_HIP_SHUFFLE_AC, 0);
+        d.warp_tile_shape[0] = t[0] / 4; d.warp_tile_shape[1] = t[1]; d.warp_tile_shape[2] = d.tile_shape[2];
+        v.push_back(d);
+      }
+    for (auto &t : sq_tiles) {
+      for (int ta = 0; ta < 2; ++ta)
+        for (int tb = 0; tb < 2; ++tb)
+          for (int tc = 0; tc < 2; ++tc) {
+            CummHipGemmDesc d;
+            fill_gemm_desc(d, dt, ta, tb, tc, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 1);
+            d.warp_tile_shape[0] = t[0] / 2; d.warp_tile_shape[1] = t[1] / 2; d.warp_tile_shape[2] = d.tile_shape[2];
+            v.push_back(d);
+          }
+      CummHipGemmDesc d;
+      fill_gemm_desc(d, dt, 1, 0, 0, t[0], t[1], CUMM_HIP_SHUFFLE_AB, 1);
+      d.warp_tile_shape[0] = t[0] / 2; d.warp_tile_shape[1] = t[1] / 2; d.warp_tile_shape[2] = d.tile_shape[2];
+      v.push_back(d);
+    }
+  }
+  for (int i = 0; i < (int)v.size() && i < cap; ++i) out[i] = v[i];
+  return (int)v.size();
+}
+
+int cumm_hip_list_conv_algos(CummHipConvDesc *out, int cap) {
+  std::vector<CummHipConvDesc> v;
+  const int row_tiles[4][2] = {{64, 64}, {128, 64}, {64, 128}, {128, 128}};
+  const int sq_tiles[2][2] = {{64, 64}, {128, 128}};
+  auto base = [](CummHipConvDesc &c, int op) {
+    c.ndim = 3; c.op_type = op; c.mask_sparse = 1; c.increment_k_first = 1; c.dynamic_mask = 0;
+    c.is_int8_inference = 0;
+  };
+  const int fdts[2] = {CUMM_HIP_F16, CUMM_HIP_BF16};
+  for (int dt : fdts) {
+    for (auto &t : row_tiles) {
+      // forward: A = input [N,C] row major, B = weight [K, kv*C] ("tn"), C = output
+      CummHipConvDesc c;
+      fill_gemm_desc(c.gemm, dt, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
+      base(c, CUMM_HIP_OP_FORWARD);
+      v.push_back(c);
+      // backward input: A = dOut [N,K], B = weight viewed [kv*K, C] ("tt")
+      fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
+      base(c, CUMM_HIP_OP_BACKWARD_INPUT);
+      v.push_back(c);
+    }
+    for (auto &t : sq_tiles) {
+      // backward weight: A = dOut^T [K,N] ("n"), B = input [N, kv*C] ("t"), serial split-K
+      CummHipConvDesc c;
+      fill_gemm_desc(c.gemm, dt, 1, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 1);
+      c.gemm.warp_tile_shape[0] = t[0] / 2; c.gemm.warp_tile_shape[1] = t[1] / 2; c.gemm.warp_tile_shape[2] = 32;
+      base(c, CUMM_HIP_OP_BACKWARD_WEIGHT);
+      v.push_back(c);
+    }
+  }
+  for (auto &t : row_tiles) {
+    for (int s8inf = 0; s8inf < 2; ++s8inf) {
+      CummHipConvDesc c;
+      fill_gemm_desc(c.gemm, CUMM_HIP_S8, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 64;
+      base(c, CUMM_HIP_OP_FORWARD);
+      c.is_int8_inference = s8inf;
+      v.push_back(c);
+    }
+  }
+  for (int i = 0; i < (int)v.size() && i < cap; ++i) out[i] = v[i];
+  return (int)v.size();
+}
+
+// ---------------------------------------------------------------------------------------------
+int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *stream_) {
+  if (!desc || !a) return fail(CUMM_HIP_EINVAL, "null descriptor or arguments");
+  const CummHipGemmDesc &d = *desc;
+  const int fam = gemm_family(d);
+  if (fam == 0) return fail(CUMM_HIP_ENOALGO, "can't find any suitable algo for your parameters.");
+  hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+  const int dt = d.dtype_a;
+  const int pv = per_vec(dt);
+  if (a->m < 0 || a->n < 0 || a->k < 0) return fail(CUMM_HIP_EINVAL, "negative m, n or k");
+  if (a->m == 0 || a->n == 0) return CUMM_HIP_OK;
+  if (!a->ptr_A || !a->ptr_B || !a->ptr_C) return fail(CUMM_HIP_ERUNTIME, "a,b,c must not empty");
+  if (!aligned16(a->ptr_A) || !aligned16(a->ptr_B) || !aligned16(a->ptr_C) ||
+      (a->ptr_D && !aligned16(a->ptr_D)))
+    return fail(CUMM_HIP_EINVAL, "operand pointers must be 16-byte aligned");
+  if (!d.split_k_serial && a->split_k_slices > 1)
+    return fail(CUMM_HIP_ERUNTIME, "algo don't support splitk but you provide split_k_slices > 1.");
+  if (a->split_k_slices < 1) return fail(CUMM_HIP_EINVAL, "split_k_slices must be >= 1");
+  const void *ptr_D = a->ptr_D ? a->ptr_D : a->ptr_C;
+  const int64_t ldd = a->ptr_D ? a->stride_D : a->stride_C;
+
+  if (fam == 1) {
+    // ShuffleAC: C[c_inds[i]] = act(alpha * A[a_inds[i]] @ op(B) + beta * D[c_inds[i]])
+    if (!a->indiceBorC) return fail(CUMM_HIP_ERUNTIME, "a_inds,c_inds tensor must not empty");
+    if (a->k % pv || a->n % pv || a->stride_A % pv || a->stride_B % pv || a->stride_C % pv || ldd % pv)
+      return fail(CUMM_HIP_EINVAL, "this m, n, k isn't supported due to misaligned contiguous dim.");
+    RowGemmParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.A = a->ptr_A; p.W = a->ptr_B; p.C = a->ptr_C; p.D = ptr_D;
+    p.out_rows = a->indiceBorC;
+    p.gather = a->indiceA;
+    p.lda = a->stride_A; p.ldc = a->stride_C; p.ldd = ldd;
+    if (d.trans_b) {  // B stored [n, k]
+      p.w_stride_n = a->stride_B; p.w_stride_c = 1;
+    } else {          // B stored [k, n]
+      p.w_stride_n = 1; p.w_stride_c = a->stride_B;
+    }
+    p.w_stride_k = 0;
+    p.n_pos = a->m; p.n_idx = a->m; p.rows_a = a->rows_A; p.rows_c = a->rows_C;
+    p.c_in = a->k; p.k_out = a->n; p.kv = 1;
+    p.mask_filter = 0xffffffffu;
+    p.gather_by_pos = 1;
+    p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act_beta = a->act_beta;
+    p.act = a->act_type;
+    p.read_source = a->beta != 0.0f;
+    if (p.read_source && ldd != 0 && a->indiceD == nullptr && a->ptr_D != nullptr)
+      return fail(CUMM_HIP_EINVAL, "a 2-D D needs the scatter indices (indiceD)");
+    p.xcd_swizzle = 0;
+    hipError_t e = launch_rowgemm(dt, d.tile_shape[0], d.tile_shape[1], pick_ks(a->k, dt), !d.trans_b, p, stream);
+    if (e != hipSuccess) return hip_fail(e, "gather-GEMM-scatter launch");
+    return CUMM_HIP_OK;
+  }
+
+  // tilegemm: D[m][n] = sum_k Y[m][k] X[n][k]
+  TileGemmParams p;
+  std::memset(&p, 0, sizeof(p));
+  // With trans_c the prelude has already swapped the operands (C^T = B^T A^T,
+  // cumm/gemm/nvrtc_code.py:62-67 of the reference): A, B, m, n arrive swapped and only the
+  // effective transposes remain to be derived from the descriptor.
+  bool ta = d.trans_a, tb = d.trans_b;
+  if (d.trans_c) {
+    const bool nta = !d.trans_b, ntb = !d.trans_a;
+    ta = nta; tb = ntb;
+  }
+  const void *A = a->ptr_A, *B = a->ptr_B;
+  const int64_t lda = a->stride_A, ldb = a->stride_B;
+  const int m = a->m, n = a->n;
+  if (a->stride_C % 4 || ldd % 4 || n % 4)
+    return fail(CUMM_HIP_EINVAL, "this m, n, k isn't supported due to misaligned contiguous dim.");
+  if (lda % pv || ldb % pv)
+    return fail(CUMM_HIP_EINVAL, "this m, n, k isn't supported due to misaligned contiguous dim.");
+  if ((ta ? m : a->k) % pv || (tb ? a->k : n) % pv)
+    return fail(CUMM_HIP_EINVAL, "this m, n, k isn't supported due to misaligned contiguous dim.");
+  p.Y = A; p.ldy = lda;
+  p.X = B; p.ldx = ldb;
+  p.C = a->ptr_C; p.D = ptr_D; p.ldc = a->stride_C; p.ldd = ldd;
+  p.m = m; p.n = n; p.k = a->k; p.kv = 1; p.mask_filter = 0xffffffffu;
+  p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act = a->act_type;
+  p.split_k = a->split_k_slices;
+  p.spin_limit = kSpinLimit;
+  p.rows_x = 0x7fffffff; p.rows_y = 0x7fffffff;
+  bool xk, yk;
+  if (d.shuffle_type == CUMM_HIP_SHUFFLE_AB) {
+    if (!a->indiceA || !a->indiceBorC) return fail(CUMM_HIP_ERUNTIME, "a_inds,b_inds tensor must not empty");
+    yk = false; xk = false;
+    p.y_gather = a->indiceA; p.x_gather = a->indiceBorC;
+    p.rows_y = a->rows_A; p.rows_x = a->rows_B;
+  } else {
+    yk = !ta;  // A stored [m, k]
+    xk = tb;   // B stored [n, k]
+  }
+  const int tm = d.tile_shape[0], tn = d.tile_shape[1];
+  dim3 grid((m + tm - 1) / tm, (n + tn - 1) / tn, p.split_k);
+  if (p.split_k > 1) {
+    const size_t need = sizeof(int32_t) * grid.x * grid.y;
+    if (!a->workspace || a->workspace_bytes < need)
+      return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
+    HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
+    p.sem = reinterpret_cast<int32_t *>(a->workspace);
+  }
+  hipError_t e = launch_tilegemm(dt, tm, tn, xk, yk, p, grid, stream);
+  if (e != hipSuccess) return hip_fail(e, "GEMM launch");
+  return CUMM_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a, void *stream_) {
+  if (!desc || !a) return fail(CUMM_HIP_EINVAL, "null descriptor or arguments");
+  const CummHipConvDesc &c = *desc;
+  const CummHipGemmDesc &d = c.gemm;
+  const int fam = conv_family(c);
+  if (fam == 0) return fail(CUMM_HIP_ENOALGO, "can't find any suitable algo for your parameters.");
+  hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+  const int dt = d.dtype_a;
+  const int pv = per_vec(dt);
+  const int kv = a->kernel_volume;
+  if (a->N < 0 || a->C <= 0 || a->K <= 0 || kv <= 0) return fail(CUMM_HIP_EINVAL, "bad N, C, K or kernel volume");
+  if (kv > 32) return fail(CUMM_HIP_EINVAL, "kernel volume > 32 needs dynamic_mask, which this build has no kernel for");
+  if (!a->ptr_A || !a->ptr_B || !a->ptr_C) return fail(CUMM_HIP_ERUNTIME, "input, weight and output must not be empty");
+  if (!a->indice_ptr || !a->mask_ptr || !a->mask_argsort_ptr)
+    return fail(CUMM_HIP_ERUNTIME, "indices, mask and mask_argsort must not be empty");
+  if (!aligned16(a->ptr_A) || !aligned16(a->ptr_B) || !aligned16(a->ptr_C) || (a->ptr_D && !aligned16(a->ptr_D)))
+    return fail(CUMM_HIP_EINVAL, "operand pointers must be 16-byte aligned");
+  if (a->C % pv || a->K % pv) return fail(CUMM_HIP_ERUNTIME, "C and K must be multiples of %d for this element type", pv);
+  if (!d.split_k_serial && a->split_k_slices > 1)
+    return fail(CUMM_HIP_ERUNTIME, "algo don't support splitk but you provide split_k_slices > 1.");
+  if (a->N == 0) return CUMM_HIP_OK;
+  const void *ptr_D = a->ptr_D ? a->ptr_D : a->ptr_C;
+
+  if (fam == 1) {
+    const bool fwd = c.op_type == CUMM_HIP_OP_FORWARD;
+    RowGemmParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.A = a->ptr_A; p.W = a->ptr_B; p.C = a->ptr_C; p.D = ptr_D;
+    p.out_rows = a->mask_argsort_ptr;
+    p.gather = a->indice_ptr;
+    p.mask = a->mask_ptr;
+    p.mask_out = fwd ? a->mask_out_ptr : nullptr;
+    p.n_pos = a->N; p.n_idx = a->N; p.kv = kv;
+    p.mask_filter = a->mask_filter;
+    if (fwd) {
+      // input [rows_in, C] x weight [K, kv, C] -> output [rows_out, K]
+      p.lda = a->C; p.ldc = a->K; p.c_in = a->C; p.k_out = a->K;
+      p.rows_a = a->rows_in; p.rows_c = a->rows_out;
+      p.w_stride_n = (int64_t)kv * a->C; p.w_stride_k = a->C; p.w_stride_c = 1;
+    } else {
+      // dOut [rows_out, K] x weight -> dIn [rows_in, C]; contraction over K
+      p.lda = a->K; p.ldc = a->C; p.c_in = a->K; p.k_out = a->C;
+      p.rows_a = a->rows_out; p.rows_c = a->rows_in;
+      p.w_stride_n = 1; p.w_stride_k = a->C; p.w_stride_c = (int64_t)kv * a->C;
+      p.reverse_mask = a->reverse_mask;
+      p.exit_on_empty = 1;
+    }
+    p.ldd = a->d_is_bias ? 0 : p.ldc;
+    p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act_beta = a->act_beta;
+    p.act = a->act_type;
+    p.read_source = a->beta != 0.0f;
+    if (c.is_int8_inference) {
+      if (!a->bias_pointer || !a->scale_pointer)
+        return fail(CUMM_HIP_ERUNTIME, "int8 inference must have both scale and bias");
+      p.int8_epilogue = 1;
+      p.scale = reinterpret_cast<const float *>(a->scale_pointer);
+      p.bias = reinterpret_cast<const float *>(a->bias_pointer);
+      p.ldd = p.ldc;  // the only source of the int8 epilogue is output_add (or the output itself)
+    }
+    p.xcd_swizzle = 0;
+    hipError_t e = launch_rowgemm(dt, d.tile_shape[0], d.tile_shape[1], pick_ks(p.c_in, dt), !fwd, p, stream);
+    if (e != hipSuccess) return hip_fail(e, "sparse conv launch");
+    return CUMM_HIP_OK;
+  }
+
+  // backward weight: dW[K, kv, C]; A = dOut [N, K], B = input [*, C]
+  const int tm = d.tile_shape[0], tn = d.tile_shape[1], tk = d.tile_shape[2];
+  if (a->mask_width <= 0 || a->mask_width % tk) return fail(CUMM_HIP_ERUNTIME, "mask_width must be a positive multiple of tile k");
+  TileGemmParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.Y = a->ptr_A; p.ldy = a->K;       // dOut rows, m = K
+  p.X = a->ptr_B; p.ldx = a->C;       // input rows, n = C
+  p.C = a->ptr_C; p.D = ptr_D;
+  p.ldc = (int64_t)kv * a->C; p.ldd = p.ldc; p.c_off = a->C;
+  p.y_gather = a->mask_argsort_ptr;
+  p.x_gather = a->indice_ptr; p.x_gather_via_y = 1;
+  p.red_mask = a->mask_ptr;
+  p.num_red_mask = (a->N + a->mask_width - 1) / a->mask_width;
+  p.mask_width = a->mask_width;
+  p.mask_filter = a->mask_filter;
+  p.m = a->K; p.n = a->C; p.k = a->N; p.n_idx = a->N;
+  p.rows_y = a->rows_out; p.rows_x = a->rows_in;
+  p.kv = kv;
+  p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act = a->act_type;
+  p.split_k = a->split_k_slices < 1 ? 1 : a->split_k_slices;
+  p.spin_limit = kSpinLimit;
+  const int n_tiles = (a->C + tn - 1) / tn;
+  dim3 grid((a->K + tm - 1) / tm, n_tiles * kv, p.split_k);
+  if (p.split_k > 1) {
+    const size_t need = sizeof(int32_t) * grid.x * grid.y;
+    if (!a->workspace || a->workspace_bytes < need)
+      return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
+    HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
+    p.sem = reinterpret_cast<int32_t *>(a->workspace);
+  }
+  hipError_t e = launch_tilegemm(dt, tm, tn, false, false, p, grid, stream);
+  if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
+  return CUMM_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+int cumm_hip_device_count(int *count) {
+  if (!count) return fail(CUMM_HIP_EINVAL, "null out-param");
+  hipError_t e = hipGetDeviceCount(count);
+  if (e != hipSuccess) { *count = 0; return hip_fail(e, "hipGetDeviceCount"); }
+  return CUMM_HIP_OK;
+}
+int cumm_hip_malloc(void **ptr, size_t bytes) {
+  if (!ptr) return fail(CUMM_HIP_EINVAL, "null out-param");
+  *ptr = nullptr;
+  if (bytes == 0) return CUMM_HIP_OK;
+  HIP_TRY(hipMalloc(ptr, bytes));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_free(void *ptr) {
+  if (ptr) HIP_TRY(hipFree(ptr));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_host_malloc(void **ptr, size_t bytes) {
+  if (!ptr) return fail(CUMM_HIP_EINVAL, "null out-param");
+  *ptr = nullptr;
+  if (bytes == 0) return CUMM_HIP_OK;
+  HIP_TRY(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_host_free(void *ptr) {
+  if (ptr) HIP_TRY(hipHostFree(ptr));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return CUMM_HIP_OK;
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, reinterpret_cast<hipStream_t>(stream)));
+  HIP_TRY(hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return CUMM_HIP_OK;
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, reinterpret_cast<hipStream_t>(stream)));
+  HIP_TRY(hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return CUMM_HIP_OK;
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, reinterpret_cast<hipStream_t>(stream)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_memset(void *ptr, int value, size_t bytes, void *stream) {
+  if (bytes == 0) return CUMM_HIP_OK;
+  HIP_TRY(hipMemsetAsync(ptr, value, bytes, reinterpret_cast<hipStream_t>(stream)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_stream_create(void **stream) {
+  if (!stream) return fail(CUMM_HIP_EINVAL, "null out-param");
+  hipStream_t s;
+  HIP_TRY(hipStreamCreate(&s));
+  *stream = s;
+  return CUMM_HIP_OK;
+}
+int cumm_hip_stream_destroy(void *stream) {
+  HIP_TRY(hipStreamDestroy(reinterpret_cast<hipStream_t>(stream)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_stream_synchronize(void *stream) {
+  HIP_TRY(hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_device_synchronize(void) {
+  HIP_TRY(hipDeviceSynchronize());
+  return CUMM_HIP_OK;
+}
+int cumm_hip_event_create(void **event) {
+  if (!event) return fail(CUMM_HIP_EINVAL, "null out-param");
+  hipEvent_t e;
+  HIP_TRY(hipEventCreate(&e));
+  *event = e;
+  return CUMM_HIP_OK;
+}
+int cumm_hip_event_destroy(void *event) {
+  HIP_TRY(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_event_record(void *event, void *stream) {
+  HIP_TRY(hipEventRecord(reinterpret_cast<hipEvent_t>(event), reinterpret_cast<hipStream_t>(stream)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_event_synchronize(void *event) {
+  HIP_TRY(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));
+  return CUMM_HIP_OK;
+}
+int cumm_hip_event_elapsed_ms(void *start, void *stop, float *ms) {
+  if (!ms) return fail(CUMM_HIP_EINVAL, "null out-param");
+  HIP_TRY(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop)));
+  return CUMM_HIP_OK;
+}
+
+__global__ void copy16_kernel(v4i *dst, const v4i *src, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) dst[i] = src[i];
+}
+
+int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes % 16 || !aligned16(dst) || !aligned16(src)) return fail(CUMM_HIP_EINVAL, "copy needs 16-byte alignment");
+  const size_t n = bytes / 16;
+  if (n == 0) return CUMM_HIP_OK;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     reinterpret_cast<v4i *>(dst), reinterpret_cast<const v4i *>(src), n);
+  HIP_TRY(hipGetLastError());
+  return CUMM_HIP_OK;
+}
+
+}  // extern "C"

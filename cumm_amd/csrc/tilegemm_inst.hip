@@ -1,0 +1,27 @@
+// Instantiations of the LDS-tiled GEMM for one element type (selected with -DCUMM_ELEM=...).
+#include "launch.h"
+
+namespace cummhip {
+
+#define CUMM_CAT_(a, b) a##b
+#define CUMM_CAT(a, b) CUMM_CAT_(a, b)
+
+template <class T, int BM, int BN>
+static hipError_t launch_xy(bool xk, bool yk, const TileGemmParams &p, dim3 grid, hipStream_t s) {
+  if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
+  if (xk && yk) hipLaunchKernelGGL((tilegemm_kernel<T, true, true, BM, BN, 1>), grid, dim3(256), 0, s, p);
+  else if (xk && !yk) hipLaunchKernelGGL((tilegemm_kernel<T, true, false, BM, BN, 1>), grid, dim3(256), 0, s, p);
+  else if (!xk && yk) hipLaunchKernelGGL((tilegemm_kernel<T, false, true, BM, BN, 1>), grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((tilegemm_kernel<T, false, false, BM, BN, 1>), grid, dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+hipError_t CUMM_CAT(launch_tilegemm_, CUMM_NAME)(int tm, int tn, bool xk, bool yk,
+                                                 const TileGemmParams &p, dim3 grid, hipStream_t s) {
+  using T = CUMM_ELEM;
+  if (tm == 64 && tn == 64) return launch_xy<T, 2, 2>(xk, yk, p, grid, s);
+  if (tm == 128 && tn == 128) return launch_xy<T, 4, 4>(xk, yk, p, grid, s);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace cummhip

@@ -1,0 +1,135 @@
+"""Host-side pair-table builder for mask-based sparse convolution.
+
+The reference does not build pair tables itself: its callers get them from
+spconv (``SpconvOps.generate_subm_conv_inds`` / ``generate_conv_inds_mask_stage1/2``
+/ ``sort_1d_by_key``; call sites cumm/conv/main_real_spconv.py:91-145).  This
+module is the host (numpy) stand-in that prepares operator inputs: sorted-key
+lookups, O(kv * N log N).
+
+Conventions of this build (spconv's own are not part of the reference tree):
+kernel offset index k = (kz*KY + ky)*KX + kx; cross-correlation, i.e. output o
+gathers the input at ``coord[o]*stride - padding + k_zyx*dilation``; rows of a
+strided convolution's output are ordered by ascending (batch, z, y, x); the
+mask sort is a stable ascending argsort.
+"""
+from typing import NamedTuple, Sequence, Tuple
+
+import numpy as np
+
+
+class PairTable(NamedTuple):
+    indices_fwd: np.ndarray   # [kv, N_out] int32: output row -> input row, -1 = none
+    indices_bwd: np.ndarray   # [kv, N_in]  int32: input row -> output row, -1 = none
+    mask_fwd: np.ndarray      # [N_out] uint32, bit k set iff indices_fwd[k][o] >= 0
+    mask_bwd: np.ndarray      # [N_in]  uint32, bit k set iff indices_bwd[k][i] >= 0
+    out_coords: np.ndarray    # [N_out, 4] int32 (batch, z, y, x)
+    out_shape: Tuple[int, int, int]
+
+
+def _linear(coords: np.ndarray, shape: Sequence[int]) -> np.ndarray:
+    c = coords.astype(np.int64)
+    return ((c[:, 0] * shape[0] + c[:, 1]) * shape[1] + c[:, 2]) * shape[2] + c[:, 3]
+
+
+def _offsets(ksize: Sequence[int]) -> np.ndarray:
+    kz, ky, kx = np.meshgrid(np.arange(ksize[0]), np.arange(ksize[1]), np.arange(ksize[2]),
+                             indexing="ij")
+    return np.stack([kz.ravel(), ky.ravel(), kx.ravel()], axis=1).astype(np.int64)
+
+
+def _masks(indices: np.ndarray) -> np.ndarray:
+    kv = indices.shape[0]
+    assert kv <= 32
+    bits = (np.uint32(1) << np.arange(kv, dtype=np.uint32))[:, None]
+    return np.bitwise_or.reduce(np.where(indices >= 0, bits, np.uint32(0)), axis=0).astype(np.uint32)
+
+
+def _lookup(sorted_keys, order, query_keys, valid):
+    pos = np.searchsorted(sorted_keys, query_keys)
+    pos = np.minimum(pos, len(sorted_keys) - 1)
+    hit = valid & (sorted_keys[pos] == query_keys)
+    return np.where(hit, order[pos], -1).astype(np.int32)
+
+
+def calc_output_dims(in_shape, ksize, padding, stride, dilation):
+    """cumm/conv/params.py:268-292 of the reference (ConvProblem.calc_output_dims)."""
+    return tuple((int(i) + 2 * int(p) - int(d) * (int(k) - 1) - 1) // int(s) + 1
+                 for i, k, p, s, d in zip(in_shape, ksize, padding, stride, dilation))
+
+
+def subm_pairs(coords: np.ndarray, spatial_shape: Sequence[int], ksize=(3, 3, 3),
+               dilation=(1, 1, 1)) -> PairTable:
+    """Submanifold convolution: outputs sit on the input sites."""
+    coords = np.ascontiguousarray(coords, dtype=np.int32)
+    n = coords.shape[0]
+    offs = _offsets(ksize)
+    kv = offs.shape[0]
+    center = np.array([k // 2 for k in ksize], dtype=np.int64)
+    keys = _linear(coords, spatial_shape)
+    order = np.argsort(keys, kind="stable")
+    skeys = keys[order]
+    assert n == 0 or np.all(skeys[1:] != skeys[:-1]), "duplicate voxel coordinates"
+    ind = np.full((kv, n), -1, dtype=np.int32)
+    sp = np.asarray(spatial_shape, dtype=np.int64)
+    c64 = coords.astype(np.int64)
+    for k in range(kv):
+        q = c64.copy()
+        q[:, 1:] += (offs[k] - center) * np.asarray(dilation, dtype=np.int64)
+        valid = np.all((q[:, 1:] >= 0) & (q[:, 1:] < sp), axis=1)
+        if n:
+            ind[k] = _lookup(skeys, order, _linear(np.where(valid[:, None], q, 0), spatial_shape), valid)
+    ind_b = ind[::-1].copy()  # input i feeds output o through offset k iff o sees i through kv-1-k
+    return PairTable(ind, ind_b, _masks(ind), _masks(ind_b), coords, tuple(int(s) for s in spatial_shape))
+
+
+def sparse_conv_pairs(coords: np.ndarray, spatial_shape: Sequence[int], ksize=(3, 3, 3),
+                      stride=(2, 2, 2), padding=(1, 1, 1), dilation=(1, 1, 1)) -> PairTable:
+    """Regular (strided) sparse convolution: an output site is active iff any
+    input falls in its receptive field."""
+    coords = np.ascontiguousarray(coords, dtype=np.int32)
+    n_in = coords.shape[0]
+    offs = _offsets(ksize)
+    kv = offs.shape[0]
+    out_shape = calc_output_dims(spatial_shape, ksize, padding, stride, dilation)
+    st = np.asarray(stride, dtype=np.int64)
+    pd = np.asarray(padding, dtype=np.int64)
+    dl = np.asarray(dilation, dtype=np.int64)
+    osz = np.asarray(out_shape, dtype=np.int64)
+    c64 = coords.astype(np.int64)
+    cand_keys = []
+    per_k = []
+    for k in range(kv):
+        num = c64[:, 1:] + pd - offs[k] * dl
+        o = num // st
+        valid = np.all((num % st == 0) & (o >= 0) & (o < osz), axis=1)
+        oc = np.concatenate([c64[:, :1], o], axis=1)
+        okey = _linear(np.where(valid[:, None], oc, 0), out_shape)
+        per_k.append((valid, okey))
+        cand_keys.append(okey[valid])
+    all_keys = np.unique(np.concatenate(cand_keys)) if n_in else np.zeros(0, np.int64)
+    n_out = all_keys.shape[0]
+    out_coords = np.zeros((n_out, 4), dtype=np.int32)
+    rem = all_keys.copy()
+    for d, s in zip((3, 2, 1), out_shape[::-1]):
+        out_coords[:, d] = rem % s
+        rem //= s
+    out_coords[:, 0] = rem
+    ind_f = np.full((kv, n_out), -1, dtype=np.int32)
+    ind_b = np.full((kv, n_in), -1, dtype=np.int32)
+    for k in range(kv):
+        valid, okey = per_k[k]
+        rows_in = np.nonzero(valid)[0]
+        rows_out = np.searchsorted(all_keys, okey[valid])
+        ind_f[k, rows_out] = rows_in
+        ind_b[k, rows_in] = rows_out
+    return PairTable(ind_f, ind_b, _masks(ind_f), _masks(ind_b), out_coords, out_shape)
+
+
+def sort_by_mask(mask: np.ndarray, mask_filter: int = 0xFFFFFFFF):
+    """(sorted mask, argsort): stable ascending sort of ``mask & mask_filter``
+    (spconv's sort_1d_by_key[_split]; the kernel reads the mask by sorted position
+    and the pair table by real row, cumm/conv/kernel.py:853-855,
+    cumm/conv/sparse_iters.py:349-352 of the reference)."""
+    key = mask & np.uint32(mask_filter)
+    order = np.argsort(key, kind="stable").astype(np.int32)
+    return np.ascontiguousarray(key[order]), order

@@ -1,0 +1,175 @@
+/*
+ * cumm_hip.h - C ABI of libcummhip.so: gfx950 (MI355X) kernels for the GEMM and
+ * mask-based implicit-GEMM sparse-convolution path of FindDefinition/cumm.
+ *
+ * Every entry point takes plain pointers and sizes (device pointers unless a
+ * comment says host) and returns 0 on success or a CUMM_HIP_E* code; the text
+ * of the last error of the calling thread is read with cumm_hip_last_error().
+ * Launches are asynchronous on the given stream (0 = the default stream); no
+ * entry point synchronises unless its name says so.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the reference tree).
+ */
+#ifndef CUMM_HIP_H_
+#define CUMM_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes */
+#define CUMM_HIP_OK 0
+#define CUMM_HIP_EINVAL 1      /* bad argument: the reference raises ValueError (TV_ASSERT_INVALID_ARG) */
+#define CUMM_HIP_ERUNTIME 2    /* failed check / HIP error: the reference raises RuntimeError (TV_ASSERT_RT_ERR) */
+#define CUMM_HIP_ENOALGO 3     /* no kernel for this descriptor ("can't find any suitable algo") */
+
+/* tv::DType values, include/tensorview/dtypes.h:39-64 */
+#define CUMM_HIP_F32 0
+#define CUMM_HIP_S32 1
+#define CUMM_HIP_S8 3
+#define CUMM_HIP_F16 7
+#define CUMM_HIP_U32 10
+#define CUMM_HIP_BF16 12
+
+/* tv::gemm::ConvOpType / ShuffleStrideType / Activation,
+ * include/tensorview/gemm/core/constants.h:20-55 */
+#define CUMM_HIP_OP_FORWARD 0
+#define CUMM_HIP_OP_BACKWARD_INPUT 1
+#define CUMM_HIP_OP_BACKWARD_WEIGHT 2
+#define CUMM_HIP_NO_SHUFFLE 0
+#define CUMM_HIP_SHUFFLE_AC 1
+#define CUMM_HIP_SHUFFLE_AB 2
+#define CUMM_HIP_ACT_NONE 0
+#define CUMM_HIP_ACT_RELU 1
+#define CUMM_HIP_ACT_SIGMOID 2
+#define CUMM_HIP_ACT_LEAKY_RELU 3
+
+/* The fields of tv::gemm::GemmAlgoDesp that select a kernel
+ * (include/tensorview/gemm/core/params.h:24-54). */
+typedef struct CummHipGemmDesc {
+  int32_t dtype_a, dtype_b, dtype_c, dacc, dcomp;
+  int32_t trans_a, trans_b, trans_c;
+  int32_t tile_shape[3];
+  int32_t warp_tile_shape[3];
+  int32_t num_stage;
+  int32_t shuffle_type;
+  int32_t split_k_serial, split_k_parallel;
+} CummHipGemmDesc;
+
+/* tv::gemm::ConvAlgoDesp adds these (params.h:166-196). */
+typedef struct CummHipConvDesc {
+  CummHipGemmDesc gemm;
+  int32_t ndim, op_type;
+  int32_t mask_sparse, increment_k_first, dynamic_mask, is_int8_inference;
+} CummHipConvDesc;
+
+/* Operands of one GEMM launch: tv::gemm::GemmNVRTCParams
+ * (include/tensorview/gemm/core/nvrtc_params.h:23-37) as filled by the prelude
+ * cumm/gemm/nvrtc_code.py:34-198.  Strides are row strides in elements;
+ * stride_D == 0 means D is a bias over n. */
+typedef struct CummHipGemmArgs {
+  int32_t m, n, k;
+  const void *ptr_A, *ptr_B, *ptr_D;
+  void *ptr_C;
+  int64_t stride_A, stride_B, stride_C, stride_D;
+  const int32_t *indiceA;    /* ShuffleAC: a_inds or NULL; ShuffleAB: a_inds */
+  const int32_t *indiceBorC; /* ShuffleAC: c_inds; ShuffleAB: b_inds */
+  const int32_t *indiceD;    /* ShuffleAC: c_inds or NULL when D is a bias */
+  float alpha, beta, act_alpha, act_beta;
+  int32_t act_type;
+  int32_t split_k_slices;
+  void *workspace;           /* split-K scratch, zeroed by the callee before use */
+  size_t workspace_bytes;
+  int32_t rows_A, rows_B, rows_C; /* row counts of the underlying tensors: gathered/scattered
+                                     row numbers outside them are treated as absent */
+} CummHipGemmArgs;
+
+/* Operands of one mask-based sparse-convolution launch:
+ * tv::gemm::SparseConvNVRTCParams (nvrtc_params.h:39-65) as filled by the
+ * prelude cumm/conv/nvrtc_code.py:20-197.  (A,B,C) are (input,weight,output)
+ * permuted by op_type exactly as there: forward (input, weight, output),
+ * dgrad (output, weight, input), wgrad (output, input, weight).
+ * Rows of input/output are dense (row stride == channel count); the weight is
+ * [K, kernel_volume, C]. */
+typedef struct CummHipSparseConvArgs {
+  const void *ptr_A, *ptr_B, *ptr_D;
+  void *ptr_C;
+  float alpha, beta, act_alpha, act_beta;
+  int32_t act_type;
+  int32_t split_k_slices;
+  void *workspace;
+  size_t workspace_bytes;
+  const uint32_t *mask_ptr;         /* fwd/dgrad: per sorted position; wgrad: forward's mask_output */
+  uint32_t *mask_out_ptr;           /* forward only, may be NULL */
+  const int32_t *indice_ptr;        /* [kernel_volume, N] */
+  const int32_t *mask_argsort_ptr;  /* [N] */
+  uint32_t mask_filter;
+  int32_t reverse_mask;
+  int32_t mask_width;               /* wgrad: positions covered by one mask word */
+  int32_t ndim, N, C, K;
+  int32_t kernel_volume;
+  int32_t d_is_bias;
+  const void *bias_pointer;         /* int8 inference: f32 [K] */
+  const void *scale_pointer;        /* int8 inference: f32 [K] */
+  int32_t rows_in, rows_out;        /* row counts of the input / output feature tensors */
+} CummHipSparseConvArgs;
+
+/* Replaces GemmMainUnitTest.matmul2 below its prelude
+ * (cumm/gemm/main.py:1176-1335: dispatch on the descriptor and launch). */
+int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *args, void *stream);
+
+/* Replaces ConvMainUnitTest.implicit_gemm2 below its prelude for mask_sparse
+ * descriptors (cumm/conv/main.py:483-745). */
+int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArgs *args,
+                         void *stream);
+
+/* GemmMainUnitTest.get_all_algo_desp / ConvMainUnitTest.get_all_conv_algo_desp
+ * (cumm/gemm/main.py:914-965, cumm/conv/main.py:467-481): the descriptors this
+ * build has kernels for.  Writes at most cap entries, returns the total. */
+int cumm_hip_list_gemm_algos(CummHipGemmDesc *out, int cap);
+int cumm_hip_list_conv_algos(CummHipConvDesc *out, int cap);
+
+/* 1 if a kernel exists for the descriptor, else 0 (the "found" flag of the
+ * dispatch chains, cumm/gemm/main.py:1325-1334, cumm/conv/main.py:734-744). */
+int cumm_hip_gemm_supported(const CummHipGemmDesc *desc);
+int cumm_hip_conv_supported(const CummHipConvDesc *desc);
+
+/* Text of the last error returned to the calling thread. */
+const char *cumm_hip_last_error(void);
+
+/* ---- device backend of tv::Tensor / tv::Context (include/tensorview/tensor.h:181-330
+ * allocation, :1395 zero_, :1525-1766 copy_/cpu()/cuda(); include/tensorview/contexts/core.h:429-500) */
+int cumm_hip_device_count(int *count);                 /* host out-param */
+int cumm_hip_malloc(void **ptr, size_t bytes);         /* host out-param */
+int cumm_hip_free(void *ptr);
+int cumm_hip_host_malloc(void **ptr, size_t bytes);    /* pinned host memory */
+int cumm_hip_host_free(void *ptr);
+int cumm_hip_memcpy_h2d(void *dst, const void *src_host, size_t bytes, void *stream);
+int cumm_hip_memcpy_d2h(void *dst_host, const void *src, size_t bytes, void *stream);
+int cumm_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int cumm_hip_memset(void *ptr, int value, size_t bytes, void *stream);
+int cumm_hip_stream_create(void **stream);             /* host out-param; default priority */
+int cumm_hip_stream_destroy(void *stream);
+/* GemmMainUnitTest.stream_synchronize / device_synchronize (cumm/gemm/main.py:1028-1047) */
+int cumm_hip_stream_synchronize(void *stream);
+int cumm_hip_device_synchronize(void);
+
+/* ---- events: tv::CUDAEvent / CUDAKernelTimer (include/tensorview/profile/cuda_profiler.h:97-406) */
+int cumm_hip_event_create(void **event);               /* host out-param */
+int cumm_hip_event_destroy(void *event);
+int cumm_hip_event_record(void *event, void *stream);
+int cumm_hip_event_synchronize(void *event);
+int cumm_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* host out-param */
+
+/* Plain device-to-device copy kernel of `bytes` bytes (16-byte aligned); used to
+ * calibrate the HBM traffic counters against a transfer of known size. */
+int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUMM_HIP_H_ */

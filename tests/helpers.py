@@ -1,0 +1,71 @@
+"""Shared builders for the parity tests: seeded inputs, descriptor lookup and
+calls through the operator API (which goes through the C ABI)."""
+import numpy as np
+
+from cumm_amd import pairs, synth
+from cumm_amd import tensorview as tv
+from cumm_amd.conv.main import ConvMainUnitTest
+from cumm_amd.gemm.main import GemmMainUnitTest
+from cumm_amd.tensorview.gemm import (Activation, ConvOpType, ConvParams, GemmParams,
+                                      ShuffleStrideType)
+
+TV_DTYPE = {"f16": tv.float16, "bf16": tv.bfloat16, "s8": tv.int8, "f32": tv.float32}
+
+
+def to_storage(x_f32, dtype):
+    """float32 values -> array in the storage dtype (bf16 as uint16 bits)."""
+    if dtype == "f16":
+        return x_f32.astype(np.float16)
+    if dtype == "bf16":
+        return synth.f32_to_bf16_bits(x_f32)
+    if dtype == "s8":
+        return x_f32.astype(np.int8)
+    return x_f32.astype(np.float32)
+
+
+def as_f32(x, dtype):
+    if dtype == "bf16":
+        return synth.bf16_bits_to_f32(x)
+    return np.asarray(x).astype(np.float32)
+
+
+def dev(arr, dtype):
+    """numpy array in storage dtype -> device tv.Tensor."""
+    t = tv.from_numpy(np.ascontiguousarray(arr))
+    if dtype == "bf16":
+        t = t.type_view(tv.bfloat16)
+    return t.cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def rel_err(got_f32, ref_f32):
+    """max |got-ref| / max |ref|: the reference's own criterion
+    (cumm/gemm/main_real.py:672-677)."""
+    denom = max(float(np.max(np.abs(ref_f32))), 1e-6)
+    return float(np.max(np.abs(got_f32.astype(np.float64) - ref_f32.astype(np.float64)))) / denom
+
+
+def find_conv_desp(dtype, op, tile_m, tile_n, int8_inference=False):
+    for d in ConvMainUnitTest.get_all_conv_algo_desp():
+        if (d.dtype_a == TV_DTYPE[dtype] and ConvOpType(d.op_type) == op and
+                d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and
+                d.is_int8_inference == int8_inference):
+            return d
+    raise KeyError((dtype, op, tile_m, tile_n, int8_inference))
+
+
+def find_gemm_desp(dtype, shuffle, tile_m, tile_n, trans_a, trans_b, trans_c=False):
+    for d in GemmMainUnitTest.get_all_algo_desp():
+        if (d.dtype_a == TV_DTYPE[dtype] and d.shuffle_type == shuffle and
+                d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and
+                d.trans_a == trans_a and d.trans_b == trans_b and d.trans_c == trans_c):
+            return d
+    raise KeyError((dtype, shuffle, tile_m, tile_n, trans_a, trans_b, trans_c))
+
+
+def small_cloud(seed, n, grid=(12, 40, 36), clusters=6, sigma=3.0):
+    rng = np.random.default_rng(seed)
+    return synth.clustered_voxels(rng, n, grid, clusters, sigma=sigma), grid

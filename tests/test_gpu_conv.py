@@ -1,0 +1,224 @@
+"""GPU parity: mask-based sparse convolution through ConvMainUnitTest.implicit_gemm2
+(-> C ABI -> HIP kernels) against the CPU oracle on the same seeded inputs.
+
+Modelled on the reference's own check script cumm/conv/main_real_spconv.py:54-411
+(forward / backward-input / backward-weight vs per-offset gather-matmul-scatter).
+Tolerance for f16/bf16: max relative error 1e-2 (fp32 accumulate); pair tables,
+s32 accumulators and s8 outputs are compared bit-exactly.
+"""
+import numpy as np
+import pytest
+
+from oracle import conv_ref
+from oracle import numerics as onm
+
+from cumm_amd import pairs, synth
+from cumm_amd import tensorview as tv
+from cumm_amd.conv.main import ConvMainUnitTest
+from cumm_amd.tensorview.gemm import Activation, ConvOpType, ConvParams
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _case(seed, n, c_in, k_out, dtype, grid=(12, 40, 36), strided=False):
+    rng = np.random.default_rng(seed)
+    coords = synth.clustered_voxels(rng, n, grid, 6, sigma=3.0)
+    if strided:
+        pt = pairs.sparse_conv_pairs(coords, grid)
+    else:
+        pt = pairs.subm_pairs(coords, grid)
+    n_in = coords.shape[0]
+    n_out = pt.indices_fwd.shape[1]
+    if dtype == "s8":
+        feat = rng.integers(-127, 128, size=(n_in, c_in)).astype(np.int8)
+        w = rng.integers(-127, 128, size=(k_out, 27, c_in)).astype(np.int8)
+    else:
+        feat = H.to_storage(rng.normal(0, 1, size=(n_in, c_in)).astype(np.float32), dtype)
+        w = H.to_storage(rng.normal(0, 0.05, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    return rng, coords, pt, feat, w, n_in, n_out
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("tile", [(64, 64), (128, 64), (64, 128), (128, 128)])
+@pytest.mark.parametrize("c_in,k_out", [(64, 64), (32, 96), (128, 128), (72, 40)])
+def test_subm_forward(dtype, tile, c_in, k_out):
+    print("case subm_forward", dtype, tile, c_in, k_out, flush=True)
+    rng, coords, pt, feat, w, n_in, n_out = _case(1, 3000, c_in, k_out, dtype)
+    mask_sorted, argsort = pairs.sort_by_mask(pt.mask_fwd)
+    desp = H.find_conv_desp(dtype, ConvOpType.Forward, *tile)
+    out0 = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    for beta in (0.0, 1.0):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = desp
+        p.input, p.weight = H.dev(feat, dtype), H.dev(w, dtype)
+        p.output = H.dev(out0, dtype)
+        p.indices = H.dev(pt.indices_fwd, "i32")
+        p.mask, p.mask_argsort = H.dev(mask_sorted, "u32"), H.dev(argsort, "i32")
+        tiles = (n_out + tile[0] - 1) // tile[0]
+        p.mask_output = tv.zeros([tiles], tv.uint32, 0)
+        p.mask_width = tile[0]
+        p.beta = beta
+        ConvMainUnitTest.implicit_gemm2(p)
+        got = H.host(p.output)
+        ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(
+            feat, w, out0, pt.indices_fwd, mask_sorted, argsort, tile_m=tile[0], dtype_in=dtype,
+            dtype_w=dtype, dtype_out=dtype, beta=beta)
+        assert H.rel_err(H.as_f32(got, dtype), H.as_f32(ref, dtype)) < TOL
+        np.testing.assert_array_equal(H.host(p.mask_output), ref_mo)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_forward_bias_relu_and_mask_filter(dtype):
+    rng, coords, pt, feat, w, n_in, n_out = _case(2, 2500, 64, 64, dtype)
+    bias = H.to_storage(rng.normal(0, 1, size=(64,)).astype(np.float32), dtype)
+    desp = H.find_conv_desp(dtype, ConvOpType.Forward, 64, 64)
+    out0 = H.to_storage(np.zeros((n_out, 64), np.float32), dtype)
+    # two mask splits as in cumm/conv/main_real_spconv.py:270-294: the second pass accumulates
+    filters = [0x3FFF, 0x1FFF << 14]
+    cur = out0
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = desp
+    p.input, p.weight = H.dev(feat, dtype), H.dev(w, dtype)
+    p.output = H.dev(out0, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    for j, f in enumerate(filters):
+        ms, order = pairs.sort_by_mask(pt.mask_fwd, f)
+        p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+        p.mask_filter = f
+        p.beta = 0.0 if j == 0 else 1.0
+        ConvMainUnitTest.implicit_gemm2(p)
+        cur, _ = conv_ref.implicit_gemm_fwd_ref(
+            feat, w, cur, pt.indices_fwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype,
+            dtype_out=dtype, mask_filter=f, beta=p.beta)
+    assert H.rel_err(H.as_f32(H.host(p.output), dtype), H.as_f32(cur, dtype)) < TOL
+    # bias as the source operand + ReLU (BN folded into the epilogue)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = desp
+    p.input, p.weight = H.dev(feat, dtype), H.dev(w, dtype)
+    p.output = H.dev(out0, dtype)
+    p.bias = H.dev(bias, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    p.beta = 1.0
+    p.act_type = Activation.ReLU
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref, _ = conv_ref.implicit_gemm_fwd_ref(
+        feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype,
+        dtype_out=dtype, beta=1.0, bias=bias, act=onm.ACT_RELU)
+    got = H.as_f32(H.host(p.output), dtype)
+    assert got.min() >= 0.0
+    assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("tile", [(64, 64), (128, 128)])
+@pytest.mark.parametrize("strided", [False, True])
+def test_backward_input(dtype, tile, strided):
+    print("case backward_input", dtype, tile, strided, flush=True)
+    c_in, k_out = 64, 96
+    rng, coords, pt, feat, w, n_in, n_out = _case(3, 2500, c_in, k_out, dtype, strided=strided)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    din0 = H.to_storage(rng.normal(0, 1, size=(n_in, c_in)).astype(np.float32), dtype)
+    desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, *tile)
+    if strided:
+        ms, order = pairs.sort_by_mask(pt.mask_bwd)
+        reverse = False
+    else:
+        # SubM: the forward mask is reused, bit-reversed inside the kernel
+        ms, order = pairs.sort_by_mask(pt.mask_fwd)
+        reverse = True
+    p = ConvParams(3, ConvOpType.BackwardInput)
+    p.conv_algo_desp = desp
+    p.input, p.weight, p.output = H.dev(din0, dtype), H.dev(w, dtype), H.dev(dout, dtype)
+    p.indices = H.dev(pt.indices_bwd, "i32")
+    p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    p.reverse_mask = reverse
+    p.beta = 0.0
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref = conv_ref.implicit_gemm_dgrad_ref(
+        dout, w, din0, pt.indices_bwd, ms, order, tile_m=tile[0], dtype_in=dtype, dtype_w=dtype,
+        dtype_out=dtype, reverse_mask=reverse)
+    assert H.rel_err(H.as_f32(H.host(p.input), dtype), H.as_f32(ref, dtype)) < TOL
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("tile", [(64, 64), (128, 128)])
+@pytest.mark.parametrize("split_k", [1, 4, 32])
+def test_backward_weight(dtype, tile, split_k):
+    print("case backward_weight", dtype, tile, split_k, flush=True)
+    c_in, k_out = 64, 96
+    rng, coords, pt, feat, w, n_in, n_out = _case(4, 3000, c_in, k_out, dtype)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    mask_width = 64
+    red = conv_ref.tile_masks(ms, mask_width)
+    dw0 = H.to_storage(np.zeros((k_out, 27, c_in), np.float32), dtype)
+    desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, *tile)
+    p = ConvParams(3, ConvOpType.BackwardWeight)
+    p.conv_algo_desp = desp
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(dw0, dtype), H.dev(dout, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(red, "u32"), H.dev(order, "i32")
+    p.mask_width = mask_width
+    p.split_k_slices = split_k
+    p.beta = 0.0
+    ConvMainUnitTest.implicit_gemm2(p)
+    got = H.as_f32(H.host(p.weight), dtype)
+    ref = conv_ref.implicit_gemm_wgrad_ref(
+        dout, feat, dw0, pt.indices_fwd, red, order, mask_width=mask_width, dtype_dout=dtype,
+        dtype_in=dtype, dtype_w=dtype, split_k_slices=split_k, tile_k=32)
+    assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+
+
+@pytest.mark.parametrize("tile", [(64, 64), (128, 128), (64, 128)])
+@pytest.mark.parametrize("strided", [False, True])
+def test_int8_inference_bit_exact(tile, strided):
+    print("case int8", tile, strided, flush=True)
+    c_in, k_out = 64, 128
+    rng, coords, pt, feat, w, n_in, n_out = _case(5, 3000, c_in, k_out, "s8", strided=strided)
+    scale = rng.uniform(0.001, 0.01, size=(k_out,)).astype(np.float32)
+    bias = rng.normal(0, 1, size=(k_out,)).astype(np.float32)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    out0 = np.zeros((n_out, k_out), np.int8)
+    add = rng.integers(-127, 128, size=(n_out, k_out)).astype(np.int8)
+    desp = H.find_conv_desp("s8", ConvOpType.Forward, *tile, int8_inference=True)
+    for use_add, act in ((False, Activation.None_), (True, Activation.ReLU)):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = desp
+        p.input, p.weight, p.output = H.dev(feat, "s8"), H.dev(w, "s8"), H.dev(out0, "s8")
+        p.scale, p.bias = H.dev(scale, "f32"), H.dev(bias, "f32")
+        if use_add:
+            p.output_add = H.dev(add, "s8")
+            p.beta = 0.5
+        p.act_type = act
+        p.indices = H.dev(pt.indices_fwd, "i32")
+        p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+        ConvMainUnitTest.implicit_gemm2(p)
+        ref, _ = conv_ref.implicit_gemm_fwd_ref(
+            feat, w, out0, pt.indices_fwd, ms, order, tile_m=tile[0], dtype_in="s8", dtype_w="s8",
+            dtype_out="s8", scale=scale, bias=bias, output_add=add if use_add else None,
+            beta=p.beta, act=act.value, int8_inference=True)
+        np.testing.assert_array_equal(H.host(p.output), ref)
+
+
+def test_ragged_and_empty():
+    """N not a multiple of the tile and a single voxel."""
+    dtype = "f16"
+    desp = H.find_conv_desp(dtype, ConvOpType.Forward, 64, 64)
+    for n in (1, 65, 130):
+        rng, coords, pt, feat, w, n_in, n_out = _case(6 + n, n, 64, 64, dtype, grid=(6, 10, 10))
+        ms, order = pairs.sort_by_mask(pt.mask_fwd)
+        out0 = H.to_storage(np.zeros((n_out, 64), np.float32), dtype)
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = desp
+        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+        p.indices = H.dev(pt.indices_fwd, "i32")
+        p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+        ConvMainUnitTest.implicit_gemm2(p)
+        ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64,
+                                                dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+        assert H.rel_err(H.as_f32(H.host(p.output), dtype), H.as_f32(ref, dtype)) < TOL
