@@ -1,0 +1,245 @@
+#!/usr/bin/env python
+"""Benchmark of the sparse-convolution hot path on one MI355X.
+
+One "step" is one forward pass of the mask-based implicit-GEMM sparse convolution
+(ConvMainUnitTest.implicit_gemm2) over one synthetic voxel cloud, inputs resident
+in HBM.  Headline workload: SubM 3x3x3, f16, Cin = Cout = 64, ~120k active voxels
+on a 41x1600x1408 grid (60 Gaussian clusters + 10 % noise).  The JSON line also
+carries the s8 stride-2 configuration, the backward passes, the HBM roofline of
+the forward kernel and a CPU baseline (the numpy oracle) timed on the host cores.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from cumm_amd import pairs, synth  # noqa: E402
+from cumm_amd import tensorview as tv  # noqa: E402
+from cumm_amd.conv.main import ConvMainUnitTest  # noqa: E402
+from cumm_amd.tensorview.gemm import ConvOpType, ConvParams  # noqa: E402
+
+PEAK_HBM_GBS = 8000.0
+PEAK_MFMA_F16_TFLOPS = 2516.6
+PEAK_MFMA_I8_TOPS = 5033.2
+GRID = (41, 1600, 1408)
+SEED = 20240607
+
+
+def find_desp(tv_dtype, op, tile_m, tile_n, int8=False):
+    for d in ConvMainUnitTest.get_all_conv_algo_desp():
+        if (d.dtype_a == tv_dtype and ConvOpType(d.op_type) == op and d.tile_shape[0] == tile_m
+                and d.tile_shape[1] == tile_n and d.is_int8_inference == int8):
+            return d
+    raise KeyError((tv_dtype, op, tile_m, tile_n, int8))
+
+
+def dev(arr):
+    return tv.from_numpy(np.ascontiguousarray(arr)).cuda()
+
+
+def timed(fn, steps, warmup, stream=0):
+    """(wall ms per step, event ms per step) over exactly `steps` calls."""
+    for _ in range(warmup):
+        fn()
+    ConvMainUnitTest_sync()
+    ev0, ev1 = tv.CUDAEvent("start"), tv.CUDAEvent("stop")
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for _ in range(steps):
+        fn()
+    ev1.record(stream)
+    ConvMainUnitTest_sync()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    evms = tv.CUDAEvent.duration(ev0, ev1) / steps
+    return wall, evms
+
+
+def ConvMainUnitTest_sync():
+    from cumm_amd.gemm.main import GemmMainUnitTest
+    GemmMainUnitTest.device_synchronize()
+
+
+def build_subm_f16(rng, n_target, c, k):
+    coords = synth.clustered_voxels(rng, n_target, GRID, 60, sigma=15.0, noise_frac=0.10)
+    pt = pairs.subm_pairs(coords, GRID)
+    n = coords.shape[0]
+    feat = rng.normal(0, 1, size=(n, c)).astype(np.float16)
+    w_ref = rng.normal(0, 0.05, size=(27, k, c)).astype(np.float16)   # [kv, K, C]
+    weight = np.ascontiguousarray(w_ref.transpose(1, 0, 2))           # passed as [K, kv, C]
+    return coords, pt, feat, weight
+
+
+def bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops):
+    pd = ConvParams(3, ConvOpType.BackwardInput)
+    pd.conv_algo_desp = find_desp(tv.float16, ConvOpType.BackwardInput, tile_m, 64)
+    pd.input = tv.zeros([n, C], tv.float16, 0)
+    pd.weight, pd.output = p.weight, dout
+    pd.indices = dev(pt.indices_bwd)
+    pd.mask, pd.mask_argsort = p.mask, p.mask_argsort
+    pd.reverse_mask = True
+    w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pd), args.steps, args.warmup)
+    return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
+            "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3)}
+
+
+def bench_wgrad(args, p, dout, n, C, K, tile_m, flops):
+    pw = ConvParams(3, ConvOpType.BackwardWeight)
+    pw.conv_algo_desp = find_desp(tv.float16, ConvOpType.BackwardWeight, 64, 64)
+    pw.input, pw.output = p.input, dout
+    pw.weight = tv.zeros([K, 27, C], tv.float16, 0)
+    pw.indices, pw.mask_argsort = p.indices, p.mask_argsort
+    pw.mask = p.mask_output       # written by the forward pass above
+    pw.mask_width = tile_m
+    pw.split_k_slices = 32
+    w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), max(1, args.steps // 4),
+                       max(1, args.warmup // 4))
+    return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
+            "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3)}
+
+
+def bench_s8(args, tile_m):
+    """s8 stride-2 SparseConv3d, Cin=64 -> Cout=128, int8 inference epilogue."""
+    rng4 = np.random.default_rng(SEED + 4)
+    c4 = synth.clustered_voxels(rng4, 300000, GRID, 60, sigma=15.0, noise_frac=0.10)
+    pt4 = pairs.sparse_conv_pairs(c4, GRID)
+    n_in4, n_out4 = c4.shape[0], pt4.indices_fwd.shape[1]
+    P4 = int((pt4.indices_fwd >= 0).sum())
+    ms4, as4 = pairs.sort_by_mask(pt4.mask_fwd)
+    p4 = ConvParams(3, ConvOpType.Forward)
+    p4.conv_algo_desp = find_desp(tv.int8, ConvOpType.Forward, tile_m, 128, int8=True)
+    p4.input = dev(rng4.integers(-127, 128, size=(n_in4, 64)).astype(np.int8))
+    p4.weight = dev(rng4.integers(-127, 128, size=(128, 27, 64)).astype(np.int8))
+    p4.output = tv.zeros([n_out4, 128], tv.int8, 0)
+    p4.scale = dev(rng4.uniform(0.001, 0.01, size=(128,)).astype(np.float32))
+    p4.bias = dev(rng4.normal(0, 1, size=(128,)).astype(np.float32))
+    p4.indices, p4.mask, p4.mask_argsort = dev(pt4.indices_fwd), dev(ms4), dev(as4)
+    w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(p4), args.steps, args.warmup)
+    ops4 = 2.0 * P4 * 64 * 128
+    bytes4 = n_in4 * 64 + n_out4 * 128 + 27 * 64 * 128 + 27 * n_out4 * 4 + n_out4 * 8 + 2 * 128 * 4
+    return {"voxels_in": n_in4, "voxels_out": n_out4, "active_pairs": P4,
+            "ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
+            "tops": round(ops4 / (w_ms * 1e-3) / 1e12, 3),
+            "pct_mfma_i8_peak": round(100.0 * ops4 / (w_ms * 1e-3) / 1e12 / PEAK_MFMA_I8_TOPS, 3),
+            "hbm_frac": round(bytes4 / (e_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--tile-m", type=int, default=64)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
+    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)",
+              file=sys.stderr)
+        return 2
+    if tv.device_count() < 1:
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+
+    rng = np.random.default_rng(SEED)
+    C = K = 64
+    coords, pt, feat, weight = build_subm_f16(rng, 120000, C, K)
+    n = coords.shape[0]
+    P = int((pt.indices_fwd >= 0).sum())
+    mask_sorted, argsort = pairs.sort_by_mask(pt.mask_fwd)
+    tile_m = args.tile_m
+
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = find_desp(tv.float16, ConvOpType.Forward, tile_m, 64)
+    p.input, p.weight = dev(feat), dev(weight)
+    p.output = tv.zeros([n, K], tv.float16, 0)
+    p.indices, p.mask, p.mask_argsort = dev(pt.indices_fwd), dev(mask_sorted), dev(argsort)
+    tiles = (n + tile_m - 1) // tile_m
+    p.mask_output = tv.zeros([tiles], tv.uint32, 0)
+    p.mask_width = tile_m
+    p.beta = 0.0
+
+    def step():
+        ConvMainUnitTest.implicit_gemm2(p)
+
+    wall_ms, ev_ms = timed(step, args.steps, args.warmup)
+    flops = 2.0 * P * C * K
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    alg_bytes = (n * C * 2 + n * K * 2 + 27 * C * K * 2 + 27 * n * 4 + n * 8)
+    achieved_gbs = alg_bytes / (ev_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "active-pair TFLOP/s + % MFMA peak, SubM 3x3x3 f16 C=64 and s8 C=128, 1 GPU",
+        "value": round(tflops, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "SubMConv3d 3x3x3 forward, f16, Cin=Cout=64, mask-based implicit GEMM",
+                   "voxels": n, "active_pairs": P, "pairs_per_voxel": round(P / n, 3),
+                   "grid_zyx": list(GRID), "clusters": 60, "sigma": 15, "noise_frac": 0.1,
+                   "tile_m": tile_m, "seed": SEED},
+        "pct_mfma_peak": round(100.0 * tflops / PEAK_MFMA_F16_TFLOPS, 3),
+        "kernel_ms_events": round(ev_ms, 5),
+        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(achieved_gbs / PEAK_HBM_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": alg_bytes},
+    }
+
+    if not args.no_extra:
+        extra = {}
+        legs = set(args.extra_only.split(",")) if args.extra_only else {"dgrad", "wgrad", "s8"}
+        # backward input (reverse mask, backward table) and backward weight (serial split-K)
+        dout = dev(rng.normal(0, 1, size=(n, K)).astype(np.float16))
+        if "dgrad" in legs:
+            extra["subm_f16_dgrad"] = bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops)
+        if "wgrad" in legs:
+            extra["subm_f16_wgrad_splitk32"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops)
+        if "s8" in legs:
+            extra["sparseconv_s8_stride2"] = bench_s8(args, tile_m)
+        result["extra"] = extra
+    if not args.no_cpu:
+        # CPU baseline: the numpy oracle (per-offset gather -> matmul -> scatter-add) on the
+        # same inputs; repeated until ~10 s of CPU work or 40 repetitions.
+        from oracle import conv_ref
+        try:
+            from threadpoolctl import threadpool_info
+            threads = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
+        except Exception:
+            threads = len(os.sched_getaffinity(0))
+        out0 = np.zeros((n, K), np.float16)
+        reps, spent, best = 0, 0.0, None
+        while reps < 40 and spent < 10.0:
+            t0 = time.perf_counter()
+            conv_ref.implicit_gemm_fwd_ref(feat, weight, out0, pt.indices_fwd, mask_sorted, argsort,
+                                           tile_m=tile_m, dtype_in="f16", dtype_w="f16", dtype_out="f16")
+            dt = time.perf_counter() - t0
+            spent += dt
+            reps += 1
+            best = dt if best is None else min(best, dt)
+        result["cpu_baseline"] = {
+            "value": round(flops / best / 1e12, 5), "unit": "TFLOP/s", "cores": int(threads),
+            "kind": "port",
+            "sample": "full headline workload (%d voxels, %d pairs), best of %d repetitions of the "
+                      "numpy oracle, %.1f s total" % (n, P, reps, spent)}
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

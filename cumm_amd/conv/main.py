@@ -60,6 +60,15 @@ class ConvMainUnitTest:
     @staticmethod
     def implicit_gemm2(params: ConvParams) -> None:
         desp = params.conv_algo_desp
+        # A call whose parameter object has not changed since it was last validated goes
+        # straight to the C ABI with the argument block prepared then.
+        prep = params.__dict__.get("_prepared")
+        if prep is not None and prep[0] == (params._version, desp._version, desp.tile_shape[0],
+                                            desp.tile_shape[1], desp.tile_shape[2]):
+            status = prep[1](prep[2], prep[3], params.stream)
+            if status:
+                _capi.check(status)
+            return
         if not desp.mask_sparse:
             raise RuntimeError("can't find any suitable algo for your parameters. "
                                "(dense convolution is not built)")
@@ -183,8 +192,14 @@ class ConvMainUnitTest:
         name = repr(desp) if params.timer.enable else ""
         if name:
             params.timer.record(name, params.stream)
-        status = _capi.lib().cumm_hip_sparse_conv(ctypes.byref(cdesc), ctypes.byref(args),
-                                                  params.stream)
+        fn = _capi.lib().cumm_hip_sparse_conv
+        status = fn(ctypes.byref(cdesc), ctypes.byref(args), params.stream)
         if name:
             params.timer.record(name, params.stream)
         _capi.check(status)
+        if not name:
+            # remember the validated argument block (the tensors it points into stay referenced
+            # by params; any later assignment to params or the descriptor invalidates it)
+            params.__dict__["_prepared"] = (
+                (params._version, desp._version, desp.tile_shape[0], desp.tile_shape[1],
+                 desp.tile_shape[2]), fn, ctypes.byref(cdesc), ctypes.byref(args), cdesc, args)

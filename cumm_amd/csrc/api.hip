@@ -80,6 +80,15 @@ hipError_t launch_tilegemm(int dt, int tm, int tn, bool xk, bool yk, const TileG
 
 constexpr int kSpinLimit = 1 << 24;
 
+// byte extent of a row-major 2-D operand for the buffer range checks; false if it does not fit
+// the 32-bit offsets the kernels use
+bool extent32(int64_t rows, int64_t ld, int64_t cols, int esize, uint32_t *out) {
+  const int64_t bytes = rows <= 0 ? 0 : ((rows - 1) * ld + cols) * esize;
+  if (bytes < 0 || bytes >= (int64_t)1 << 32) return false;
+  *out = (uint32_t)bytes;
+  return true;
+}
+
 // which kernel family serves a GEMM descriptor: 1 rowgemm, 2 tilegemm, 0 none
 int gemm_family(const CummHipGemmDesc &d) {
   if (!same_dtype3(d) || !acc_ok(d)) return 0;
@@ -268,7 +277,14 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
     p.read_source = a->beta != 0.0f;
     if (p.read_source && ldd != 0 && a->indiceD == nullptr && a->ptr_D != nullptr)
       return fail(CUMM_HIP_EINVAL, "a 2-D D needs the scatter indices (indiceD)");
-    p.xcd_swizzle = 0;
+    const int eb = elem_bytes(dt);
+    const int64_t b_rows = d.trans_b ? a->n : a->k, b_cols = d.trans_b ? a->k : a->n;
+    if (!extent32(a->rows_A, a->stride_A, a->k, eb, &p.a_bytes) ||
+        !extent32(b_rows, a->stride_B, b_cols, eb, &p.w_bytes) ||
+        !extent32(a->rows_C, a->stride_C, a->n, eb, &p.c_bytes) ||
+        !extent32(ldd ? a->rows_C : 1, ldd, a->n, eb, &p.d_bytes))
+      return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
+    p.gather_bytes = (uint32_t)a->m * 4u;
     hipError_t e = launch_rowgemm(dt, d.tile_shape[0], d.tile_shape[1], pick_ks(a->k, dt), !d.trans_b, p, stream);
     if (e != hipSuccess) return hip_fail(e, "gather-GEMM-scatter launch");
     return CUMM_HIP_OK;
@@ -386,7 +402,14 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
       p.bias = reinterpret_cast<const float *>(a->bias_pointer);
       p.ldd = p.ldc;  // the only source of the int8 epilogue is output_add (or the output itself)
     }
-    p.xcd_swizzle = 0;
+    const int eb = elem_bytes(dt);
+    if (!extent32(p.rows_a, p.lda, p.c_in, eb, &p.a_bytes) ||
+        !extent32((int64_t)a->K * kv, a->C, a->C, eb, &p.w_bytes) ||
+        !extent32(p.rows_c, p.ldc, p.k_out, eb, &p.c_bytes) ||
+        !extent32(p.ldd ? p.rows_c : 1, p.ldd, p.k_out, eb, &p.d_bytes) ||
+        (int64_t)kv * a->N * 4 >= (int64_t)1 << 32)
+      return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
+    p.gather_bytes = (uint32_t)((int64_t)kv * a->N * 4);
     hipError_t e = launch_rowgemm(dt, d.tile_shape[0], d.tile_shape[1], pick_ks(p.c_in, dt), !fwd, p, stream);
     if (e != hipSuccess) return hip_fail(e, "sparse conv launch");
     return CUMM_HIP_OK;

@@ -13,15 +13,20 @@
 //     output row: the epilogue reads the source row and writes the result row with 16-byte
 //     accesses and no LDS transpose, and no two lanes of different workgroups touch one row
 //     (atomic-free scatter);
-//   * a lane (m = lane%16, q = lane/16) needs, for row m, 16*KS contiguous bytes of the gathered
-//     row per channel chunk: they are loaded from global memory straight into the MFMA operand
+//   * a lane (m = lane%16, q = lane/16) needs, for row m, KS 16-byte pieces of the gathered row per
+//     channel chunk (piece s*4 + q for fragment s): they are loaded from global memory straight into the MFMA operand
 //     registers (the order of the contraction index inside a chunk is permuted identically for
 //     both operands, which leaves the product unchanged), so gathered rows never pass through LDS;
-//   * the weight slice of the current (offset, channel chunk) is staged by the whole workgroup
-//     into LDS in fragment order (double buffered, one barrier per step) and read back with
-//     conflict-free 16-byte reads;
-//   * each wave owns RB blocks of 16 rows; a block none of whose rows has a pair at offset k is
-//     skipped (its contribution would be exactly zero).
+//   * all gathers go through buffer descriptors: an absent pair (index -1), a row past the end or
+//     a channel past C is an out-of-range offset that the hardware answers with zeros, so the hot
+//     loop has no divergent branches;
+//   * kernel offsets are processed in batches of B: the gathered rows of a whole batch are
+//     requested together and the pair-table entries and weight slices of the NEXT batch are
+//     requested before the MFMAs of the current one, so a batch costs one memory round trip;
+//     weight slices are staged by the whole workgroup into LDS in fragment order (double
+//     buffered) and read back with conflict-free 16-byte reads;
+//   * tiles are handed out heaviest first; each wave owns RB blocks of 16 rows and skips a block
+//     none of whose rows has a pair at offset k (its contribution would be exactly zero).
 #pragma once
 #include "common.h"
 
@@ -40,6 +45,7 @@ struct RowGemmParams {
   const float *bias;
   int64_t lda, ldc, ldd;
   int64_t w_stride_n, w_stride_k, w_stride_c;  // element strides: out channel, offset, contraction
+  uint32_t a_bytes, w_bytes, c_bytes, d_bytes, gather_bytes;  // extents for the range checks
   int32_t n_pos, n_idx, rows_a, rows_c;
   int32_t c_in, k_out, kv;
   uint32_t mask_filter;
@@ -48,24 +54,31 @@ struct RowGemmParams {
   int32_t act;
   int32_t int8_epilogue;  // scale/bias requantisation instead of alpha/beta
   int32_t read_source;    // D is read (beta != 0)
-  int32_t xcd_swizzle;    // remap blockIdx.x so that neighbouring tiles share an XCD
 };
+
+constexpr uint32_t kOob = 0xffffffffu;  // an offset no buffer contains
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
 
 // T: element tag; NW: waves per workgroup; RB: 16-row blocks per wave; TN: output channels per
 // workgroup; KS: 16-byte fragments per lane per channel chunk; WT: weight is contiguous along the
-// output channel (needs a transposing stage) instead of along the contraction.
-template <class T, int NW, int RB, int TN, int KS, bool WT>
+// output channel (needs a transposing stage) instead of along the contraction; B: kernel offsets
+// per batch.
+template <class T, int NW, int RB, int TN, int KS, bool WT, int B>
 __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
   constexpr int TM = NW * RB * 16;
   constexpr int NB = TN / 16;               // MFMA row blocks (output channel blocks)
   constexpr int CPL = TN / 4;               // output channels per lane
-  constexpr int CHUNK_E = 4 * KS * E::kPerVec;  // contraction elements per chunk
-  constexpr int STAGE_V = NB * KS * 64;     // 16-byte vectors per LDS stage
+  constexpr int PV = E::kPerVec;
+  constexpr int CHUNK_E = 4 * KS * PV;      // contraction elements per chunk
+  constexpr int SLICE_V = NB * KS * 64;     // 16-byte vectors of one staged weight slice
   constexpr int NT = NW * 64;
 
-  __shared__ v4i lds_w[2][STAGE_V];
+  __shared__ v4i lds_w[2][B * SLICE_V];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -73,13 +86,10 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
   const int m = lane & 15;
   const int q = lane >> 4;
 
-  int tile = blockIdx.x;
-  if (p.xcd_swizzle) {
-    // workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous range of tiles
-    const int nt = gridDim.x;
-    const int per = nt >> 3;
-    if (tile < per * 8) tile = (tile & 7) * per + (tile >> 3);
-  }
+  // Tiles are handed out last-to-first: positions are sorted by ascending mask value, so the
+  // tiles with the most kernel offsets (the longest running ones) sit at the end of the sorted
+  // order and should start first, not last.
+  const int tile = (int)gridDim.x - 1 - (int)blockIdx.x;
   const int n0 = blockIdx.y * TN;
   const int pos_base = tile * TM;
 
@@ -104,14 +114,17 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
 
   // ---- rows owned by this lane
   int out_row[RB];
-  int key[RB];  // what the gather table is indexed with
+  uint32_t key_off[RB];  // byte offset of the lane's entry inside one row of the gather table
+  bool key_ok[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int pos = pos_base + (wave * RB + rb) * 16 + m;
     int o = -1;
     if (pos < p.n_pos) o = p.out_rows ? p.out_rows[pos] : pos;
     out_row[rb] = o;
-    key[rb] = p.gather_by_pos ? (pos < p.n_pos ? pos : -1) : o;
+    const int key = p.gather_by_pos ? (pos < p.n_pos ? pos : -1) : o;
+    key_ok[rb] = key >= 0 && key < p.n_idx;
+    key_off[rb] = key_ok[rb] ? (uint32_t)key * 4u : kOob;
   }
 
   AccV acc[RB][NB];
@@ -121,45 +134,49 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
     for (int nb = 0; nb < NB; ++nb) acc[rb][nb] = AccV{0, 0, 0, 0};
 
   const int n_chunks = (p.c_in + CHUNK_E - 1) / CHUNK_E;
-  const char *a_base = reinterpret_cast<const char *>(p.A);
-  const int64_t a_row_bytes = p.lda * E::kBytes;
+  const uint32_t a_row_bytes = (uint32_t)p.lda * E::kBytes;
+  const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(p.A, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(p.W, p.w_bytes);
+  const __amdgpu_buffer_rsrc_t rs_g = make_rsrc(p.gather, p.gather ? p.gather_bytes : 0u);
+  const bool has_gather = p.gather != nullptr;
 
+  // pair-table entries of offset k for the lane's rows (raw: fix_idx() maps absent ones to -1)
   auto load_idx = [&](int k, int (&idx)[RB]) {
+    const uint32_t base = (uint32_t)k * (uint32_t)p.n_idx * 4u;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      int v = -1;
-      const int kk = key[rb];
-      if (kk >= 0) {
-        if (p.gather != nullptr) {
-          if (p.gather_by_pos || kk < p.n_idx) v = p.gather[(int64_t)k * p.n_idx + kk];
-        } else {
-          v = kk;
-        }
+      if (has_gather) {
+        idx[rb] = __builtin_amdgcn_raw_buffer_load_b32(rs_g, key_ok[rb] ? base + key_off[rb] : kOob, 0, 0);
+      } else {
+        idx[rb] = (int)(key_off[rb] >> 2);
       }
-      if (v >= p.rows_a) v = -1;
-      idx[rb] = v;
     }
+  };
+  auto fix_idx = [&](int (&idx)[RB]) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      if (!key_ok[rb] || idx[rb] >= p.rows_a) idx[rb] = -1;
   };
 
   auto load_a = [&](const int (&idx)[RB], int chunk, v4i (&frag)[RB][KS]) {
-    const int e0 = chunk * CHUNK_E + q * KS * E::kPerVec;
+    // fragment s of lane quarter q is 16-byte piece s*4 + q of the chunk, so that one load
+    // instruction touches a single 64-byte segment of each gathered row
+    const int e0 = chunk * CHUNK_E + q * PV;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      const char *row = a_base + (int64_t)(idx[rb] < 0 ? 0 : idx[rb]) * a_row_bytes;
+      const uint32_t row = (uint32_t)idx[rb] * a_row_bytes;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
-        const int e = e0 + s * E::kPerVec;
-        v4i v = {0, 0, 0, 0};
-        if (idx[rb] >= 0 && e < p.c_in) v = *reinterpret_cast<const v4i *>(row + (int64_t)e * E::kBytes);
-        frag[rb][s] = v;
+        const int e = e0 + s * 4 * PV;
+        const uint32_t off = (idx[rb] >= 0 && e < p.c_in) ? row + (uint32_t)e * E::kBytes : kOob;
+        frag[rb][s] = __builtin_amdgcn_raw_buffer_load_b128(rs_a, off, 0, 0);
       }
     }
   };
 
   // weight staging: granule id -> (output channel, 16-byte piece of the chunk)
-  constexpr int GRAN = TN * 4 * KS;  // 16-byte granules per stage
+  constexpr int GRAN = TN * 4 * KS;  // 16-byte granules per offset
   constexpr int GPT = (GRAN + NT - 1) / NT;
-  const char *w_base = reinterpret_cast<const char *>(p.W);
 
   auto lds_slot = [&](int n_local, int g) -> int {
     // lane (m', q') of the reading wave holds channel n0 + q'*CPL + nb*4 + r as MFMA row 4*q'+r
@@ -168,76 +185,58 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
     const int nb = rem >> 2;
     const int r = rem & 3;
     const int rho = qo * 4 + r;
-    const int qq = g / KS;
-    const int s = g % KS;
-    return (nb * KS + s) * 64 + qq * 16 + rho;
+    const int qq = g % 4;
+    const int s = g / 4;
+    // the low bits are XOR-swizzled so that the staging writes of a wave spread over all banks
+    return (nb * KS + s) * 64 + qq * 16 + (rho ^ (qq << 2) ^ (nb & 3));
   };
 
-  v4i wreg[GPT];
-  auto load_w = [&](int k, int chunk) {
-    if constexpr (!WT) {
+  auto load_w = [&](int k, int chunk, v4i (&wreg)[GPT]) {
 #pragma unroll
-      for (int i = 0; i < GPT; ++i) {
-        const int id = tid + i * NT;
-        v4i v = {0, 0, 0, 0};
-        if (id < GRAN) {
-          const int n_local = id / (4 * KS);
-          const int g = id % (4 * KS);
-          const int n = n0 + n_local;
-          const int e = chunk * CHUNK_E + g * E::kPerVec;
-          if (n < p.k_out && e < p.c_in) {
-            const int64_t off = (int64_t)n * p.w_stride_n + (int64_t)k * p.w_stride_k + e;
-            v = *reinterpret_cast<const v4i *>(w_base + off * E::kBytes);
-          }
-        }
-        wreg[i] = v;
+    for (int i = 0; i < GPT; ++i) {
+      const int id = tid + i * NT;
+      uint32_t off = kOob;
+      if constexpr (!WT) {
+        const int n = n0 + id / (4 * KS);
+        const int e = chunk * CHUNK_E + (id % (4 * KS)) * PV;
+        if (id < GRAN && n < p.k_out && e < p.c_in)
+          off = (uint32_t)((int64_t)n * p.w_stride_n + (int64_t)k * p.w_stride_k + e) * E::kBytes;
+      } else {
+        // granule = PV consecutive OUTPUT channels at one contraction index
+        constexpr int NG = TN / PV;
+        const int n = n0 + (id % NG) * PV;
+        const int e = chunk * CHUNK_E + id / NG;
+        if (id < GRAN && n < p.k_out && e < p.c_in)
+          off = (uint32_t)((int64_t)e * p.w_stride_c + (int64_t)k * p.w_stride_k + n) * E::kBytes;
       }
-    } else {
-      // granule = kPerVec consecutive OUTPUT channels at one contraction index
-#pragma unroll
-      for (int i = 0; i < GPT; ++i) {
-        const int id = tid + i * NT;
-        v4i v = {0, 0, 0, 0};
-        if (id < GRAN) {
-          constexpr int NG = TN / E::kPerVec;  // granules along the output channels
-          const int c_local = id / NG;         // contraction index inside the chunk
-          const int ng = id % NG;
-          const int n = n0 + ng * E::kPerVec;
-          const int e = chunk * CHUNK_E + c_local;
-          if (n < p.k_out && e < p.c_in) {
-            const int64_t off = (int64_t)e * p.w_stride_c + (int64_t)k * p.w_stride_k + n;
-            v = *reinterpret_cast<const v4i *>(w_base + off * E::kBytes);
-          }
-        }
-        wreg[i] = v;
-      }
+      wreg[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, off, 0, 0);
     }
   };
 
-  auto store_w = [&](int buf) {
+  auto store_w = [&](v4i *stage, const v4i (&wreg)[GPT]) {
     if constexpr (!WT) {
 #pragma unroll
       for (int i = 0; i < GPT; ++i) {
         const int id = tid + i * NT;
-        if (id < GRAN) lds_w[buf][lds_slot(id / (4 * KS), id % (4 * KS))] = wreg[i];
+        if (id < GRAN) stage[lds_slot(id / (4 * KS), id % (4 * KS))] = wreg[i];
       }
     } else {
-      constexpr int NG = TN / E::kPerVec;
+      constexpr int NG = TN / PV;
 #pragma unroll
       for (int i = 0; i < GPT; ++i) {
         const int id = tid + i * NT;
         if (id < GRAN) {
           const int c_local = id / NG;
           const int ng = id % NG;
-          const int g = c_local / E::kPerVec;  // 16-byte piece along the contraction
-          const int j = c_local % E::kPerVec;  // element inside the piece
+          const int g = c_local / PV;  // 16-byte piece along the contraction
+          const int j = c_local % PV;  // element inside the piece
           if constexpr (E::kBytes == 2) {
-            uint16_t *dst = reinterpret_cast<uint16_t *>(&lds_w[buf][0]);
+            uint16_t *dst = reinterpret_cast<uint16_t *>(stage);
             const uint16_t *src = reinterpret_cast<const uint16_t *>(&wreg[i]);
 #pragma unroll
             for (int x = 0; x < 8; ++x) dst[lds_slot(ng * 8 + x, g) * 8 + j] = src[x];
           } else {
-            uint8_t *dst = reinterpret_cast<uint8_t *>(&lds_w[buf][0]);
+            uint8_t *dst = reinterpret_cast<uint8_t *>(stage);
             const uint8_t *src = reinterpret_cast<const uint8_t *>(&wreg[i]);
 #pragma unroll
             for (int x = 0; x < 16; ++x) dst[lds_slot(ng * 16 + x, g) * 16 + j] = src[x];
@@ -247,73 +246,93 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
     }
   };
 
+  // ---- steps: (batch of up to B offsets) x (channel chunk); the next step's pair-table entries
+  // and weight slices are in flight while the current step computes
   if (kmask != 0) {
-    // ---- software pipeline over (offset, chunk) steps
     uint32_t rem = kmask;
-    int k_cur = __builtin_ctz(rem);
-    rem &= rem - 1;
-    int k_nxt = rem ? __builtin_ctz(rem) : -1;
-    if (rem) rem &= rem - 1;
-
-    int idx_cur[RB], idx_nxt[RB];
-    load_idx(k_cur, idx_cur);
-    if (k_nxt >= 0) load_idx(k_nxt, idx_nxt);
-
-    v4i a_nxt[RB][KS];
-    load_a(idx_cur, 0, a_nxt);
-    load_w(k_cur, 0);
-    bool any_nxt[RB];
+    auto take = [&](int (&ko)[B]) {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) any_nxt[rb] = __ballot(idx_cur[rb] >= 0) != 0;
-
+      for (int j = 0; j < B; ++j) {
+        ko[j] = rem ? __builtin_ctz(rem) : -1;
+        if (rem) rem &= rem - 1;
+      }
+    };
+    int koff[B];
+    take(koff);
     int chunk = 0;
+    int idx[B][RB];
+    v4i wreg[B][GPT];
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      if (koff[j] >= 0) {
+        load_w(koff[j], 0, wreg[j]);
+        load_idx(koff[j], idx[j]);
+      }
+    }
     int buf = 0;
     bool more = true;
     while (more) {
-      v4i a_cur[RB][KS];
-      bool any_cur[RB];
+      // park the weight slices of this step in LDS (their requests went out a step ago)
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        any_cur[rb] = any_nxt[rb];
+      for (int j = 0; j < B; ++j)
+        if (koff[j] >= 0) store_w(&lds_w[buf][j * SLICE_V], wreg[j]);
+      if (chunk == 0) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) a_cur[rb][s] = a_nxt[rb][s];
-      }
-      store_w(buf);
-      __syncthreads();
-
-      // advance to the next step and start its loads
-      if (chunk + 1 < n_chunks) {
-        ++chunk;
-      } else {
-        chunk = 0;
-        k_cur = k_nxt;
-        if (k_cur >= 0) {
+        for (int j = 0; j < B; ++j) {
+          if (koff[j] >= 0) {
+            fix_idx(idx[j]);
+          } else {
 #pragma unroll
-          for (int rb = 0; rb < RB; ++rb) idx_cur[rb] = idx_nxt[rb];
-          k_nxt = rem ? __builtin_ctz(rem) : -1;
-          if (rem) rem &= rem - 1;
-          if (k_nxt >= 0) load_idx(k_nxt, idx_nxt);
+            for (int rb = 0; rb < RB; ++rb) idx[j][rb] = -1;
+          }
         }
       }
-      more = k_cur >= 0;
-      if (more) {
-        load_a(idx_cur, chunk, a_nxt);
-        load_w(k_cur, chunk);
+      // request every gathered row of the step
+      v4i afrag[B][RB][KS];
+      bool any[B][RB];
+      int kcur[B];
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) any_nxt[rb] = __ballot(idx_cur[rb] >= 0) != 0;
+      for (int j = 0; j < B; ++j) {
+        kcur[j] = koff[j];
+        if (koff[j] >= 0) load_a(idx[j], chunk, afrag[j]);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) any[j][rb] = koff[j] >= 0 && __ballot(idx[j][rb] >= 0) != 0;
       }
-
-      // ---- MFMA over the staged weight slice
+      // advance and request the next step's weight slices and pair-table entries
+      if (chunk + 1 < n_chunks) {
+        ++chunk;
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        v4i wf[KS];
+        for (int j = 0; j < B; ++j)
+          if (koff[j] >= 0) load_w(koff[j], chunk, wreg[j]);
+      } else if (rem != 0) {
+        chunk = 0;
+        take(koff);
 #pragma unroll
-        for (int s = 0; s < KS; ++s) wf[s] = lds_w[buf][(nb * KS + s) * 64 + lane];
+        for (int j = 0; j < B; ++j) {
+          if (koff[j] >= 0) {
+            load_w(koff[j], 0, wreg[j]);
+            load_idx(koff[j], idx[j]);
+          }
+        }
+      } else {
+        more = false;
+      }
+      __syncthreads();  // this stage is written; every wave has left the other one
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          if (any_cur[rb]) {
+      for (int j = 0; j < B; ++j) {
+        if (kcur[j] < 0) continue;
+        const v4i *stage = &lds_w[buf][j * SLICE_V];
 #pragma unroll
-            for (int s = 0; s < KS; ++s) acc[rb][nb] = E::mfma(wf[s], a_cur[rb][s], acc[rb][nb]);
+        for (int nb = 0; nb < NB; ++nb) {
+          v4i wf[KS];
+#pragma unroll
+          for (int s = 0; s < KS; ++s) wf[s] = stage[(nb * KS + s) * 64 + (lane ^ ((q << 2) ^ (nb & 3)))];
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            if (any[j][rb]) {
+#pragma unroll
+              for (int s = 0; s < KS; ++s) acc[rb][nb] = E::mfma(wf[s], afrag[j][rb][s], acc[rb][nb]);
+            }
           }
         }
       }
@@ -322,21 +341,25 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
   }
 
   // ---- epilogue: lane (m, q) owns channels [n0 + q*CPL, n0 + (q+1)*CPL) of row out_row[rb]
+  const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.c_bytes);
+  const __amdgpu_buffer_rsrc_t rs_d = make_rsrc(p.D, p.read_source ? p.d_bytes : 0u);
   const int ch0 = n0 + q * CPL;
   if constexpr (E::kBytes == 2) {
     constexpr int NG = CPL / 8;  // 16-byte groups of 8 channels
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const int o = out_row[rb];
-      if (o < 0 || o >= p.rows_c) continue;
-      uint16_t *crow = reinterpret_cast<uint16_t *>(p.C) + (int64_t)o * p.ldc;
-      const uint16_t *drow = reinterpret_cast<const uint16_t *>(p.D) + (int64_t)o * p.ldd;
+      const bool row_ok = o >= 0 && o < p.rows_c;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
         const int ch = ch0 + g * 8;
-        if (ch >= p.k_out) continue;
+        const bool ok = row_ok && ch < p.k_out;
+        const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
         v4i src = {0, 0, 0, 0};
-        if (p.read_source) src = *reinterpret_cast<const v4i *>(drow + ch);
+        if (p.read_source) {
+          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 2u : kOob;
+          src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
+        }
         const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
         v4i outv;
         uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
@@ -352,7 +375,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
           t = apply_act(t, p.act, p.act_alpha);
           oh[x] = E::from_float(t);
         }
-        *reinterpret_cast<v4i *>(crow + ch) = outv;
+        __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
       }
     }
   } else {
@@ -362,15 +385,17 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const int o = out_row[rb];
-      if (o < 0 || o >= p.rows_c) continue;
-      int8_t *crow = reinterpret_cast<int8_t *>(p.C) + (int64_t)o * p.ldc;
-      const int8_t *drow = reinterpret_cast<const int8_t *>(p.D) + (int64_t)o * p.ldd;
+      const bool row_ok = o >= 0 && o < p.rows_c;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
         const int ch = ch0 + g * 16;
-        if (ch >= p.k_out) continue;
+        const bool ok = row_ok && ch < p.k_out;
+        const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) : kOob;
         v4i src = {0, 0, 0, 0};
-        if (p.read_source) src = *reinterpret_cast<const v4i *>(drow + ch);
+        if (p.read_source) {
+          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) : kOob;
+          src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
+        }
         const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
         v4i outv;
         int8_t *ob = reinterpret_cast<int8_t *>(&outv);
@@ -381,7 +406,8 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
           if (p.int8_epilogue) {
             // Int8Inference: scale*acc + bias, then beta*source + that
             // (cumm/gemm/output_op/linear.py:279-325 of the reference)
-            t = __builtin_fmaf(p.scale[ch + x], (float)a, p.bias[ch + x]);
+            const int c = ch + x < p.k_out ? ch + x : 0;
+            t = __builtin_fmaf(p.scale[c], (float)a, p.bias[c]);
             if (p.read_source) t = __builtin_fmaf(p.beta, (float)sb[x], t);
           } else if (p.read_source) {
             t = __builtin_fmaf(p.alpha, (float)a, p.beta * (float)sb[x]);
@@ -391,7 +417,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
           t = apply_act(t, p.act, p.act_alpha);
           ob[x] = (int8_t)f32_to_s8(t);
         }
-        *reinterpret_cast<v4i *>(crow + ch) = outv;
+        __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
       }
     }
   }

@@ -1,17 +1,47 @@
 // Instantiations of the gather-rows GEMM for one element type (selected with -DCUMM_ELEM=...).
 #include "launch.h"
+#include "rowgemm_pipe.h"
 
 namespace cummhip {
 
 #define CUMM_CAT_(a, b) a##b
 #define CUMM_CAT(a, b) CUMM_CAT_(a, b)
 
+// kernel offsets per batch of the chunked kernel: bounded by the two LDS stages (TN * 64 * KS
+// bytes per offset and stage, at most 32 KB per workgroup) and by the registers that hold the
+// batch's gathered rows
+constexpr int batch_size(int RB, int TN, int KS) {
+  int b = 4;
+  while (b > 1 && (2 * b * TN * 64 * KS > 32768 || RB * KS * b > 16)) b >>= 1;
+  return b;
+}
+// offsets per step of the pipelined kernel: two where both LDS stages then fit 32 KB
+constexpr int step_width(int TN, int KS) { return 2 * 2 * TN * 64 * KS <= 32768 ? 2 : 1; }
+// steps of gathered rows kept in flight: as many as fit about 48 registers
+constexpr int rows_ahead(int RB, int KS, int BW) {
+  int d = 3;
+  while (d > 1 && (d + 1) * BW * RB * KS * 4 > 64) --d;
+  return d;
+}
+
 template <class T, int NW, int RB, int TN, int KS, bool WT>
 static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   constexpr int TM = NW * RB * 16;
   dim3 grid((p.n_pos + TM - 1) / TM, (p.k_out + TN - 1) / TN, 1);
   if (grid.x == 0 || grid.y == 0) return hipSuccess;
-  hipLaunchKernelGGL((rowgemm_kernel<T, NW, RB, TN, KS, WT>), grid, dim3(NW * 64), 0, s, p);
+  constexpr int chunk_e = 4 * KS * Elem<T>::kPerVec;
+  if (p.c_in <= chunk_e) {
+    constexpr int BW = step_width(TN, KS);
+    constexpr int DA = rows_ahead(RB, KS, BW);
+    hipLaunchKernelGGL((rowgemm_pipe_kernel<T, NW, RB, TN, KS, WT, BW, DA, DA>), grid, dim3(NW * 64), 0, s, p);
+  } else {
+    if constexpr (KS == 4) {
+      constexpr int B = batch_size(RB, TN, KS);
+      hipLaunchKernelGGL((rowgemm_kernel<T, NW, RB, TN, KS, WT, B>), grid, dim3(NW * 64), 0, s, p);
+    } else {
+      return hipErrorInvalidValue;  // a contraction longer than one chunk always selects KS == 4
+    }
+  }
   return hipGetLastError();
 }
 

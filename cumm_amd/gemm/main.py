@@ -167,8 +167,15 @@ class GemmMainUnitTest:
     def matmul2(params: GemmParams) -> None:
         """C = act(alpha * op(A) @ op(B) + beta * D) with optional row gather /
         scatter; prelude cumm/gemm/nvrtc_code.py:34-146 of the reference."""
-        params.check_valid()
         desp = params.algo_desp
+        prep = params.__dict__.get("_prepared")
+        if prep is not None and prep[0] == (params._version, desp._version, desp.tile_shape[0],
+                                            desp.tile_shape[1], desp.tile_shape[2]):
+            status = prep[1](prep[2], prep[3], params.stream)
+            if status:
+                _capi.check(status)
+            return
+        params.check_valid()
         a, b, c = params.a, params.b, params.c
         d = params.d if not params.d.empty() else c
         _check_shape(a, [-1, -1])
@@ -260,7 +267,15 @@ class GemmMainUnitTest:
         name = repr(desp) if params.timer.enable else ""
         if name:
             params.timer.record(name, params.stream)
-        status = _capi.lib().cumm_hip_gemm(ctypes.byref(cdesc), ctypes.byref(args), params.stream)
+        fn = _capi.lib().cumm_hip_gemm
+        status = fn(ctypes.byref(cdesc), ctypes.byref(args), params.stream)
         if name:
             params.timer.record(name, params.stream)
         _capi.check(status)
+        if not name:
+            # validated argument block for unchanged repeat calls; the workspace it may point to
+            # is kept alive with it
+            params.__dict__["_prepared"] = (
+                (params._version, desp._version, desp.tile_shape[0], desp.tile_shape[1],
+                 desp.tile_shape[2]), fn, ctypes.byref(cdesc), ctypes.byref(args), cdesc, args,
+                workspace)

@@ -140,7 +140,18 @@ class NVRTCParams:
         self.mode = -1
 
 
-class GemmAlgoDesp:
+class _Versioned:
+    """Counts attribute assignments so that the operators can tell cheaply whether a
+    parameter object changed since they last validated it."""
+    _version = 0
+
+    def __setattr__(self, name, value):
+        object.__setattr__(self, name, value)   # honours the property setters
+        d = self.__dict__
+        d["_version"] = d.get("_version", 0) + 1
+
+
+class GemmAlgoDesp(_Versioned):
     """tv::gemm::GemmAlgoDesp, include/tensorview/gemm/core/params.h:24-164."""
 
     def __init__(self):
@@ -354,7 +365,7 @@ def _empty_tensor():
     return Tensor()
 
 
-class GemmParams:
+class GemmParams(_Versioned):
     """tv::gemm::GemmParams, params.h:329-390.  Setting ``a``/``b``/``c`` also
     records the dtype in ``algo_desp`` (params.h:366-383)."""
 
@@ -411,7 +422,7 @@ class GemmParams:
                 raise RuntimeError("a_inds,b_inds tensor must not empty")
 
 
-class ConvParams:
+class ConvParams(_Versioned):
     """tv::gemm::ConvParams, params.h:392-428."""
 
     def __init__(self, ndim: int, op_type, timer=None):
