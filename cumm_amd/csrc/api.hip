@@ -81,10 +81,10 @@ hipError_t launch_tilegemm(int dt, int tm, int tn, bool xk, bool yk, const TileG
 constexpr int kSpinLimit = 1 << 24;
 
 // byte extent of a row-major 2-D operand for the buffer range checks; false if it does not fit
-// the 32-bit offsets the kernels use
+// below 2 GiB (the kernels use 32-bit offsets and reserve the upper half for "absent")
 bool extent32(int64_t rows, int64_t ld, int64_t cols, int esize, uint32_t *out) {
   const int64_t bytes = rows <= 0 ? 0 : ((rows - 1) * ld + cols) * esize;
-  if (bytes < 0 || bytes >= (int64_t)1 << 32) return false;
+  if (bytes < 0 || bytes >= (int64_t)1 << 31) return false;
   *out = (uint32_t)bytes;
   return true;
 }
@@ -407,7 +407,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
         !extent32((int64_t)a->K * kv, a->C, a->C, eb, &p.w_bytes) ||
         !extent32(p.rows_c, p.ldc, p.k_out, eb, &p.c_bytes) ||
         !extent32(p.ldd ? p.rows_c : 1, p.ldd, p.k_out, eb, &p.d_bytes) ||
-        (int64_t)kv * a->N * 4 >= (int64_t)1 << 32)
+        (int64_t)kv * a->N * 4 >= (int64_t)1 << 31)
       return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
     p.gather_bytes = (uint32_t)((int64_t)kv * a->N * 4);
     hipError_t e = launch_rowgemm(dt, d.tile_shape[0], d.tile_shape[1], pick_ks(p.c_in, dt), !fwd, p, stream);

@@ -56,7 +56,9 @@ struct RowGemmParams {
   int32_t read_source;    // D is read (beta != 0)
 };
 
-constexpr uint32_t kOob = 0xffffffffu;  // an offset no buffer contains
+// An offset no buffer contains: every operand is smaller than 2 GiB (checked on the host), and
+// adding a scalar offset below 2 GiB to it cannot wrap back into range.
+constexpr uint32_t kOob = 0x80000000u;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);

@@ -19,7 +19,7 @@ constexpr int batch_size(int RB, int TN, int KS) {
 constexpr int step_width(int TN, int KS) { return 2 * 2 * TN * 64 * KS <= 32768 ? 2 : 1; }
 // steps of gathered rows kept in flight: as many as fit about 48 registers
 constexpr int rows_ahead(int RB, int KS, int BW) {
-  int d = 3;
+  int d = 2;
   while (d > 1 && (d + 1) * BW * RB * KS * 4 > 64) --d;
   return d;
 }

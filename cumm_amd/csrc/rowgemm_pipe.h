@@ -14,7 +14,11 @@
 // pair-table entries, then rows): waiting for what the next step needs never waits for what a
 // later step needs.  The register sets form rings that are indexed at compile time (the step
 // loop is unrolled by the ring length), because copying a register that a load is still filling
-// would wait for the load.
+// would wait for the load.  For the same reason the step body is straight-line code: a load that
+// is skipped on one path makes the number of outstanding loads path dependent and the compiler
+// then waits for all of them; a kernel offset past the end of the tile mask is therefore not
+// skipped but loaded through an empty buffer descriptor (every lane out of range, zeros back,
+// no memory traffic).
 #pragma once
 #include <type_traits>
 #include <utility>
@@ -103,18 +107,55 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
   const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(p.A, p.a_bytes);
   const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(p.W, p.w_bytes);
   const __amdgpu_buffer_rsrc_t rs_g = make_rsrc(p.gather, p.gather ? p.gather_bytes : 0u);
+  const __amdgpu_buffer_rsrc_t rs_none = make_rsrc(p.A, 0u);   // every offset out of range
   const bool has_gather = p.gather != nullptr;
 
   constexpr int GRAN = TN * 4 * KS;
   constexpr int GPT = (GRAN + NT - 1) / NT;
 
+  // ---- everything about addresses that does not depend on the kernel offset is computed once:
+  // the step loop is bound by instruction issue as soon as it recomputes them per step.
+  // gathered rows: piece s*4 + q of the row (one 64-byte segment of each row per instruction)
+  const uint32_t a_col = (uint32_t)q * 16u;
+  bool a_col_ok[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) a_col_ok[s] = (s * 4 + q) * PV < p.c_in;
+  // weight granules of this thread: byte offset at kernel offset 0 and LDS slot (16-byte units)
+  uint32_t w_voff[GPT];
+  int w_slot[GPT];   // non-transposing: slot of the granule; transposing: see park_w
+  const uint32_t w_k_bytes = (uint32_t)p.w_stride_k * E::kBytes;
+#pragma unroll
+  for (int i = 0; i < GPT; ++i) {
+    const int id = tid + i * NT;
+    w_voff[i] = kOob;
+    w_slot[i] = 0;
+    if constexpr (!WT) {
+      const int n_local = id / (4 * KS), g = id % (4 * KS);
+      const int n = n0 + n_local, e = g * PV;
+      if (id < GRAN && n < p.k_out && e < p.c_in)
+        w_voff[i] = (uint32_t)((int64_t)n * p.w_stride_n + e) * E::kBytes;
+      const int qo = n_local / CPL, rem = n_local % CPL, nb = rem >> 2, r = rem & 3, qq = g % 4;
+      // the low bits are XOR-swizzled so that the staging writes of a wave spread over all banks
+      w_slot[i] = (nb * KS + g / 4) * 64 + qq * 16 + ((qo * 4 + r) ^ (qq << 2) ^ (nb & 3));
+    } else {
+      constexpr int NG = TN / PV;
+      const int n = n0 + (id % NG) * PV, e = id / NG;
+      if (id < GRAN && n < p.k_out && e < p.c_in)
+        w_voff[i] = (uint32_t)((int64_t)e * p.w_stride_c + n) * E::kBytes;
+    }
+  }
+  // LDS read position of this lane inside a 64-slot fragment, one per swizzle variant (nb & 3)
+  int rd_slot[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) rd_slot[v] = lane ^ ((q << 2) ^ v);
+
+  // slot of (output channel n_local, contraction piece g) for the transposing stage
   auto lds_slot = [&](int n_local, int g) -> int {
     const int qo = n_local / CPL;
     const int rem = n_local % CPL;
     const int nb = rem >> 2;
     const int r = rem & 3;
     const int qq = g % 4;
-    // the low bits are XOR-swizzled so that the staging writes of a wave spread over all banks
     return (nb * KS + g / 4) * 64 + qq * 16 + ((qo * 4 + r) ^ (qq << 2) ^ (nb & 3));
   };
 
@@ -136,21 +177,19 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
     }
   };
 
+  const uint32_t g_k_bytes = (uint32_t)p.n_idx * 4u;
   auto issue_idx = [&](int (&dst)[BW][RB]) {
     int ko[BW];
     take(rem_i, ko);
 #pragma unroll
     for (int j = 0; j < BW; ++j) {
-      const uint32_t base = (uint32_t)(ko[j] < 0 ? 0 : ko[j]) * (uint32_t)p.n_idx * 4u;
+      const bool live = ko[j] >= 0 && has_gather;
+      const __amdgpu_buffer_rsrc_t rs = live ? rs_g : rs_none;
+      const uint32_t soff = live ? (uint32_t)ko[j] * g_k_bytes : 0u;   // row of the table
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        if (ko[j] < 0) {
-          dst[j][rb] = -1;
-        } else if (has_gather) {
-          dst[j][rb] = __builtin_amdgcn_raw_buffer_load_b32(rs_g, key_ok[rb] ? base + key_off[rb] : kOob, 0, 0);
-        } else {
-          dst[j][rb] = key_ok[rb] ? (int)(key_off[rb] >> 2) : -1;
-        }
+        const int v = __builtin_amdgcn_raw_buffer_load_b32(rs, key_off[rb], soff, 0);
+        dst[j][rb] = has_gather ? v : (int)(key_off[rb] >> 2);
       }
     }
   };
@@ -160,17 +199,20 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
     take(rem_a, kdst);
 #pragma unroll
     for (int j = 0; j < BW; ++j) {
+      const bool live = kdst[j] >= 0;
+      const __amdgpu_buffer_rsrc_t rs = live ? rs_a : rs_none;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        int v = src[j][rb];
-        if (kdst[j] < 0 || !key_ok[rb] || v >= p.rows_a) v = -1;
-        anyd[j][rb] = __ballot(v >= 0);
-        const uint32_t row = (uint32_t)v * a_row_bytes;
+        const int v = src[j][rb];
+        const bool ok = key_ok[rb] && v >= 0 && v < p.rows_a;
+        anyd[j][rb] = live ? __ballot(ok) : 0;
+        const uint32_t row = (uint32_t)v * a_row_bytes + a_col;
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-          const int e = (s * 4 + q) * PV;   // one 64-byte segment of each row per instruction
-          const uint32_t off = (v >= 0 && e < p.c_in) ? row + (uint32_t)e * E::kBytes : kOob;
-          if (kdst[j] >= 0) dst[j][rb][s] = __builtin_amdgcn_raw_buffer_load_b128(rs_a, off, 0, 0);
+          // branch-free select (a ?: here is turned into two loads under complementary masks)
+          const uint32_t keep = 0u - (uint32_t)(ok && a_col_ok[s]);
+          dst[j][rb][s] = __builtin_amdgcn_raw_buffer_load_b128(
+              rs, ((row + (uint32_t)(s * 64)) & keep) | (kOob & ~keep), 0, 0);
         }
       }
     }
@@ -181,39 +223,22 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
     take(rem_w, ko);
 #pragma unroll
     for (int j = 0; j < BW; ++j) {
-      if (ko[j] < 0) continue;
+      const bool live = ko[j] >= 0;
+      const __amdgpu_buffer_rsrc_t rs = live ? rs_w : rs_none;
+      const uint32_t soff = live ? (uint32_t)ko[j] * w_k_bytes : 0u;
 #pragma unroll
-      for (int i = 0; i < GPT; ++i) {
-        const int id = tid + i * NT;
-        uint32_t off = kOob;
-        if constexpr (!WT) {
-          const int n = n0 + id / (4 * KS);
-          const int e = (id % (4 * KS)) * PV;
-          if (id < GRAN && n < p.k_out && e < p.c_in)
-            off = (uint32_t)((int64_t)n * p.w_stride_n + (int64_t)ko[j] * p.w_stride_k + e) * E::kBytes;
-        } else {
-          constexpr int NG = TN / PV;
-          const int n = n0 + (id % NG) * PV;
-          const int e = id / NG;
-          if (id < GRAN && n < p.k_out && e < p.c_in)
-            off = (uint32_t)((int64_t)e * p.w_stride_c + (int64_t)ko[j] * p.w_stride_k + n) * E::kBytes;
-        }
-        wreg[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, off, 0, 0);
-      }
+      for (int i = 0; i < GPT; ++i) wreg[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rs, w_voff[i], soff, 0);
     }
   };
 
   auto park_w = [&](int buf, const int (&kcur)[BW]) {
 #pragma unroll
     for (int j = 0; j < BW; ++j) {
-      if (kcur[j] < 0) continue;
       v4i *stage = &lds_w[buf][j * SLICE_V];
       if constexpr (!WT) {
 #pragma unroll
-        for (int i = 0; i < GPT; ++i) {
-          const int id = tid + i * NT;
-          if (id < GRAN) stage[lds_slot(id / (4 * KS), id % (4 * KS))] = wreg[j][i];
-        }
+        for (int i = 0; i < GPT; ++i)
+          if (tid + i * NT < GRAN) stage[w_slot[i]] = wreg[j][i];
       } else {
         constexpr int NG = TN / PV;
 #pragma unroll
@@ -270,20 +295,23 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
       __syncthreads();
 #pragma unroll
       for (int j = 0; j < BW; ++j) {
-        if (kcur[j] < 0) continue;
+        uint64_t any_j = 0;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) any_j |= any_a[sa][j][rb];
+        if (any_j == 0) continue;   // no row of this wave has a pair at this offset
         const v4i *stage = &lds_w[buf][j * SLICE_V];
+        v4i wf[NB][KS];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          v4i wf[KS];
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int s = 0; s < KS; ++s) wf[s] = stage[(nb * KS + s) * 64 + (lane ^ ((q << 2) ^ (nb & 3)))];
+          for (int s = 0; s < KS; ++s) wf[nb][s] = stage[(nb * KS + s) * 64 + rd_slot[nb & 3]];
 #pragma unroll
-          for (int rb = 0; rb < RB; ++rb) {
-            if (any_a[sa][j][rb] != 0) {
+        for (int rb = 0; rb < RB; ++rb) {
+          if (RB > 1 && any_a[sa][j][rb] == 0) continue;
 #pragma unroll
-              for (int s = 0; s < KS; ++s) acc[rb][nb] = E::mfma(wf[s], afrag[sa][j][rb][s], acc[rb][nb]);
-            }
-          }
+          for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int s = 0; s < KS; ++s) acc[rb][nb] = E::mfma(wf[nb][s], afrag[sa][j][rb][s], acc[rb][nb]);
         }
       }
       buf ^= 1;
