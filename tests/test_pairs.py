@@ -1,0 +1,58 @@
+"""The host pair-table builder against the oracle's brute-force dictionary search
+(bit-exact), on SubM and strided problems, with ragged / tiny / dilated cases."""
+import numpy as np
+import pytest
+
+from oracle import pairs_ref
+
+from cumm_amd import pairs, synth
+
+
+@pytest.mark.parametrize("seed,n,grid,dil", [(0, 300, (8, 20, 18), (1, 1, 1)), (1, 1, (3, 3, 3), (1, 1, 1)),
+                                             (2, 500, (5, 30, 30), (2, 1, 2)), (3, 64, (4, 4, 4), (1, 1, 1))])
+def test_subm_pairs_bit_exact(seed, n, grid, dil):
+    rng = np.random.default_rng(seed)
+    coords = synth.clustered_voxels(rng, n, grid, 3, sigma=2.5)
+    pt = pairs.subm_pairs(coords, grid, dilation=dil)
+    ref = pairs_ref.subm_pairs_ref(coords, grid, dilation=dil)
+    np.testing.assert_array_equal(pt.indices_fwd, ref)
+    np.testing.assert_array_equal(pt.mask_fwd, pairs_ref.masks_ref(ref))
+    assert pt.indices_fwd.dtype == np.int32 and pt.mask_fwd.dtype == np.uint32
+
+
+@pytest.mark.parametrize("seed,n,grid,stride,pad", [(0, 300, (9, 21, 18), (2, 2, 2), (1, 1, 1)),
+                                                    (1, 2, (4, 4, 4), (2, 2, 2), (1, 1, 1)),
+                                                    (2, 400, (8, 16, 17), (1, 2, 2), (1, 1, 1)),
+                                                    (3, 200, (10, 10, 10), (2, 2, 2), (0, 0, 0))])
+def test_strided_pairs_bit_exact(seed, n, grid, stride, pad):
+    rng = np.random.default_rng(seed)
+    coords = synth.clustered_voxels(rng, n, grid, 3, sigma=2.5)
+    pt = pairs.sparse_conv_pairs(coords, grid, stride=stride, padding=pad)
+    f, b, oc = pairs_ref.sparse_conv_pairs_ref(coords, grid, (3, 3, 3), stride, pad, (1, 1, 1))
+    np.testing.assert_array_equal(pt.out_coords, oc)
+    np.testing.assert_array_equal(pt.indices_fwd, f)
+    np.testing.assert_array_equal(pt.indices_bwd, b)
+    np.testing.assert_array_equal(pt.mask_fwd, pairs_ref.masks_ref(f))
+    np.testing.assert_array_equal(pt.mask_bwd, pairs_ref.masks_ref(b))
+    assert pt.out_shape == pairs_ref.calc_output_dims(grid, (3, 3, 3), pad, stride, (1, 1, 1))
+    assert (pt.indices_fwd >= 0).sum() == (pt.indices_bwd >= 0).sum()
+
+
+def test_sort_by_mask_is_stable_and_filtered():
+    m = np.array([5, 1, 5, 0, 1, 8 | 5], np.uint32)
+    ms, order = pairs.sort_by_mask(m)
+    np.testing.assert_array_equal(order, [3, 1, 4, 0, 2, 5])
+    np.testing.assert_array_equal(ms, m[order])
+    ms2, order2 = pairs.sort_by_mask(m, 0x4)
+    np.testing.assert_array_equal(ms2, (m & 4)[order2])
+    np.testing.assert_array_equal(order2, [1, 3, 4, 0, 2, 5])
+
+
+def test_synthetic_cloud_is_unique_in_grid_and_seeded():
+    grid = (41, 200, 176)
+    a = synth.clustered_voxels(np.random.default_rng(7), 5000, grid, 8)
+    b = synth.clustered_voxels(np.random.default_rng(7), 5000, grid, 8)
+    np.testing.assert_array_equal(a, b)
+    assert len({tuple(r) for r in a.tolist()}) == a.shape[0]
+    assert (a[:, 1:] >= 0).all() and (a[:, 1:] < np.array(grid)).all()
+    assert abs(a.shape[0] - 5000) < 100
