@@ -140,6 +140,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
     ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch the plain copy kernel on 512 MiB (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)",
@@ -169,6 +172,15 @@ def main():
 
     def step():
         ConvMainUnitTest.implicit_gemm2(p)
+
+    if args.calibrate_copy:
+        import ctypes
+        from cumm_amd import _capi
+        nbytes = 512 << 20
+        src, dst = tv.zeros([nbytes], tv.uint8, 0), tv.zeros([nbytes], tv.uint8, 0)
+        for _ in range(5):
+            _capi.check(_capi.lib().cumm_hip_copy_kernel(dst.byte_pointer(), src.byte_pointer(), nbytes, 0))
+        ConvMainUnitTest_sync()
 
     wall_ms, ev_ms = timed(step, args.steps, args.warmup)
     flops = 2.0 * P * C * K
