@@ -33,12 +33,13 @@ GRID = (41, 1600, 1408)
 SEED = 20240607
 
 
-def find_desp(tv_dtype, op, tile_m, tile_n, int8=False):
+def find_desp(tv_dtype, op, tile_m, tile_n, int8=False, parallel=False):
     for d in ConvMainUnitTest.get_all_conv_algo_desp():
         if (d.dtype_a == tv_dtype and ConvOpType(d.op_type) == op and d.tile_shape[0] == tile_m
-                and d.tile_shape[1] == tile_n and d.is_int8_inference == int8):
+                and d.tile_shape[1] == tile_n and d.is_int8_inference == int8
+                and d.split_k_parallel == parallel):
             return d
-    raise KeyError((tv_dtype, op, tile_m, tile_n, int8))
+    raise KeyError((tv_dtype, op, tile_m, tile_n, int8, parallel))
 
 
 def dev(arr):
@@ -90,17 +91,18 @@ def bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops):
             "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3)}
 
 
-def bench_wgrad(args, p, dout, n, C, K, tile_m, flops):
+def bench_wgrad(args, p, dout, n, C, K, tile_m, flops, parallel):
     pw = ConvParams(3, ConvOpType.BackwardWeight)
-    pw.conv_algo_desp = find_desp(tv.float16, ConvOpType.BackwardWeight, 64, 64)
+    pw.conv_algo_desp = find_desp(tv.float16, ConvOpType.BackwardWeight, 64, 64, parallel=parallel)
     pw.input, pw.output = p.input, dout
     pw.weight = tv.zeros([K, 27, C], tv.float16, 0)
     pw.indices, pw.mask_argsort = p.indices, p.mask_argsort
     pw.mask = p.mask_output       # written by the forward pass above
     pw.mask_width = tile_m
     pw.split_k_slices = 32
-    w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), max(1, args.steps // 4),
-                       max(1, args.warmup // 4))
+    div = 1 if parallel else 4
+    w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), max(1, args.steps // div),
+                       max(1, args.warmup // div))
     return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
             "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3)}
 
@@ -220,7 +222,8 @@ def main():
         if "dgrad" in legs:
             extra["subm_f16_dgrad"] = bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops)
         if "wgrad" in legs:
-            extra["subm_f16_wgrad_splitk32"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops)
+            extra["subm_f16_wgrad_balanced_atomic"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops, True)
+            extra["subm_f16_wgrad_serial_splitk32"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops, False)
         if "s8" in legs:
             extra["sparseconv_s8_stride2"] = bench_s8(args, tile_m)
         result["extra"] = extra

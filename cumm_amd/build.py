@@ -27,7 +27,8 @@ def _units():
     for tag, name in ELEMS:
         defs = ["-DCUMM_ELEM=%s" % tag, "-DCUMM_NAME=%s" % name]
         units.append(("rowgemm_" + name, os.path.join(CSRC, "rowgemm_inst.hip"), defs))
-        units.append(("tilegemm_" + name, os.path.join(CSRC, "tilegemm_inst.hip"), defs))
+        extra = ["-DCUMM_NO_WGRAD_ATOMIC"] if tag == "S8" else []   # no s8 backward pass
+        units.append(("tilegemm_" + name, os.path.join(CSRC, "tilegemm_inst.hip"), defs + extra))
     return units
 
 

@@ -112,10 +112,15 @@ int conv_family(const CummHipConvDesc &c) {
   const CummHipGemmDesc &d = c.gemm;
   if (!c.mask_sparse || c.dynamic_mask) return 0;
   if (!same_dtype3(d) || !acc_ok(d)) return 0;
-  if (d.split_k_parallel) return 0;
   const int tm = d.tile_shape[0], tn = d.tile_shape[1], tk = d.tile_shape[2];
   const int mk = d.dtype_a == CUMM_HIP_S8 ? 64 : 32;
   if (tk != mk) return 0;
+  if (d.split_k_parallel) {
+    // only the balanced backward-weight kernel (fp32 atomic partial sums) splits "in parallel"
+    if (c.op_type != CUMM_HIP_OP_BACKWARD_WEIGHT || d.dtype_a == CUMM_HIP_S8 || d.split_k_serial) return 0;
+    if (!d.trans_a || d.trans_b || d.trans_c) return 0;
+    return (tm == 64 && tn == 64) ? 3 : 0;
+  }
   if (c.is_int8_inference && (d.dtype_a != CUMM_HIP_S8 || c.op_type != CUMM_HIP_OP_FORWARD)) return 0;
   if (c.op_type == CUMM_HIP_OP_FORWARD || c.op_type == CUMM_HIP_OP_BACKWARD_INPUT) {
     if (d.split_k_serial) return 0;
@@ -205,6 +210,15 @@ int cumm_hip_list_conv_algos(CummHipConvDesc *out, int cap) {
       fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
       c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
       base(c, CUMM_HIP_OP_BACKWARD_INPUT);
+      v.push_back(c);
+    }
+    {
+      // backward weight, work balanced over live tiles, fp32 atomic partial sums
+      CummHipConvDesc c;
+      fill_gemm_desc(c.gemm, dt, 1, 0, 0, 64, 64, CUMM_HIP_NO_SHUFFLE, 0);
+      c.gemm.split_k_parallel = 1;
+      c.gemm.warp_tile_shape[0] = 32; c.gemm.warp_tile_shape[1] = 32; c.gemm.warp_tile_shape[2] = 32;
+      base(c, CUMM_HIP_OP_BACKWARD_WEIGHT);
       v.push_back(c);
     }
     for (auto &t : sq_tiles) {
@@ -361,7 +375,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
   if (!aligned16(a->ptr_A) || !aligned16(a->ptr_B) || !aligned16(a->ptr_C) || (a->ptr_D && !aligned16(a->ptr_D)))
     return fail(CUMM_HIP_EINVAL, "operand pointers must be 16-byte aligned");
   if (a->C % pv || a->K % pv) return fail(CUMM_HIP_ERUNTIME, "C and K must be multiples of %d for this element type", pv);
-  if (!d.split_k_serial && a->split_k_slices > 1)
+  if (!d.split_k_serial && !d.split_k_parallel && a->split_k_slices > 1)
     return fail(CUMM_HIP_ERUNTIME, "algo don't support splitk but you provide split_k_slices > 1.");
   if (a->N == 0) return CUMM_HIP_OK;
   const void *ptr_D = a->ptr_D ? a->ptr_D : a->ptr_C;
@@ -418,6 +432,32 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
   // backward weight: dW[K, kv, C]; A = dOut [N, K], B = input [*, C]
   const int tm = d.tile_shape[0], tn = d.tile_shape[1], tk = d.tile_shape[2];
   if (a->mask_width <= 0 || a->mask_width % tk) return fail(CUMM_HIP_ERUNTIME, "mask_width must be a positive multiple of tile k");
+  if (fam == 3 && a->split_k_slices > 1 && a->mask_width <= kWgradMaxPos) {
+    const size_t need = sizeof(float) * (size_t)a->K * kv * a->C;
+    if (!a->workspace || a->workspace_bytes < need)
+      return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
+    if (reinterpret_cast<uintptr_t>(a->workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
+    HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
+    WgradParams w;
+    std::memset(&w, 0, sizeof(w));
+    w.dout = a->ptr_A; w.inp = a->ptr_B; w.scratch = reinterpret_cast<float *>(a->workspace);
+    w.argsort = a->mask_argsort_ptr; w.indices = a->indice_ptr; w.red_mask = a->mask_ptr;
+    w.num_red = (a->N + a->mask_width - 1) / a->mask_width; w.mask_width = a->mask_width;
+    w.mask_filter = a->mask_filter;
+    w.n_pos = a->N; w.n_idx = a->N; w.rows_x = a->rows_in; w.rows_y = a->rows_out;
+    w.K = a->K; w.C = a->C; w.kv = kv;
+    int qt = 512 / a->mask_width;
+    if (qt < 1) qt = 1;
+    w.tiles_per_wg = qt;
+    WgradFinalizeParams f;
+    std::memset(&f, 0, sizeof(f));
+    f.scratch = w.scratch; f.dw = a->ptr_C; f.src = ptr_D;
+    f.total = (int64_t)a->K * kv * a->C; f.C = a->C; f.kv = kv; f.mask_filter = a->mask_filter;
+    f.alpha = a->alpha; f.beta = a->beta;
+    hipError_t e = dt == CUMM_HIP_F16 ? launch_wgrad_atomic_f16(w, f, stream) : launch_wgrad_atomic_bf16(w, f, stream);
+    if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
+    return CUMM_HIP_OK;
+  }
   TileGemmParams p;
   std::memset(&p, 0, sizeof(p));
   p.Y = a->ptr_A; p.ldy = a->K;       // dOut rows, m = K
@@ -435,6 +475,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
   p.kv = kv;
   p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act = a->act_type;
   p.split_k = a->split_k_slices < 1 ? 1 : a->split_k_slices;
+  if (fam == 3) p.split_k = 1;   // a single slice needs no partial sums: plain tiled kernel
   p.spin_limit = kSpinLimit;
   const int n_tiles = (a->C + tn - 1) / tn;
   dim3 grid((a->K + tm - 1) / tm, n_tiles * kv, p.split_k);

@@ -24,4 +24,20 @@ hipError_t CUMM_CAT(launch_tilegemm_, CUMM_NAME)(int tm, int tn, bool xk, bool y
   return hipErrorInvalidValue;
 }
 
+#ifndef CUMM_NO_WGRAD_ATOMIC
+hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const WgradFinalizeParams &f,
+                                                     hipStream_t s) {
+  using T = CUMM_ELEM;
+  const int groups = (p.num_red + p.tiles_per_wg - 1) / p.tiles_per_wg;
+  const int kblocks = (p.K + 63) / 64, cblocks = (p.C + 63) / 64;
+  dim3 grid(groups, p.kv * kblocks * cblocks, 1);
+  if (grid.x == 0 || grid.y == 0) return hipSuccess;
+  hipLaunchKernelGGL((wgrad_atomic_kernel<T>), grid, dim3(256), 0, s, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL((wgrad_finalize_kernel<T>), dim3((unsigned)((f.total + 255) / 256)), dim3(256), 0, s, f);
+  return hipGetLastError();
+}
+#endif
+
 }  // namespace cummhip

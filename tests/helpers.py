@@ -48,13 +48,13 @@ def rel_err(got_f32, ref_f32):
     return float(np.max(np.abs(got_f32.astype(np.float64) - ref_f32.astype(np.float64)))) / denom
 
 
-def find_conv_desp(dtype, op, tile_m, tile_n, int8_inference=False):
+def find_conv_desp(dtype, op, tile_m, tile_n, int8_inference=False, split_k_parallel=False):
     for d in ConvMainUnitTest.get_all_conv_algo_desp():
         if (d.dtype_a == TV_DTYPE[dtype] and ConvOpType(d.op_type) == op and
                 d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and
-                d.is_int8_inference == int8_inference):
+                d.is_int8_inference == int8_inference and d.split_k_parallel == split_k_parallel):
             return d
-    raise KeyError((dtype, op, tile_m, tile_n, int8_inference))
+    raise KeyError((dtype, op, tile_m, tile_n, int8_inference, split_k_parallel))
 
 
 def find_gemm_desp(dtype, shuffle, tile_m, tile_n, trans_a, trans_b, trans_c=False):

@@ -174,6 +174,39 @@ def test_backward_weight(dtype, tile, split_k):
     assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(64, 64, 64), (64, 96, 128), (40, 72, 32)])
+@pytest.mark.parametrize("strided", [False, True])
+def test_backward_weight_balanced_atomic(dtype, shape, strided):
+    """The split_k_parallel descriptor: work balanced over live tiles, fp32 atomic partial sums;
+    compared with the oracle's once-rounded float32 sum, for two mask splits with beta."""
+    c_in, k_out, mask_width = shape
+    print("case backward_weight_atomic", dtype, shape, strided, flush=True)
+    rng, coords, pt, feat, w, n_in, n_out = _case(14, 3000, c_in, k_out, dtype, strided=strided)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    red = conv_ref.tile_masks(ms, mask_width)
+    dw0 = H.to_storage(rng.normal(0, 1, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=True)
+    p = ConvParams(3, ConvOpType.BackwardWeight)
+    p.conv_algo_desp = desp
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(dw0, dtype), H.dev(dout, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(red, "u32"), H.dev(order, "i32")
+    p.mask_width = mask_width
+    p.split_k_slices = 4
+    cur = dw0
+    for filt, beta in ((0x3FFF, 0.0), (0x1FFF << 14, 1.0)):
+        p.mask_filter, p.beta, p.alpha = filt, beta, 0.5
+        ConvMainUnitTest.implicit_gemm2(p)
+        cur = conv_ref.implicit_gemm_wgrad_ref(
+            dout, feat, cur, pt.indices_fwd, red, order, mask_width=mask_width, dtype_dout=dtype,
+            dtype_in=dtype, dtype_w=dtype, mask_filter=filt, alpha=0.5, beta=beta,
+            split_k_slices=1)
+    got = H.as_f32(H.host(p.weight), dtype)
+    assert H.rel_err(got, H.as_f32(cur, dtype)) < TOL
+
+
 @pytest.mark.parametrize("tile", [(64, 64), (128, 128), (64, 128)])
 @pytest.mark.parametrize("strided", [False, True])
 def test_int8_inference_bit_exact(tile, strided):
