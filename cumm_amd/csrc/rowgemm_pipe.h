@@ -167,6 +167,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
   int k_of_a[RA][BW];        // offsets whose rows sit in afrag[slot]
   uint64_t any_a[RA][BW][RB];
 
+  int koff1[BW];
   // cursors over the set bits of the tile mask
   uint32_t rem_i = kmask, rem_a = kmask, rem_w = kmask;
   auto take = [&](uint32_t &rem, int (&ko)[BW]) {
@@ -266,7 +267,67 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
     }
   };
 
-  if (kmask != 0) {
+  if (kmask != 0 && __builtin_popcount(kmask) <= BW) {
+    // ---- a tile with a single step (the common case with sorted masks): nothing to pipeline,
+    // so request exactly what is needed, once, and do not pay for the speculative ring fills
+    take(rem_w, koff1);
+#pragma unroll
+    for (int j = 0; j < BW; ++j) {
+      if (koff1[j] < 0) continue;
+      const uint32_t soff = (uint32_t)koff1[j] * w_k_bytes;
+#pragma unroll
+      for (int i = 0; i < GPT; ++i) wreg[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, w_voff[i], soff, 0);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+        idx[0][j][rb] = has_gather ? __builtin_amdgcn_raw_buffer_load_b32(rs_g, key_off[rb], (uint32_t)koff1[j] * g_k_bytes, 0)
+                                   : (int)(key_off[rb] >> 2);
+    }
+#pragma unroll
+    for (int j = 0; j < BW; ++j) {
+      if (koff1[j] < 0) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) any_a[0][j][rb] = 0;
+        continue;
+      }
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const int v = idx[0][j][rb];
+        const bool ok = key_ok[rb] && v >= 0 && v < p.rows_a;
+        any_a[0][j][rb] = __ballot(ok);
+        const uint32_t row = (uint32_t)v * a_row_bytes + a_col;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          const uint32_t keep = 0u - (uint32_t)(ok && a_col_ok[s]);
+          afrag[0][j][rb][s] = __builtin_amdgcn_raw_buffer_load_b128(
+              rs_a, ((row + (uint32_t)(s * 64)) & keep) | (kOob & ~keep), 0, 0);
+        }
+      }
+    }
+    park_w(0, koff1);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < BW; ++j) {
+      if (koff1[j] < 0) continue;
+      uint64_t any_j = 0;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) any_j |= any_a[0][j][rb];
+      if (any_j == 0) continue;
+      const v4i *stage = &lds_w[0][j * SLICE_V];
+      v4i wf[NB][KS];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) wf[nb][s] = stage[(nb * KS + s) * 64 + rd_slot[nb & 3]];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        if (RB > 1 && any_a[0][j][rb] == 0) continue;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int s = 0; s < KS; ++s) acc[rb][nb] = E::mfma(wf[nb][s], afrag[0][j][rb][s], acc[rb][nb]);
+      }
+    }
+  } else if (kmask != 0) {
     // ---- prologue: fill the pipeline
     issue_w();                                   // weights of step 0
 #pragma unroll
