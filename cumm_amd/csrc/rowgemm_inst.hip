@@ -4,6 +4,10 @@
 
 namespace cummhip {
 
+#ifndef CUMM_DW
+#define CUMM_DW 1   // steps of weight slices in flight
+#endif
+
 #define CUMM_CAT_(a, b) a##b
 #define CUMM_CAT(a, b) CUMM_CAT_(a, b)
 
@@ -33,7 +37,7 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   if (p.c_in <= chunk_e) {
     constexpr int BW = step_width(TN, KS);
     constexpr int DA = rows_ahead(RB, KS, BW);
-    hipLaunchKernelGGL((rowgemm_pipe_kernel<T, NW, RB, TN, KS, WT, BW, DA, DA>), grid, dim3(NW * 64), 0, s, p);
+    hipLaunchKernelGGL((rowgemm_pipe_kernel<T, NW, RB, TN, KS, WT, BW, DA, DA, CUMM_DW>), grid, dim3(NW * 64), 0, s, p);
   } else {
     if constexpr (KS == 4) {
       constexpr int B = batch_size(RB, TN, KS);

@@ -39,7 +39,7 @@ __device__ __forceinline__ bool run_unrolled(F &f, std::integer_sequence<int, Is
   return (f(std::integral_constant<int, Is>{}) || ...);
 }
 
-template <class T, int NW, int RB, int TN, int KS, bool WT, int BW, int DA, int DI>
+template <class T, int NW, int RB, int TN, int KS, bool WT, int BW, int DA, int DI, int DW>
 __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmParams p) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
   constexpr int NT = NW * 64;
   constexpr int RA = DA + 1;        // ring of gathered-row register sets
   constexpr int RI = DI + 1;        // ring of pair-table register sets
-  constexpr int UNROLL = ring_lcm(RA, RI);  // after this many steps both rings are back at slot 0
+  constexpr int UNROLL = ring_lcm(ring_lcm(RA, RI), DW);  // all rings are back at slot 0 after this many steps
 
   __shared__ v4i lds_w[2][BW * SLICE_V];
 
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
   // register rings
   int idx[RI][BW][RB];
   v4i afrag[RA][BW][RB][KS];
-  v4i wreg[BW][GPT];
+  v4i wreg[DW][BW][GPT];   // weight slices of steps p .. p + DW - 1
   // per-step scalars travel with the ring slots
   int k_of_a[RA][BW];        // offsets whose rows sit in afrag[slot]
   uint64_t any_a[RA][BW][RB];
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
     }
   };
 
-  auto issue_w = [&]() {
+  auto issue_w = [&](v4i (&wdst)[BW][GPT]) {
     int ko[BW];
     take(rem_w, ko);
 #pragma unroll
@@ -228,18 +228,18 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
       const __amdgpu_buffer_rsrc_t rs = live ? rs_w : rs_none;
       const uint32_t soff = live ? (uint32_t)ko[j] * w_k_bytes : 0u;
 #pragma unroll
-      for (int i = 0; i < GPT; ++i) wreg[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rs, w_voff[i], soff, 0);
+      for (int i = 0; i < GPT; ++i) wdst[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rs, w_voff[i], soff, 0);
     }
   };
 
-  auto park_w = [&](int buf, const int (&kcur)[BW]) {
+  auto park_w = [&](int buf, const int (&kcur)[BW], const v4i (&wsrc)[BW][GPT]) {
 #pragma unroll
     for (int j = 0; j < BW; ++j) {
       v4i *stage = &lds_w[buf][j * SLICE_V];
       if constexpr (!WT) {
 #pragma unroll
         for (int i = 0; i < GPT; ++i)
-          if (tid + i * NT < GRAN) stage[w_slot[i]] = wreg[j][i];
+          if (tid + i * NT < GRAN) stage[w_slot[i]] = wsrc[j][i];
       } else {
         constexpr int NG = TN / PV;
 #pragma unroll
@@ -252,12 +252,12 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
             const int jj = c_local % PV;
             if constexpr (E::kBytes == 2) {
               uint16_t *dst = reinterpret_cast<uint16_t *>(stage);
-              const uint16_t *src = reinterpret_cast<const uint16_t *>(&wreg[j][i]);
+              const uint16_t *src = reinterpret_cast<const uint16_t *>(&wsrc[j][i]);
 #pragma unroll
               for (int x = 0; x < 8; ++x) dst[lds_slot(ng * 8 + x, g) * 8 + jj] = src[x];
             } else {
               uint8_t *dst = reinterpret_cast<uint8_t *>(stage);
-              const uint8_t *src = reinterpret_cast<const uint8_t *>(&wreg[j][i]);
+              const uint8_t *src = reinterpret_cast<const uint8_t *>(&wsrc[j][i]);
 #pragma unroll
               for (int x = 0; x < 16; ++x) dst[lds_slot(ng * 16 + x, g) * 16 + jj] = src[x];
             }
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
       if (koff1[j] < 0) continue;
       const uint32_t soff = (uint32_t)koff1[j] * w_k_bytes;
 #pragma unroll
-      for (int i = 0; i < GPT; ++i) wreg[j][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, w_voff[i], soff, 0);
+      for (int i = 0; i < GPT; ++i) wreg[0][j][i] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, w_voff[i], soff, 0);
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
         idx[0][j][rb] = has_gather ? __builtin_amdgcn_raw_buffer_load_b32(rs_g, key_off[rb], (uint32_t)koff1[j] * g_k_bytes, 0)
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
         }
       }
     }
-    park_w(0, koff1);
+    park_w(0, koff1, wreg[0]);
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < BW; ++j) {
@@ -329,7 +329,8 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
     }
   } else if (kmask != 0) {
     // ---- prologue: fill the pipeline
-    issue_w();                                   // weights of step 0
+#pragma unroll
+    for (int i = 0; i < DW; ++i) issue_w(wreg[i]);    // weights of steps 0 .. DW-1
 #pragma unroll
     for (int i = 0; i < RI; ++i) issue_idx(idx[i]);   // pair-table entries of steps 0 .. DI
     // rows of steps 0 .. DA-1 need entries of steps 0 .. DA-1; the entry ring holds DI+1 steps, so
@@ -349,8 +350,8 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
       int kcur[BW];
 #pragma unroll
       for (int j = 0; j < BW; ++j) kcur[j] = k_of_a[sa][j];
-      park_w(buf, kcur);                 // waits for this step's weights only
-      issue_w();                         // weights of step p + 1
+      park_w(buf, kcur, wreg[u % DW]);   // waits for this step's weights only
+      issue_w(wreg[u % DW]);             // weights of step p + DW, first: they are needed soonest
       issue_a(idx[si], afrag[sn], k_of_a[sn], any_a[sn]);   // rows of step p + DA
       issue_idx(idx[si]);                // entries of step p + DA + DI + 1
       __syncthreads();
