@@ -1,6 +1,7 @@
 // Instantiations of the gather-rows GEMM for one element type (selected with -DCUMM_ELEM=...).
 #include "launch.h"
 #include "rowgemm_pipe.h"
+#include "rowgemm_lds.h"
 
 namespace cummhip {
 
@@ -28,12 +29,29 @@ constexpr int rows_ahead(int RB, int KS, int BW) {
   return d;
 }
 
+// ring stages of the LDS-streaming kernel: three where they fit 64 KB, else two, else none
+constexpr int lds_stages(int TM, int TN, int KS) {
+  const int stage = (TM + TN) * KS * 64;
+#ifdef CUMM_LDS_NS
+  if (CUMM_LDS_NS * stage <= 65536) return CUMM_LDS_NS;
+#endif
+  return 3 * stage <= 65536 ? 3 : (2 * stage <= 65536 ? 2 : 0);
+}
+
 template <class T, int NW, int RB, int TN, int KS, bool WT>
 static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   constexpr int TM = NW * RB * 16;
   dim3 grid((p.n_pos + TM - 1) / TM, (p.k_out + TN - 1) / TN, 1);
   if (grid.x == 0 || grid.y == 0) return hipSuccess;
   constexpr int chunk_e = 4 * KS * Elem<T>::kPerVec;
+  constexpr int NS = lds_stages(TM, TN, KS);
+  if constexpr (!WT && NS > 0) {
+    if (p.c_in <= chunk_e && p.w_stride_c == 1) {
+      // 2 x 2 waves, each TM/2 rows by TN/2 channels
+      hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS>), grid, dim3(256), 0, s, p);
+      return hipGetLastError();
+    }
+  }
   if (p.c_in <= chunk_e) {
     constexpr int BW = step_width(TN, KS);
     constexpr int DA = rows_ahead(RB, KS, BW);

@@ -1,0 +1,423 @@
+// Gather-rows GEMM that streams both operands through LDS with direct-to-LDS buffer loads, for
+// contractions that fit one channel chunk (see rowgemm.h for the problem statement).
+//
+// Why: in the register-gather kernels a lane loads the 16 bytes its MFMA operand slot needs, so
+// neighbouring lanes read different rows and every load instruction is 64 separate 16-byte
+// requests; and the step body spends most of its issue slots on addressing, descriptor selection
+// and LDS staging of the weights.  Here
+//   * a load instruction moves whole rows: 4*KS neighbouring lanes read one row's KS*64 bytes
+//     (one request per 64-byte segment), and the data lands in LDS without passing registers
+//     (buffer_load ... lds writes lane l of the instruction at M0 + 16*l);
+//   * the LDS image of a tile is row-major with the 16-byte chunks of a row XOR-permuted by
+//     swz(row) = (row*KS/4) mod 4*KS.  The permutation is applied on the global side (a lane picks
+//     which chunk of its row it fetches), which keeps the global access coalesced, and makes the
+//     MFMA-layout reads (16 lanes = 16 rows, same chunk) hit 16 different bank groups;
+//   * the weight tile is stored in the row order the MFMA fragments want (LDS row wn*NBW*16 +
+//     nb*16 + i holds output channel wn*NBW*16 + (i/4)*4*NBW + nb*4 + i%4), so that a lane's
+//     accumulators are 4*NBW consecutive channels of one output row (vector stores, no atomics);
+//   * waves form a WM x WN grid over the tile; each wave reads RBW row fragments and NBW weight
+//     fragments per 16-byte k-step from LDS, i.e. (WM*TN + WN*TM)*KS*64 bytes per offset instead
+//     of NW*TN*KS*64;
+//   * NS stages of (rows + weights) form a ring; one barrier per kernel offset.  Step i waits for
+//     its own loads of offset i, passes the barrier (now everybody's loads of offset i have landed
+//     and everybody has finished computing offset i-1), issues the loads of offset i+NS-1 into the
+//     stage that offset i-1 used, then computes.  Pair-table entries run NS steps ahead of the row
+//     loads that need them.  A kernel offset past the end of the tile's list is loaded through a
+//     descriptor with zero records (no memory traffic, zeros into LDS), which keeps the number of
+//     outstanding loads the same on every path: the waits below count instructions.
+//   * every stage is its own __shared__ array: the compiler then knows which direct-to-LDS loads
+//     an LDS read can depend on and does not wait for the younger ones.
+#pragma once
+#include <type_traits>
+#include <utility>
+
+#include "rowgemm.h"
+
+namespace cummhip {
+
+#define CUMM_LDS_PTR(x) ((__attribute__((address_space(3))) void *)(x))
+
+// s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt = simm16[15:14,3:0])
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// OR over the 64 lanes of a wave with row shifts and row broadcasts (no LDS round trips)
+__device__ __forceinline__ uint32_t wave_or_dpp(uint32_t v) {
+  int t = (int)v;
+  t |= __builtin_amdgcn_update_dpp(0, t, 0x111, 0xf, 0xf, true);   // row_shr:1
+  t |= __builtin_amdgcn_update_dpp(0, t, 0x112, 0xf, 0xf, true);   // row_shr:2
+  t |= __builtin_amdgcn_update_dpp(0, t, 0x114, 0xf, 0xf, true);   // row_shr:4
+  t |= __builtin_amdgcn_update_dpp(0, t, 0x118, 0xf, 0xf, true);   // row_shr:8 -> lane 15 of a row
+  t |= __builtin_amdgcn_update_dpp(0, t, 0x142, 0xa, 0xf, true);   // row_bcast:15 into rows 1, 3
+  t |= __builtin_amdgcn_update_dpp(0, t, 0x143, 0xc, 0xf, true);   // row_bcast:31 into rows 2, 3
+  return (uint32_t)__builtin_amdgcn_readlane(t, 63);
+}
+
+// Direct-to-LDS buffer loads, written as asm so that the compiler's wait-count pass does not see
+// them: it guards LDS reads that may alias an outstanding direct-to-LDS load with waits of its
+// own, and at a loop header it assumes the worst (waits for all of them), which would drain the
+// ring once per trip.  Every wait for these loads is placed by hand (wait_vmcnt).  Hidden loads
+// cannot make a wait of the compiler too weak: loads complete in order, so more outstanding loads
+// than it counted only make its waits stricter than needed.
+// rsrc: buffer descriptor words; lds: byte address of the destination of lane 0 (lane l lands at
+// lds + l*size); voff: per-lane byte offset; soff: wave-uniform byte offset.
+__device__ __forceinline__ v4i rsrc_words(const void *ptr, uint32_t bytes) {
+  const uint64_t a = (uint64_t)ptr;
+  return v4i{(int)(uint32_t)a, (int)((uint32_t)(a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+}
+template <class P>
+__device__ __forceinline__ uint32_t lds_addr(P *ptr) {
+  return (uint32_t)(uintptr_t)CUMM_LDS_PTR(ptr);
+}
+__device__ __forceinline__ void dma_b128(v4i rsrc, uint32_t lds, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+}
+__device__ __forceinline__ void dma_b32(v4i rsrc, uint32_t lds, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :: "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
+}
+
+// Workgroup barrier without the fence of __syncthreads(): the fence would wait for every
+// outstanding direct-to-LDS load, i.e. also for the stages that are being prefetched.  The empty
+// asm statements keep the compiler from moving LDS accesses across the barrier; the caller waits
+// for the loads that the other waves are going to read before calling this.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <class F, int... Is>
+__device__ __forceinline__ bool run_steps(F &f, std::integer_sequence<int, Is...>) {
+  return (f(std::integral_constant<int, Is>{}) || ...);
+}
+
+// T: element tag; WM x WN: wave grid; RBW: 16-row blocks per wave; NBW: 16-channel blocks per
+// wave; KS: 64-byte pieces per row (contraction <= KS*64 bytes); NS: ring stages.
+// Weights must be contiguous along the contraction (w_stride_c == 1).
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS>
+__global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmParams p) {
+  using E = Elem<T>;
+  using AccV = typename E::AccV;
+  constexpr int NW = WM * WN;
+  constexpr int NT = NW * 64;
+  constexpr int TM = WM * RBW * 16;
+  constexpr int TN = WN * NBW * 16;
+  constexpr int PV = E::kPerVec;
+  constexpr int LPR = 4 * KS;              // lanes (16-byte chunks) per row
+  constexpr int RPI = 64 / LPR;            // rows per load instruction
+  constexpr int IPA = TM * LPR / NT;       // row-load instructions per wave and offset
+  constexpr int IPW = TN * LPR / NT;       // weight-load instructions per wave and offset
+  static_assert(IPA >= 1 && IPW >= 1, "tile too small for the workgroup");
+  constexpr int A_V = TM * LPR;            // 16-byte vectors of the row part of a stage
+  constexpr int STAGE_V = (TM + TN) * LPR;
+  constexpr int L = NS - 1;                // steps the operand loads run ahead
+  constexpr int DI = NS;                   // steps the pair-table loads run ahead of the row loads
+  constexpr int RPW = TM / NW;             // rows whose entries a wave fetches (one instruction)
+  static_assert(RPW <= 64, "one entry instruction per wave");
+  constexpr int PER_STEP = IPA + IPW + 1;  // load instructions a wave issues per step
+  // loads issued after those of offset i when step i starts: the entries issued with them, then
+  // L-1 whole steps
+  constexpr int WAIT_OPERANDS = 1 + (L - 1) * PER_STEP;
+  static_assert(WAIT_OPERANDS < 64, "too many loads in flight for the counter");
+
+  __shared__ v4i st0[STAGE_V];
+  __shared__ v4i st1[STAGE_V];
+  __shared__ v4i st2[NS > 2 ? STAGE_V : 1];
+  __shared__ v4i st3[NS > 3 ? STAGE_V : 1];
+  // pair-table entries also travel global -> LDS directly: every vector load of the step loop is
+  // then counted by hand, none returns into a register the compiler would guard with waits of
+  // its own.  Slot [d][wave][l] is written by lane l of the wave (lanes >= RPW write zeros).
+  // (one array per slot, like the stages)
+  __shared__ int ix0[NW][64];
+  __shared__ int ix1[NW][64];
+  __shared__ int ix2[NS > 2 ? NW : 1][64];
+  __shared__ int ix3[NS > 3 ? NW : 1][64];
+  auto stage = [&](auto sc) -> v4i * {
+    constexpr int s = decltype(sc)::value;
+    if constexpr (s == 0) return st0;
+    else if constexpr (s == 1) return st1;
+    else if constexpr (s == 2) return st2;
+    else return st3;
+  };
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int m = lane & 15;
+  const int q = lane >> 4;
+  auto idx_slot = [&](auto sc) -> int * {
+    constexpr int s = decltype(sc)::value;
+    if constexpr (s == 0) return ix0[wave];
+    else if constexpr (s == 1) return ix1[wave];
+    else if constexpr (s == 2) return ix2[wave];
+    else return ix3[wave];
+  };
+
+  const int tile = (int)gridDim.x - 1 - (int)blockIdx.x;  // heaviest tiles first (masks sorted ascending)
+  const int n0 = blockIdx.y * TN;
+  const int pos_base = tile * TM;
+
+  // ---- tile mask: OR over the tile's positions (cumm/conv/kernel.py:844-889 of the reference)
+  uint32_t kmask;
+  if (p.mask != nullptr) {
+    uint32_t mk = 0;
+#pragma unroll
+    for (int i = 0; i < (TM + 63) / 64; ++i) {
+      const int pp = pos_base + i * 64 + lane;
+      if (i * 64 + lane < TM && pp < p.n_pos) mk |= p.mask[pp];
+    }
+    kmask = wave_or_dpp(mk) & p.mask_filter;
+    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
+    if (p.exit_on_empty && kmask == 0) return;
+    if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
+    if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
+  } else {
+    kmask = 1u;
+  }
+  const int n_steps = __builtin_popcount(kmask);
+
+  // ---- loader role of this lane: rows of the tile it fetches, weight rows it fetches
+  const int lrow = lane / LPR;             // row inside a load instruction
+  const int lchunk = lane % LPR;           // LDS chunk slot inside the row
+  auto swz = [](int row) { return ((row * KS) >> 2) & (LPR - 1); };
+  const bool has_gather = p.gather != nullptr;
+  // entries: lane l < RPW fetches the entry of tile row wave*RPW + l
+  uint32_t key_off = kOob;
+  {
+    const int pos = pos_base + wave * RPW + lane;
+    int key = -1;
+    if (lane < RPW && pos < p.n_pos) key = p.gather_by_pos ? pos : (p.out_rows ? p.out_rows[pos] : pos);
+    if (key >= 0 && key < p.n_idx) key_off = (uint32_t)key * 4u;
+  }
+  int a_key[IPA];          // without a pair table the gathered row is the key itself
+  uint32_t a_col[IPA];     // byte offset of the fetched chunk inside the gathered row, or kOob
+#pragma unroll
+  for (int t = 0; t < IPA; ++t) {
+    const int r = (wave * IPA + t) * RPI + lrow;
+    const int pos = pos_base + r;
+    int key = -1;
+    if (pos < p.n_pos) key = p.gather_by_pos ? pos : (p.out_rows ? p.out_rows[pos] : pos);
+    a_key[t] = key >= 0 && key < p.n_idx ? key : -1;
+    const int c = lchunk ^ swz(r);
+    a_col[t] = a_key[t] >= 0 && c * PV < p.c_in ? (uint32_t)c * 16u : kOob;
+  }
+  uint32_t w_voff[IPW];
+#pragma unroll
+  for (int t = 0; t < IPW; ++t) {
+    const int rho = (wave * IPW + t) * RPI + lrow;      // LDS row, fragment order
+    const int i = rho & 15, nb = (rho >> 4) % NBW, wq = rho / (16 * NBW);
+    const int n = n0 + wq * (16 * NBW) + (i >> 2) * (4 * NBW) + nb * 4 + (i & 3);
+    const int c = lchunk ^ swz(rho);
+    w_voff[t] = n < p.k_out && c * PV < p.c_in
+                    ? (uint32_t)((int64_t)n * p.w_stride_n * E::kBytes) + (uint32_t)c * 16u
+                    : kOob;
+  }
+
+  // ---- reader role: fragment slots (16-byte units) relative to the wave's first row
+  int a_rd[KS], w_rd[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const int slot = m * LPR + ((s * 4 + q) ^ swz(m));
+    a_rd[s] = wm * (RBW * 16) * LPR + slot;
+    w_rd[s] = A_V + wn * (NBW * 16) * LPR + slot;
+  }
+
+  // ---- output rows of this lane
+  int out_row[RBW];
+#pragma unroll
+  for (int rb = 0; rb < RBW; ++rb) {
+    const int pos = pos_base + (wm * RBW + rb) * 16 + m;
+    int o = -1;
+    if (pos < p.n_pos) o = p.out_rows ? p.out_rows[pos] : pos;
+    out_row[rb] = o;
+  }
+
+  AccV acc[RBW][NBW];
+#pragma unroll
+  for (int rb = 0; rb < RBW; ++rb)
+#pragma unroll
+    for (int nb = 0; nb < NBW; ++nb) acc[rb][nb] = AccV{0, 0, 0, 0};
+
+  const uint32_t a_row_bytes = (uint32_t)p.lda * E::kBytes;
+  const uint32_t w_k_bytes = (uint32_t)p.w_stride_k * E::kBytes;
+  const uint32_t g_k_bytes = (uint32_t)p.n_idx * 4u;
+  const uint32_t g_bytes = has_gather ? p.gather_bytes : 0u;
+
+  // lane j of klist holds the j-th kernel offset of the tile (-1 past the end): lane b pushes
+  // b+1 to the lane of its rank among the set bits, lanes without a bit push into lane 63, which
+  // nobody reads; a lane nobody pushed to reads 0.
+  int klist;
+  {
+    const bool bit = lane < 32 && ((kmask >> lane) & 1u);
+    const int rank = __builtin_popcount(kmask & ((1u << (lane & 31)) - 1u));
+    klist = __builtin_amdgcn_ds_permute(bit ? rank * 4 : 63 * 4, bit ? lane + 1 : 0) - 1;
+  }
+
+  auto issue_idx = [&](int j, int *slot) {
+    const int k = __builtin_amdgcn_readlane(klist, j);
+    const v4i rs = rsrc_words(p.gather, k >= 0 ? g_bytes : 0u);
+    dma_b32(rs, lds_addr(slot), key_off, (uint32_t)k * g_k_bytes);
+  };
+  // entries of this lane's rows out of the wave's slot (its own loads: no barrier needed)
+  auto read_idx = [&](const int *slot, int (&dst)[IPA]) {
+#pragma unroll
+    for (int t = 0; t < IPA; ++t) dst[t] = has_gather ? slot[t * RPI + lrow] : a_key[t];
+  };
+  auto issue_operands = [&](int j, const int (&src)[IPA], v4i *st) {
+    const int k = __builtin_amdgcn_readlane(klist, j);
+    const v4i rs_a = rsrc_words(p.A, k >= 0 ? p.a_bytes : 0u);
+    const v4i rs_w = rsrc_words(p.W, k >= 0 ? p.w_bytes : 0u);
+#pragma unroll
+    for (int t = 0; t < IPA; ++t) {
+      // a_col is out of range already for a row without a key or a chunk past the contraction;
+      // adding a row offset below 2 GiB keeps it out of range
+      const uint32_t v = (uint32_t)src[t];
+      const uint32_t voff = v < (uint32_t)p.rows_a ? v * a_row_bytes + a_col[t] : kOob;
+      dma_b128(rs_a, lds_addr(st + (wave * IPA + t) * 64), voff, 0u);
+    }
+    const uint32_t soff = (uint32_t)k * w_k_bytes;   // k = -1 comes with zero records
+#pragma unroll
+    for (int t = 0; t < IPW; ++t)
+      dma_b128(rs_w, lds_addr(st + A_V + (wave * IPW + t) * 64), w_voff[t], soff);
+  };
+
+  if (n_steps > 0) {
+    // ---- prologue: entries of offsets 0 .. DI-1, then operands of offsets 0 .. L-1, each
+    // followed by the next entries (the order of a step, so the waits count the same everywhere)
+    auto first = [&](auto jc) -> bool {
+      issue_idx(decltype(jc)::value, idx_slot(jc));
+      return false;
+    };
+    run_steps(first, std::make_integer_sequence<int, DI>{});
+    auto fill = [&](auto jc) -> bool {
+      constexpr int j = decltype(jc)::value;
+      wait_vmcnt<DI - 1 + j * (PER_STEP - 1)>();   // entries of offset j have landed
+      int v[IPA];
+      read_idx(idx_slot(std::integral_constant<int, j % DI>{}), v);
+      issue_operands(j, v, stage(std::integral_constant<int, j % NS>{}));
+      issue_idx(j + DI, idx_slot(std::integral_constant<int, j % DI>{}));
+      return false;
+    };
+    run_steps(fill, std::make_integer_sequence<int, L>{});
+
+    int done = 0;
+    auto step = [&](auto uc) -> bool {
+      constexpr int u = decltype(uc)::value;      // step number modulo the ring lengths
+      constexpr int sc = u % NS;                  // stage computed in this step
+      constexpr int sl = (u + L) % NS;            // stage loaded for offset i + L
+      constexpr int si = (u + L) % DI;            // entries of offset i + L, then refilled
+      wait_vmcnt<WAIT_OPERANDS>();                // own loads of offset i (and all older ones)
+      int v[IPA];
+      read_idx(idx_slot(std::integral_constant<int, si>{}), v);   // the barrier hides the LDS round trip
+      lds_barrier();
+      // fragment reads first: their LDS round trip overlaps the address work of the loads below
+      const v4i *st = stage(std::integral_constant<int, sc>{});
+      v4i af[RBW][KS], wf[NBW][KS];
+#pragma unroll
+      for (int nb = 0; nb < NBW; ++nb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) wf[nb][s] = st[w_rd[s] + nb * 16 * LPR];
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) af[rb][s] = st[a_rd[s] + rb * 16 * LPR];
+      issue_operands(done + L, v, stage(std::integral_constant<int, sl>{}));
+      issue_idx(done + L + DI, idx_slot(std::integral_constant<int, si>{}));
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb)
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb)
+#pragma unroll
+          for (int s = 0; s < KS; ++s) acc[rb][nb] = E::mfma(wf[nb][s], af[rb][s], acc[rb][nb]);
+      return ++done >= n_steps;
+    };
+    constexpr int UNROLL = NS;   // DI == NS: both rings are back at slot 0
+    while (!run_steps(step, std::make_integer_sequence<int, UNROLL>{})) {
+    }
+  }
+
+  wait_vmcnt<0>();   // the loads past the end of the offset list still target this workgroup's LDS
+  // ---- epilogue: lane (q, m) holds, for each of its rows, channels ch0 .. ch0 + 4*NBW - 1
+  constexpr int CPLW = 4 * NBW;
+  const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.c_bytes);
+  const __amdgpu_buffer_rsrc_t rs_d = make_rsrc(p.D, p.read_source ? p.d_bytes : 0u);
+  const int ch0 = n0 + wn * (NBW * 16) + q * CPLW;
+  if constexpr (E::kBytes == 2) {
+    constexpr int NG = CPLW / 8;   // 16-byte groups
+    static_assert(CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
+#pragma unroll
+    for (int rb = 0; rb < RBW; ++rb) {
+      const int o = out_row[rb];
+      const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int ch = ch0 + g * 8;
+        const bool ok = row_ok && ch < p.k_out;
+        const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
+        v4i src = {0, 0, 0, 0};
+        if (p.read_source) {
+          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 2u : kOob;
+          src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
+        }
+        const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
+        v4i outv;
+        uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          const float a = acc[rb][g * 2 + (x >> 2)][x & 3];
+          float t = p.read_source ? __builtin_fmaf(p.alpha, a, p.beta * E::to_float(sh[x])) : p.alpha * a;
+          t = apply_act(t, p.act, p.act_alpha);
+          oh[x] = E::from_float(t);
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
+      }
+    }
+  } else {
+    // one-byte outputs: 4*NBW bytes per lane and row, moved as dwords
+    constexpr int ND = CPLW / 4;
+#pragma unroll
+    for (int rb = 0; rb < RBW; ++rb) {
+      const int o = out_row[rb];
+      const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+      for (int g = 0; g < ND; ++g) {
+        const int ch = ch0 + g * 4;
+        const bool ok = row_ok && ch < p.k_out;
+        const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) : kOob;
+        int src = 0;
+        if (p.read_source) {
+          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) : kOob;
+          src = __builtin_amdgcn_raw_buffer_load_b32(rs_d, doff, 0, 0);
+        }
+        const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
+        int outv;
+        int8_t *ob = reinterpret_cast<int8_t *>(&outv);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const int a = acc[rb][g][x];
+          float t;
+          if (p.int8_epilogue) {
+            const int c = ch + x < p.k_out ? ch + x : 0;
+            t = __builtin_fmaf(p.scale[c], (float)a, p.bias[c]);
+            if (p.read_source) t = __builtin_fmaf(p.beta, (float)sb[x], t);
+          } else if (p.read_source) {
+            t = __builtin_fmaf(p.alpha, (float)a, p.beta * (float)sb[x]);
+          } else {
+            t = p.alpha * (float)a;
+          }
+          t = apply_act(t, p.act, p.act_alpha);
+          ob[x] = (int8_t)f32_to_s8(t);
+        }
+        __builtin_amdgcn_raw_buffer_store_b32(outv, rs_c, coff, 0, 0);
+      }
+    }
+  }
+}
+
+}  // namespace cummhip
