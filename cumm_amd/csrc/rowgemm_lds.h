@@ -163,24 +163,16 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   const int n0 = blockIdx.y * TN;
   const int pos_base = tile * TM;
 
-  // ---- tile mask: OR over the tile's positions (cumm/conv/kernel.py:844-889 of the reference)
-  uint32_t kmask;
+  // ---- the tile's mask words are requested first and reduced only after the row keys below have
+  // been requested too: one memory round trip for both
+  uint32_t mk = 0;
   if (p.mask != nullptr) {
-    uint32_t mk = 0;
 #pragma unroll
     for (int i = 0; i < (TM + 63) / 64; ++i) {
       const int pp = pos_base + i * 64 + lane;
       if (i * 64 + lane < TM && pp < p.n_pos) mk |= p.mask[pp];
     }
-    kmask = wave_or_dpp(mk) & p.mask_filter;
-    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
-    if (p.exit_on_empty && kmask == 0) return;
-    if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
-    if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
-  } else {
-    kmask = 1u;
   }
-  const int n_steps = __builtin_popcount(kmask);
 
   // ---- loader role of this lane: rows of the tile it fetches, weight rows it fetches
   const int lrow = lane / LPR;             // row inside a load instruction
@@ -237,6 +229,17 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     if (pos < p.n_pos) o = p.out_rows ? p.out_rows[pos] : pos;
     out_row[rb] = o;
   }
+
+  // ---- tile mask: OR over the tile's positions (cumm/conv/kernel.py:844-889 of the reference)
+  uint32_t kmask = 1u;
+  if (p.mask != nullptr) {
+    kmask = wave_or_dpp(mk) & p.mask_filter;
+    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
+    if (p.exit_on_empty && kmask == 0) return;
+    if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
+    if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
+  }
+  const int n_steps = __builtin_popcount(kmask);
 
   AccV acc[RBW][NBW];
 #pragma unroll
@@ -343,80 +346,103 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   }
 
   wait_vmcnt<0>();   // the loads past the end of the offset list still target this workgroup's LDS
-  // ---- epilogue: lane (q, m) holds, for each of its rows, channels ch0 .. ch0 + 4*NBW - 1
+  // ---- epilogue: lane (q, m) holds, for each of its rows, channels ch0 .. ch0 + 4*NBW - 1.
+  // The activation and the blend mode are lifted out of the element loops (one straight-line
+  // copy per combination): tested per element they cost more issue slots than the arithmetic.
   constexpr int CPLW = 4 * NBW;
   const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.c_bytes);
   const __amdgpu_buffer_rsrc_t rs_d = make_rsrc(p.D, p.read_source ? p.d_bytes : 0u);
   const int ch0 = n0 + wn * (NBW * 16) + q * CPLW;
-  if constexpr (E::kBytes == 2) {
-    constexpr int NG = CPLW / 8;   // 16-byte groups
-    static_assert(CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
+  // MODE: 0 = alpha*acc, 1 = alpha*acc + beta*src, 2 = scale*acc + bias, 3 = ... + beta*src
+  auto store_rows = [&](auto act_c, auto mode_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    constexpr int MODE = decltype(mode_c)::value;
+    constexpr bool SRC = (MODE & 1) != 0;
+    if constexpr (E::kBytes == 2) {
+      constexpr int NG = CPLW / 8;   // 16-byte groups
+      static_assert(CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
 #pragma unroll
-    for (int rb = 0; rb < RBW; ++rb) {
-      const int o = out_row[rb];
-      const bool row_ok = o >= 0 && o < p.rows_c;
+      for (int rb = 0; rb < RBW; ++rb) {
+        const int o = out_row[rb];
+        const bool row_ok = o >= 0 && o < p.rows_c;
 #pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        const int ch = ch0 + g * 8;
-        const bool ok = row_ok && ch < p.k_out;
-        const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
-        v4i src = {0, 0, 0, 0};
-        if (p.read_source) {
-          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 2u : kOob;
-          src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
-        }
-        const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
-        v4i outv;
-        uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
-#pragma unroll
-        for (int x = 0; x < 8; ++x) {
-          const float a = acc[rb][g * 2 + (x >> 2)][x & 3];
-          float t = p.read_source ? __builtin_fmaf(p.alpha, a, p.beta * E::to_float(sh[x])) : p.alpha * a;
-          t = apply_act(t, p.act, p.act_alpha);
-          oh[x] = E::from_float(t);
-        }
-        __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
-      }
-    }
-  } else {
-    // one-byte outputs: 4*NBW bytes per lane and row, moved as dwords
-    constexpr int ND = CPLW / 4;
-#pragma unroll
-    for (int rb = 0; rb < RBW; ++rb) {
-      const int o = out_row[rb];
-      const bool row_ok = o >= 0 && o < p.rows_c;
-#pragma unroll
-      for (int g = 0; g < ND; ++g) {
-        const int ch = ch0 + g * 4;
-        const bool ok = row_ok && ch < p.k_out;
-        const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) : kOob;
-        int src = 0;
-        if (p.read_source) {
-          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) : kOob;
-          src = __builtin_amdgcn_raw_buffer_load_b32(rs_d, doff, 0, 0);
-        }
-        const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
-        int outv;
-        int8_t *ob = reinterpret_cast<int8_t *>(&outv);
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-          const int a = acc[rb][g][x];
-          float t;
-          if (p.int8_epilogue) {
-            const int c = ch + x < p.k_out ? ch + x : 0;
-            t = __builtin_fmaf(p.scale[c], (float)a, p.bias[c]);
-            if (p.read_source) t = __builtin_fmaf(p.beta, (float)sb[x], t);
-          } else if (p.read_source) {
-            t = __builtin_fmaf(p.alpha, (float)a, p.beta * (float)sb[x]);
-          } else {
-            t = p.alpha * (float)a;
+        for (int g = 0; g < NG; ++g) {
+          const int ch = ch0 + g * 8;
+          const bool ok = row_ok && ch < p.k_out;
+          const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
+          v4i src = {0, 0, 0, 0};
+          if constexpr (SRC) {
+            const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 2u : kOob;
+            src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
           }
-          t = apply_act(t, p.act, p.act_alpha);
-          ob[x] = (int8_t)f32_to_s8(t);
+          const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
+          v4i outv;
+          uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
+#pragma unroll
+          for (int x = 0; x < 8; ++x) {
+            const float a = acc[rb][g * 2 + (x >> 2)][x & 3];
+            float t = SRC ? __builtin_fmaf(p.alpha, a, p.beta * E::to_float(sh[x])) : p.alpha * a;
+            t = apply_act(t, ACT, p.act_alpha);
+            oh[x] = E::from_float(t);
+          }
+          __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
         }
-        __builtin_amdgcn_raw_buffer_store_b32(outv, rs_c, coff, 0, 0);
+      }
+    } else {
+      // one-byte outputs: 4*NBW bytes per lane and row, moved as dwords
+      constexpr int ND = CPLW / 4;
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb) {
+        const int o = out_row[rb];
+        const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+        for (int g = 0; g < ND; ++g) {
+          const int ch = ch0 + g * 4;
+          const bool ok = row_ok && ch < p.k_out;
+          const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) : kOob;
+          int src = 0;
+          if constexpr (SRC) {
+            const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) : kOob;
+            src = __builtin_amdgcn_raw_buffer_load_b32(rs_d, doff, 0, 0);
+          }
+          const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
+          int outv;
+          int8_t *ob = reinterpret_cast<int8_t *>(&outv);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            const int a = acc[rb][g][x];
+            float t;
+            if constexpr (MODE >= 2) {
+              const int c = ch + x < p.k_out ? ch + x : 0;
+              t = __builtin_fmaf(p.scale[c], (float)a, p.bias[c]);
+              if constexpr (SRC) t = __builtin_fmaf(p.beta, (float)sb[x], t);
+            } else if constexpr (SRC) {
+              t = __builtin_fmaf(p.alpha, (float)a, p.beta * (float)sb[x]);
+            } else {
+              t = p.alpha * (float)a;
+            }
+            t = apply_act(t, ACT, p.act_alpha);
+            ob[x] = (int8_t)f32_to_s8(t);
+          }
+          __builtin_amdgcn_raw_buffer_store_b32(outv, rs_c, coff, 0, 0);
+        }
       }
     }
+  };
+  auto with_mode = [&](auto act_c) {
+    const int mode = (p.read_source ? 1 : 0) | (E::kBytes == 1 && p.int8_epilogue ? 2 : 0);
+    switch (mode) {
+    case 0: store_rows(act_c, std::integral_constant<int, 0>{}); break;
+    case 1: store_rows(act_c, std::integral_constant<int, 1>{}); break;
+    case 2: if constexpr (E::kBytes == 1) store_rows(act_c, std::integral_constant<int, 2>{}); break;
+    default: if constexpr (E::kBytes == 1) store_rows(act_c, std::integral_constant<int, 3>{}); break;
+    }
+  };
+  switch (p.act) {
+  case 1: with_mode(std::integral_constant<int, 1>{}); break;
+  case 2: with_mode(std::integral_constant<int, 2>{}); break;
+  case 3: with_mode(std::integral_constant<int, 3>{}); break;
+  default: with_mode(std::integral_constant<int, 0>{}); break;
   }
 }
 
