@@ -45,10 +45,10 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   if (grid.x == 0 || grid.y == 0) return hipSuccess;
   constexpr int chunk_e = 4 * KS * Elem<T>::kPerVec;
   constexpr int NS = lds_stages(TM, TN, KS);
-  if constexpr (!WT && NS > 0) {
-    if (p.c_in <= chunk_e && p.w_stride_c == 1) {
-      // 2 x 2 waves, each TM/2 rows by TN/2 channels
-      hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS>), grid, dim3(256), 0, s, p);
+  if constexpr (NS > 0 && (!WT || Elem<T>::kBytes == 2)) {
+    // the LDS-streaming kernel: 2 x 2 waves, each TM/2 rows by TN/2 channels
+    if (p.c_in <= chunk_e && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
+      hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS, WT>), grid, dim3(256), 0, s, p);
       return hipGetLastError();
     }
   }

@@ -98,8 +98,15 @@ __device__ __forceinline__ bool run_steps(F &f, std::integer_sequence<int, Is...
 
 // T: element tag; WM x WN: wave grid; RBW: 16-row blocks per wave; NBW: 16-channel blocks per
 // wave; KS: 64-byte pieces per row (contraction <= KS*64 bytes); NS: ring stages.
-// Weights must be contiguous along the contraction (w_stride_c == 1).
-template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS>
+// WT false: weights are contiguous along the contraction (w_stride_c == 1).
+// WT true (two-byte elements): weights are contiguous along the output channel (w_stride_n == 1).
+// The weight tile then sits in LDS as [contraction][channel] rows, again with XOR-permuted
+// 16-byte chunks, and the MFMA operand is fetched with the transposing LDS read: within a group
+// of 16 lanes, ds_read_b64_tr_b16 hands lane i, element j the 16-bit element i%4 of the 8 bytes
+// that lane i/4 + 4j points to.  Lane s of a group points to row (first k) + s/4, channels
+// 4*(s%4) .. +3 of its 16-channel block, so lane i receives 4 consecutive k of channel i; two
+// reads make one operand.  A lane then owns channels nb*16 + 4q .. +3 of each block nb.
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT = false>
 __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmParams p) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
@@ -112,6 +119,12 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   constexpr int RPI = 64 / LPR;            // rows per load instruction
   constexpr int IPA = TM * LPR / NT;       // row-load instructions per wave and offset
   constexpr int IPW = TN * LPR / NT;       // weight-load instructions per wave and offset
+  // transposed weight tile: KS*64/kBytes rows of TN elements
+  constexpr int WROWS = KS * 64 / E::kBytes;         // contraction rows
+  constexpr int LPRW = TN * E::kBytes / 16;          // lanes (16-byte chunks) per row
+  constexpr int RPIW = 64 / LPRW;                    // rows per load instruction
+  static_assert(!WT || E::kBytes == 2, "the transposing read used here moves 16-bit elements");
+  static_assert(!WT || WROWS * LPRW == TN * LPR, "both weight layouts fill the same LDS bytes");
   static_assert(IPA >= 1 && IPW >= 1, "tile too small for the workgroup");
   constexpr int A_V = TM * LPR;            // 16-byte vectors of the row part of a stage
   constexpr int STAGE_V = (TM + TN) * LPR;
@@ -200,15 +213,25 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     a_col[t] = a_key[t] >= 0 && c * PV < p.c_in ? (uint32_t)c * 16u : kOob;
   }
   uint32_t w_voff[IPW];
+  auto swz_w = [](int e) { return 2 * (((e * LPRW) >> 4) & (LPRW / 2 - 1)); };   // WT: even chunk XOR
 #pragma unroll
   for (int t = 0; t < IPW; ++t) {
-    const int rho = (wave * IPW + t) * RPI + lrow;      // LDS row, fragment order
-    const int i = rho & 15, nb = (rho >> 4) % NBW, wq = rho / (16 * NBW);
-    const int n = n0 + wq * (16 * NBW) + (i >> 2) * (4 * NBW) + nb * 4 + (i & 3);
-    const int c = lchunk ^ swz(rho);
-    w_voff[t] = n < p.k_out && c * PV < p.c_in
-                    ? (uint32_t)((int64_t)n * p.w_stride_n * E::kBytes) + (uint32_t)c * 16u
-                    : kOob;
+    if constexpr (!WT) {
+      const int rho = (wave * IPW + t) * RPI + lrow;      // LDS row, fragment order
+      const int i = rho & 15, nb = (rho >> 4) % NBW, wq = rho / (16 * NBW);
+      const int n = n0 + wq * (16 * NBW) + (i >> 2) * (4 * NBW) + nb * 4 + (i & 3);
+      const int c = lchunk ^ swz(rho);
+      w_voff[t] = n < p.k_out && c * PV < p.c_in
+                      ? (uint32_t)((int64_t)n * p.w_stride_n * E::kBytes) + (uint32_t)c * 16u
+                      : kOob;
+    } else {
+      const int e = (wave * IPW + t) * RPIW + lane / LPRW;   // contraction row
+      const int c = (lane % LPRW) ^ swz_w(e);                 // chunk of the row this lane fetches
+      const int n = n0 + c * PV;
+      w_voff[t] = e < p.c_in && n < p.k_out
+                      ? (uint32_t)(((int64_t)e * p.w_stride_c + n) * E::kBytes)
+                      : kOob;
+    }
   }
 
   // ---- reader role: fragment slots (16-byte units) relative to the wave's first row
@@ -218,6 +241,21 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     const int slot = m * LPR + ((s * 4 + q) ^ swz(m));
     a_rd[s] = wm * (RBW * 16) * LPR + slot;
     w_rd[s] = A_V + wn * (NBW * 16) * LPR + slot;
+  }
+  // transposing reads: byte address inside the weight part for (k-step s, half h, block nb)
+  int wt_rd[WT ? KS : 1][2][WT ? NBW : 1];
+  if constexpr (WT) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb) {
+          const int e = s * 32 + q * 8 + h * 4 + (m >> 2);
+          const int col = (wn * NBW + nb) * 16 + 4 * (m & 3);          // first channel (tile local)
+          const int chunk = (col / PV) ^ swz_w(e);
+          wt_rd[s][h][nb] = A_V * 16 + e * (LPRW * 16) + chunk * 16 + (col % PV) * E::kBytes;
+        }
   }
 
   // ---- output rows of this lane
@@ -325,7 +363,20 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
 #pragma unroll
       for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
-        for (int s = 0; s < KS; ++s) wf[nb][s] = st[w_rd[s] + nb * 16 * LPR];
+        for (int s = 0; s < KS; ++s) {
+          if constexpr (!WT) {
+            wf[nb][s] = st[w_rd[s] + nb * 16 * LPR];
+          } else {
+            typedef short v4s __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) v4s *lds_v4s;
+            const char *base = reinterpret_cast<const char *>(st);
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(base + wt_rd[s][0][nb]));
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(base + wt_rd[s][1][nb]));
+            typedef short v8s __attribute__((ext_vector_type(8)));
+            const v8s both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            wf[nb][s] = __builtin_bit_cast(v4i, both);
+          }
+        }
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb)
 #pragma unroll
@@ -358,7 +409,37 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     constexpr int ACT = decltype(act_c)::value;
     constexpr int MODE = decltype(mode_c)::value;
     constexpr bool SRC = (MODE & 1) != 0;
-    if constexpr (E::kBytes == 2) {
+    if constexpr (E::kBytes == 2 && WT) {
+      // channels nb*16 + 4q .. +3 of each block: 8-byte pieces
+      typedef int v2i __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int rb = 0; rb < RBW; ++rb) {
+        const int o = out_row[rb];
+        const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb) {
+          const int ch = n0 + (wn * NBW + nb) * 16 + 4 * q;
+          const bool ok = row_ok && ch < p.k_out;
+          const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
+          v2i src = {0, 0};
+          if constexpr (SRC) {
+            const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 2u : kOob;
+            src = __builtin_amdgcn_raw_buffer_load_b64(rs_d, doff, 0, 0);
+          }
+          const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
+          v2i outv;
+          uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            const float a = acc[rb][nb][x];
+            float t = SRC ? __builtin_fmaf(p.alpha, a, p.beta * E::to_float(sh[x])) : p.alpha * a;
+            t = apply_act(t, ACT, p.act_alpha);
+            oh[x] = E::from_float(t);
+          }
+          __builtin_amdgcn_raw_buffer_store_b64(outv, rs_c, coff, 0, 0);
+        }
+      }
+    } else if constexpr (E::kBytes == 2) {
       constexpr int NG = CPLW / 8;   // 16-byte groups
       static_assert(CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
 #pragma unroll
