@@ -176,6 +176,28 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   const int n0 = blockIdx.y * TN;
   const int pos_base = tile * TM;
 
+  // requantisation scale and bias of this lane's output channels (one-byte outputs): requested
+  // now, used in the epilogue; without the int8 epilogue the descriptors have no records
+  float scale_v[E::kBytes == 1 ? 4 * NBW : 1], bias_v[E::kBytes == 1 ? 4 * NBW : 1];
+  if constexpr (E::kBytes == 1) {
+    const uint32_t sb_bytes = p.int8_epilogue ? (uint32_t)p.k_out * 4u : 0u;
+    const __amdgpu_buffer_rsrc_t rs_scale = make_rsrc(p.scale, sb_bytes);
+    const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(p.bias, sb_bytes);
+    const uint32_t off = (uint32_t)(n0 + wn * (NBW * 16) + q * (4 * NBW)) * 4u;
+#pragma unroll
+    for (int g = 0; g < NBW; ++g) {
+      // (whole-vector casts: a per-element cast of the loaded vector was seen to be compiled
+      // into a load of element 0 only)
+      const v4f sv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_scale, off + g * 16, 0, 0));
+      const v4f bv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_bias, off + g * 16, 0, 0));
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        scale_v[g * 4 + x] = sv[x];
+        bias_v[g * 4 + x] = bv[x];
+      }
+    }
+  }
+
   // ---- the tile's mask words are requested first and reduced only after the row keys below have
   // been requested too: one memory round trip for both
   uint32_t mk = 0;
@@ -470,43 +492,41 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
         }
       }
     } else {
-      // one-byte outputs: 4*NBW bytes per lane and row, moved as dwords
+      // one-byte outputs: the lane's 4*NBW consecutive channels are 8 or 16 bytes of the row.
+      // Scale and bias of these channels were requested when the kernel started.
       constexpr int ND = CPLW / 4;
+      typedef int vNi __attribute__((ext_vector_type(ND)));
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb) {
         const int o = out_row[rb];
-        const bool row_ok = o >= 0 && o < p.rows_c;
-#pragma unroll
-        for (int g = 0; g < ND; ++g) {
-          const int ch = ch0 + g * 4;
-          const bool ok = row_ok && ch < p.k_out;
-          const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) : kOob;
-          int src = 0;
-          if constexpr (SRC) {
-            const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) : kOob;
-            src = __builtin_amdgcn_raw_buffer_load_b32(rs_d, doff, 0, 0);
-          }
-          const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
-          int outv;
-          int8_t *ob = reinterpret_cast<int8_t *>(&outv);
-#pragma unroll
-          for (int x = 0; x < 4; ++x) {
-            const int a = acc[rb][g][x];
-            float t;
-            if constexpr (MODE >= 2) {
-              const int c = ch + x < p.k_out ? ch + x : 0;
-              t = __builtin_fmaf(p.scale[c], (float)a, p.bias[c]);
-              if constexpr (SRC) t = __builtin_fmaf(p.beta, (float)sb[x], t);
-            } else if constexpr (SRC) {
-              t = __builtin_fmaf(p.alpha, (float)a, p.beta * (float)sb[x]);
-            } else {
-              t = p.alpha * (float)a;
-            }
-            t = apply_act(t, ACT, p.act_alpha);
-            ob[x] = (int8_t)f32_to_s8(t);
-          }
-          __builtin_amdgcn_raw_buffer_store_b32(outv, rs_c, coff, 0, 0);
+        const bool ok = o >= 0 && o < p.rows_c && ch0 < p.k_out;
+        const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch0) : kOob;
+        vNi src = {};
+        if constexpr (SRC) {
+          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch0) : kOob;
+          if constexpr (ND == 4) src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
+          else src = __builtin_amdgcn_raw_buffer_load_b64(rs_d, doff, 0, 0);
         }
+        const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
+        vNi outv;
+        int8_t *ob = reinterpret_cast<int8_t *>(&outv);
+#pragma unroll
+        for (int x = 0; x < CPLW; ++x) {
+          const int a = acc[rb][x >> 2][x & 3];
+          float t;
+          if constexpr (MODE >= 2) {
+            t = __builtin_fmaf(scale_v[x], (float)a, bias_v[x]);
+            if constexpr (SRC) t = __builtin_fmaf(p.beta, (float)sb[x], t);
+          } else if constexpr (SRC) {
+            t = __builtin_fmaf(p.alpha, (float)a, p.beta * (float)sb[x]);
+          } else {
+            t = p.alpha * (float)a;
+          }
+          t = apply_act(t, ACT, p.act_alpha);
+          ob[x] = (int8_t)f32_to_s8(t);
+        }
+        if constexpr (ND == 4) __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
+        else __builtin_amdgcn_raw_buffer_store_b64(outv, rs_c, coff, 0, 0);
       }
     }
   };
