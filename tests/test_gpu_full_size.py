@@ -1,0 +1,127 @@
+"""Parity at the benchmark configurations' full sizes (thousands of tiles, many
+more than the device holds workgroups at once), against the CPU oracle on the
+same seeded inputs, plus a size-independent property (linearity in the
+features) for the f16 forward."""
+import numpy as np
+import pytest
+
+import helpers as H
+from cumm_amd import pairs, synth
+from cumm_amd import tensorview as tv
+from cumm_amd.conv.main import ConvMainUnitTest
+from cumm_amd.gemm.main import GemmMainUnitTest
+from cumm_amd.tensorview.gemm import ConvOpType, ConvParams, GemmParams, ShuffleStrideType
+from oracle import conv_ref, gemm_ref
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2          # max |got - ref| / max |ref| for f16 / bf16 outputs
+GRID = (41, 1600, 1408)
+
+
+def _subm_case(seed, n_target, dtype, c, k):
+    rng = np.random.default_rng(seed)
+    coords = synth.clustered_voxels(rng, n_target, GRID, 60, sigma=15.0, noise_frac=0.10)
+    pt = pairs.subm_pairs(coords, GRID)
+    n = coords.shape[0]
+    feat = H.to_storage(rng.normal(0, 1, size=(n, c)).astype(np.float32), dtype)
+    w = H.to_storage(rng.normal(0, 0.05, size=(k, 27, c)).astype(np.float32), dtype)
+    return rng, pt, feat, w, n
+
+
+@pytest.mark.parametrize("tile_m", [64, 128])
+def test_subm_f16_c64_forward_dgrad_full_size(tile_m):
+    print("case full size subm f16", tile_m, flush=True)
+    dtype = "f16"
+    rng, pt, feat, w, n = _subm_case(20240607, 120000, dtype, 64, 64)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    out0 = np.zeros((n, 64), np.float16)
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, tile_m, 64)
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    p.mask_output = tv.zeros([(n + tile_m - 1) // tile_m], tv.uint32, 0)
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref, mask_out = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=tile_m,
+                                                   dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+    got = H.as_f32(H.host(p.output), dtype)
+    assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+    np.testing.assert_array_equal(H.host(p.mask_output), mask_out)   # integer work: bit-exact
+
+    # linearity: conv(2 x) == 2 conv(x); scaling by two is exact in f32 and in normal f16 (no
+    # overflow here), only subnormal f16 results may round differently (one subnormal ulp, 2^-24)
+    p2 = ConvParams(3, ConvOpType.Forward)
+    p2.conv_algo_desp = p.conv_algo_desp
+    p2.input = H.dev((feat.astype(np.float32) * 2).astype(np.float16), dtype)
+    p2.weight, p2.output = p.weight, H.dev(out0, dtype)
+    p2.indices, p2.mask, p2.mask_argsort = p.indices, p.mask, p.mask_argsort
+    ConvMainUnitTest.implicit_gemm2(p2)
+    got2 = H.as_f32(H.host(p2.output), dtype)
+    normal = np.abs(got) >= 2.0 ** -14
+    np.testing.assert_array_equal(got2[normal], 2 * got[normal])
+    assert np.max(np.abs(got2 - 2 * got)) <= 2.0 ** -23
+
+    # backward-input on the same pair table
+    dout = H.to_storage(rng.normal(0, 1, size=(n, 64)).astype(np.float32), dtype)
+    din0 = np.zeros((n, 64), np.float16)
+    pd = ConvParams(3, ConvOpType.BackwardInput)
+    pd.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, tile_m, 64)
+    pd.input, pd.weight, pd.output = H.dev(din0, dtype), p.weight, H.dev(dout, dtype)
+    pd.indices = H.dev(pt.indices_bwd, "i32")
+    pd.mask, pd.mask_argsort = p.mask, p.mask_argsort
+    pd.reverse_mask = True
+    ConvMainUnitTest.implicit_gemm2(pd)
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, din0, pt.indices_bwd, ms, order, tile_m=tile_m,
+                                             dtype_in=dtype, dtype_w=dtype, dtype_out=dtype, reverse_mask=True)
+    assert H.rel_err(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_d, dtype)) < TOL
+
+
+def test_s8_stride2_full_size_bit_exact():
+    print("case full size s8 stride 2", flush=True)
+    rng = np.random.default_rng(20240611)
+    coords = synth.clustered_voxels(rng, 300000, GRID, 60, sigma=15.0, noise_frac=0.10)
+    pt = pairs.sparse_conv_pairs(coords, GRID)
+    n_in, n_out = coords.shape[0], pt.indices_fwd.shape[1]
+    feat = rng.integers(-127, 128, size=(n_in, 64)).astype(np.int8)
+    w = rng.integers(-127, 128, size=(128, 27, 64)).astype(np.int8)
+    scale = rng.uniform(0.001, 0.01, size=(128,)).astype(np.float32)
+    bias = rng.normal(0, 1, size=(128,)).astype(np.float32)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    out0 = np.zeros((n_out, 128), np.int8)
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = H.find_conv_desp("s8", ConvOpType.Forward, 64, 128, int8_inference=True)
+    p.input, p.weight, p.output = H.dev(feat, "s8"), H.dev(w, "s8"), H.dev(out0, "s8")
+    p.scale, p.bias = H.dev(scale, "f32"), H.dev(bias, "f32")
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in="s8",
+                                            dtype_w="s8", dtype_out="s8", scale=scale, bias=bias,
+                                            int8_inference=True)
+    np.testing.assert_array_equal(H.host(p.output), ref)
+
+
+def test_gather_gemm_scatter_full_size():
+    """One kernel offset: F[200000,64] f16, W[64,64], 150000 (in, out) pairs, alpha = beta = 1."""
+    print("case full size gather-gemm-scatter", flush=True)
+    dtype = "f16"
+    rng = np.random.default_rng(20240609)
+    rows, m, n, k = 200000, 150000, 64, 64
+    a = H.to_storage(rng.normal(0, 1, size=(rows, k)).astype(np.float32), dtype)
+    b = H.to_storage(rng.normal(0, 0.1, size=(k, n)).astype(np.float32), dtype)
+    a_inds = rng.permutation(rows)[:m].astype(np.int32)
+    c_inds = rng.permutation(rows)[:m].astype(np.int32)
+    c0 = H.to_storage(rng.normal(0, 1, size=(rows, n)).astype(np.float32), dtype)
+    p = GemmParams()
+    p.algo_desp = H.find_gemm_desp(dtype, ShuffleStrideType.ShuffleAC, 64, 64, False, False)
+    p.a, p.b, p.c = H.dev(a, dtype), H.dev(b, dtype), H.dev(c0, dtype)
+    p.a_inds, p.c_inds = H.dev(a_inds, "i32"), H.dev(c_inds, "i32")
+    p.alpha, p.beta = 1.0, 1.0
+    GemmMainUnitTest.matmul2(p)
+    ref = gemm_ref.matmul2_ref(a, b, c0, dtype_a=dtype, dtype_b=dtype, dtype_c=dtype,
+                               shuffle=gemm_ref.SHUFFLE_AC, a_inds=a_inds, c_inds=c_inds, alpha=1.0, beta=1.0)
+    got = H.as_f32(H.host(p.c), dtype)
+    assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+    untouched = np.setdiff1d(np.arange(rows), c_inds)
+    np.testing.assert_array_equal(H.host(p.c)[untouched], c0[untouched])   # rows not in c_inds stay as they were
