@@ -24,7 +24,9 @@ sys.path.insert(0, ROOT)
 from cumm_amd import pairs, synth  # noqa: E402
 from cumm_amd import tensorview as tv  # noqa: E402
 from cumm_amd.conv.main import ConvMainUnitTest  # noqa: E402
-from cumm_amd.tensorview.gemm import ConvOpType, ConvParams  # noqa: E402
+from cumm_amd.gemm.main import GemmMainUnitTest  # noqa: E402
+from cumm_amd.tensorview.gemm import (ConvOpType, ConvParams, GemmParams,  # noqa: E402
+                                      ShuffleStrideType)
 
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per forward launch of the default workload (tile_m = 64), from two rocprofv3 --pmc runs
@@ -111,6 +113,50 @@ def bench_wgrad(args, p, dout, n, C, K, tile_m, flops, parallel):
             "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3)}
 
 
+def find_gemm_desp(shuffle, tile_m, tile_n, trans_b):
+    for d in GemmMainUnitTest.get_all_algo_desp():
+        if (d.dtype_a == tv.float16 and d.shuffle_type == shuffle and d.tile_shape[0] == tile_m and
+                d.tile_shape[1] == tile_n and not d.trans_a and d.trans_b == trans_b and not d.trans_c):
+            return d
+    raise KeyError((shuffle, tile_m, tile_n, trans_b))
+
+
+def bench_gather_gemm(args):
+    """One kernel offset as a GEMM: F[200000,64] f16, W[64,64], 150000 (in, out) pairs,
+    out[c] = F[a] @ W + out[c] (matmul2 with A-row gather and C-row scatter)."""
+    rng2 = np.random.default_rng(SEED + 2)
+    rows, m, n, k = 200000, 150000, 64, 64
+    pg = GemmParams()
+    pg.algo_desp = find_gemm_desp(ShuffleStrideType.ShuffleAC, 64, 64, False)
+    pg.a = dev(rng2.normal(0, 1, size=(rows, k)).astype(np.float16))
+    pg.b = dev(rng2.normal(0, 0.1, size=(k, n)).astype(np.float16))
+    pg.c = tv.zeros([rows, n], tv.float16, 0)
+    pg.a_inds = dev(rng2.permutation(rows)[:m].astype(np.int32))
+    pg.c_inds = dev(rng2.permutation(rows)[:m].astype(np.int32))
+    pg.alpha, pg.beta = 1.0, 1.0
+    w_ms, e_ms = timed(lambda: GemmMainUnitTest.matmul2(pg), args.steps, args.warmup)
+    nbytes = m * k * 2 + 2 * m * n * 2 + k * n * 2 + 2 * m * 4
+    return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
+            "tflops": round(2.0 * m * n * k / (w_ms * 1e-3) / 1e12, 3),
+            "hbm_frac": round(nbytes / (e_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+
+
+def bench_dense_gemm(args):
+    """Plain matmul2, 4096^3 f16 (the only MFMA-bound shape of the path)."""
+    rng3 = np.random.default_rng(SEED + 3)
+    mnk = 4096
+    pd = GemmParams()
+    pd.algo_desp = find_gemm_desp(ShuffleStrideType.NoShuffle, 128, 128, True)
+    pd.a = dev(rng3.normal(0, 1, size=(mnk, mnk)).astype(np.float16))
+    pd.b = dev(rng3.normal(0, 0.05, size=(mnk, mnk)).astype(np.float16))   # [n, k]: trans_b
+    pd.c = tv.zeros([mnk, mnk], tv.float16, 0)
+    steps = max(5, args.steps // 10)
+    w_ms, e_ms = timed(lambda: GemmMainUnitTest.matmul2(pd), steps, max(2, args.warmup // 10))
+    tf = 2.0 * mnk ** 3 / (w_ms * 1e-3) / 1e12
+    return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5), "tflops": round(tf, 2),
+            "pct_mfma_peak": round(100.0 * tf / PEAK_MFMA_F16_TFLOPS, 3)}
+
+
 def bench_s8(args, tile_m):
     """s8 stride-2 SparseConv3d, Cin=64 -> Cout=128, int8 inference epilogue."""
     rng4 = np.random.default_rng(SEED + 4)
@@ -145,7 +191,7 @@ def main():
     ap.add_argument("--tile-m", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
-    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8")
+    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on 512 MiB (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -221,7 +267,8 @@ def main():
 
     if not args.no_extra:
         extra = {}
-        legs = set(args.extra_only.split(",")) if args.extra_only else {"dgrad", "wgrad", "s8"}
+        legs = (set(args.extra_only.split(",")) if args.extra_only
+                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)
         dout = dev(rng.normal(0, 1, size=(n, K)).astype(np.float16))
         if "dgrad" in legs:
@@ -231,6 +278,10 @@ def main():
             extra["subm_f16_wgrad_serial_splitk32"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops, False)
         if "s8" in legs:
             extra["sparseconv_s8_stride2"] = bench_s8(args, tile_m)
+        if "gather_gemm" in legs:
+            extra["gather_gemm_scatter_f16"] = bench_gather_gemm(args)
+        if "dense_gemm" in legs:
+            extra["dense_gemm_f16_4096"] = bench_dense_gemm(args)
         result["extra"] = extra
     if not args.no_cpu:
         # CPU baseline: the numpy oracle (per-offset gather -> matmul -> scatter-add) on the
