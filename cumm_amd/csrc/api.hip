@@ -436,8 +436,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
     const size_t need = sizeof(float) * (size_t)a->K * kv * a->C;
     if (!a->workspace || a->workspace_bytes < need)
       return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
-    if (reinterpret_cast<uintptr_t>(a->workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
-    HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
+    if (reinterpret_cast<uintptr_t>(a->workspace) & 15u) return fail(CUMM_HIP_EINVAL, "workspace must be 16-byte aligned");
     WgradParams w;
     std::memset(&w, 0, sizeof(w));
     w.dout = a->ptr_A; w.inp = a->ptr_B; w.scratch = reinterpret_cast<float *>(a->workspace);
@@ -446,7 +445,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
     w.mask_filter = a->mask_filter;
     w.n_pos = a->N; w.n_idx = a->N; w.rows_x = a->rows_in; w.rows_y = a->rows_out;
     w.K = a->K; w.C = a->C; w.kv = kv;
-    int qt = 512 / a->mask_width;
+    int qt = kWgradMaxPos / a->mask_width;
     if (qt < 1) qt = 1;
     w.tiles_per_wg = qt;
     WgradFinalizeParams f;
@@ -454,7 +453,35 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
     f.scratch = w.scratch; f.dw = a->ptr_C; f.src = ptr_D;
     f.total = (int64_t)a->K * kv * a->C; f.C = a->C; f.kv = kv; f.mask_filter = a->mask_filter;
     f.alpha = a->alpha; f.beta = a->beta;
-    hipError_t e = dt == CUMM_HIP_F16 ? launch_wgrad_atomic_f16(w, f, stream) : launch_wgrad_atomic_bf16(w, f, stream);
+    // With room behind the fp32 image for the per-offset live-tile lists, a prepare kernel makes
+    // them (and zeroes the image) and the unit-walking kernel runs; as many more copies of the
+    // image as fit (at most 8, at most split_k_slices) spread its atomics.  Otherwise the image is
+    // zeroed here and every workgroup of the scanning kernel reads the mask itself.
+    const size_t image_bytes = (need + 255) & ~(size_t)255;
+    const size_t lists_bytes = 128 + sizeof(int32_t) * (size_t)kv * w.num_red;
+    int images = 0;
+    for (int s = 8; s >= 1 && !images; s >>= 1)
+      if (s <= a->split_k_slices && a->workspace_bytes >= s * image_bytes + lists_bytes) images = s;
+    const bool fits32 = (int64_t)a->rows_out * a->K * 2 < (int64_t)1 << 31 && (int64_t)a->rows_in * a->C * 2 < (int64_t)1 << 31;
+    WgradPrepareParams pre;
+    std::memset(&pre, 0, sizeof(pre));
+    w.images = f.images = 1;
+    // (the unit-walking kernel divides unit numbers with a float reciprocal: exact below 2^22)
+    const int64_t unit_bound = ((int64_t)(w.num_red + qt - 1) / qt + 1) * kv * (((int64_t)a->K + 63) / 64) * (((int64_t)a->C + 63) / 64);
+    if (images && fits32 && unit_bound < ((int64_t)1 << 22) && w.num_red < (1 << 22)) {
+      char *base = reinterpret_cast<char *>(a->workspace);
+      const size_t lists_at = images * image_bytes;
+      pre.scratch = w.scratch; pre.scratch_floats = (int64_t)(lists_at / sizeof(float));
+      pre.red_mask = w.red_mask; pre.num_red = w.num_red; pre.kv = kv; pre.mask_filter = w.mask_filter;
+      pre.live_cnt = reinterpret_cast<int32_t *>(base + lists_at);
+      pre.live_list = reinterpret_cast<int32_t *>(base + lists_at + 128);
+      w.live_cnt = pre.live_cnt; w.live_list = pre.live_list;
+      w.images = f.images = images;
+      w.image_floats = f.image_floats = (int64_t)(image_bytes / sizeof(float));
+    } else {
+      HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
+    }
+    hipError_t e = dt == CUMM_HIP_F16 ? launch_wgrad_atomic_f16(w, pre, f, stream) : launch_wgrad_atomic_bf16(w, pre, f, stream);
     if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
     return CUMM_HIP_OK;
   }

@@ -20,8 +20,8 @@ hipError_t launch_tilegemm_s8(int tm, int tn, bool xk, bool yk, const TileGemmPa
                               hipStream_t s);
 
 // balanced backward-weight with fp32 atomics: main kernel then finalize (f16 / bf16 only)
-hipError_t launch_wgrad_atomic_f16(const WgradParams &p, const WgradFinalizeParams &f, hipStream_t s);
-hipError_t launch_wgrad_atomic_bf16(const WgradParams &p, const WgradFinalizeParams &f, hipStream_t s);
+hipError_t launch_wgrad_atomic_f16(const WgradParams &p, const WgradPrepareParams &pre, const WgradFinalizeParams &f, hipStream_t s);
+hipError_t launch_wgrad_atomic_bf16(const WgradParams &p, const WgradPrepareParams &pre, const WgradFinalizeParams &f, hipStream_t s);
 
 // tile shapes the tables above hold
 inline bool rowgemm_has_tile(int tm, int tn) {

@@ -31,65 +31,10 @@
 #include <type_traits>
 #include <utility>
 
+#include "lds_dma.h"
 #include "rowgemm.h"
 
 namespace cummhip {
-
-#define CUMM_LDS_PTR(x) ((__attribute__((address_space(3))) void *)(x))
-
-// s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt = simm16[15:14,3:0])
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
-}
-
-// OR over the 64 lanes of a wave with row shifts and row broadcasts (no LDS round trips)
-__device__ __forceinline__ uint32_t wave_or_dpp(uint32_t v) {
-  int t = (int)v;
-  t |= __builtin_amdgcn_update_dpp(0, t, 0x111, 0xf, 0xf, true);   // row_shr:1
-  t |= __builtin_amdgcn_update_dpp(0, t, 0x112, 0xf, 0xf, true);   // row_shr:2
-  t |= __builtin_amdgcn_update_dpp(0, t, 0x114, 0xf, 0xf, true);   // row_shr:4
-  t |= __builtin_amdgcn_update_dpp(0, t, 0x118, 0xf, 0xf, true);   // row_shr:8 -> lane 15 of a row
-  t |= __builtin_amdgcn_update_dpp(0, t, 0x142, 0xa, 0xf, true);   // row_bcast:15 into rows 1, 3
-  t |= __builtin_amdgcn_update_dpp(0, t, 0x143, 0xc, 0xf, true);   // row_bcast:31 into rows 2, 3
-  return (uint32_t)__builtin_amdgcn_readlane(t, 63);
-}
-
-// Direct-to-LDS buffer loads, written as asm so that the compiler's wait-count pass does not see
-// them: it guards LDS reads that may alias an outstanding direct-to-LDS load with waits of its
-// own, and at a loop header it assumes the worst (waits for all of them), which would drain the
-// ring once per trip.  Every wait for these loads is placed by hand (wait_vmcnt).  Hidden loads
-// cannot make a wait of the compiler too weak: loads complete in order, so more outstanding loads
-// than it counted only make its waits stricter than needed.
-// rsrc: buffer descriptor words; lds: byte address of the destination of lane 0 (lane l lands at
-// lds + l*size); voff: per-lane byte offset; soff: wave-uniform byte offset.
-__device__ __forceinline__ v4i rsrc_words(const void *ptr, uint32_t bytes) {
-  const uint64_t a = (uint64_t)ptr;
-  return v4i{(int)(uint32_t)a, (int)((uint32_t)(a >> 32) & 0xffffu), (int)bytes, 0x00020000};
-}
-template <class P>
-__device__ __forceinline__ uint32_t lds_addr(P *ptr) {
-  return (uint32_t)(uintptr_t)CUMM_LDS_PTR(ptr);
-}
-__device__ __forceinline__ void dma_b128(v4i rsrc, uint32_t lds, uint32_t voff, uint32_t soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :: "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
-}
-__device__ __forceinline__ void dma_b32(v4i rsrc, uint32_t lds, uint32_t voff, uint32_t soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
-               :: "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
-}
-
-// Workgroup barrier without the fence of __syncthreads(): the fence would wait for every
-// outstanding direct-to-LDS load, i.e. also for the stages that are being prefetched.  The empty
-// asm statements keep the compiler from moving LDS accesses across the barrier; the caller waits
-// for the loads that the other waves are going to read before calling this.
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
 
 template <class F, int... Is>
 __device__ __forceinline__ bool run_steps(F &f, std::integer_sequence<int, Is...>) {

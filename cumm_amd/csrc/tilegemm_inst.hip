@@ -25,17 +25,41 @@ hipError_t CUMM_CAT(launch_tilegemm_, CUMM_NAME)(int tm, int tn, bool xk, bool y
 }
 
 #ifndef CUMM_NO_WGRAD_ATOMIC
-hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const WgradFinalizeParams &f,
-                                                     hipStream_t s) {
+hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const WgradPrepareParams &pre,
+                                                     const WgradFinalizeParams &f, hipStream_t s) {
   using T = CUMM_ELEM;
   const int groups = (p.num_red + p.tiles_per_wg - 1) / p.tiles_per_wg;
   const int kblocks = (p.K + 63) / 64, cblocks = (p.C + 63) / 64;
-  dim3 grid(groups, p.kv * kblocks * cblocks, 1);
-  if (grid.x == 0 || grid.y == 0) return hipSuccess;
-  hipLaunchKernelGGL((wgrad_atomic_kernel<T>), grid, dim3(256), 0, s, p);
-  hipError_t e = hipGetLastError();
+  if (groups == 0 || p.kv == 0) return hipSuccess;
+  hipError_t e;
+  if (p.live_list != nullptr) {
+    // lists + zeroed image, then a resident grid that walks the units
+    static int resident_of[16] = {};
+    int dev = 0;
+    e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    int &resident = resident_of[dev & 15];
+    if (resident == 0) {
+      int cus = 0, per_cu = 0;
+      e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (e == hipSuccess) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wgrad_units_kernel<T>, 256, 0);
+      if (e != hipSuccess) return e;
+      resident = cus * per_cu > 0 ? cus * per_cu : 1;
+    }
+    hipLaunchKernelGGL(wgrad_prepare_kernel, dim3(p.kv + 256), dim3(256), 0, s, pre);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    // never more workgroups than units can exist
+    const long long max_units = ((long long)groups * p.kv + p.kv) * kblocks * cblocks;
+    hipLaunchKernelGGL((wgrad_units_kernel<T>), dim3((unsigned)(max_units < resident ? max_units : resident)),
+                       dim3(256), 0, s, p);
+  } else {
+    dim3 grid(groups, p.kv * kblocks * cblocks, 1);
+    hipLaunchKernelGGL((wgrad_atomic_kernel<T>), grid, dim3(256), 0, s, p);
+  }
+  e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL((wgrad_finalize_kernel<T>), dim3((unsigned)((f.total + 255) / 256)), dim3(256), 0, s, f);
+  hipLaunchKernelGGL((wgrad_finalize_kernel<T>), dim3((unsigned)((f.total / 4 + 255) / 256)), dim3(256), 0, s, f);
   return hipGetLastError();
 }
 #endif

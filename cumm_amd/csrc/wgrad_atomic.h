@@ -5,19 +5,25 @@
 //
 // The reference splits the positions into split_k_slices equal strides per kernel offset
 // (cumm/conv/kernel.py:891-897, cumm/gemm/blockmma/mma.py:580-765): with sorted masks almost all
-// work sits in one offset (the centre) and its slices serialise on a semaphore.  Here
-//   * for its offset r every workgroup scans the reduced mask (one word per mask_width positions,
-//     the forward's mask_output), counts the live tiles L_r and the offset gets ceil(L_r / QT)
-//     workgroups, each taking an equal share of the LIVE tiles only; surplus workgroups exit;
-//   * the workgroup first loads argsort and the pair-table entries of all its positions into LDS
-//     (two memory round trips for everything), then streams 32 positions per step: gathered dOut
-//     and In rows go to LDS transposed (contraction = positions must be contiguous for the MFMA),
-//     the next step's rows are in flight while the current step computes;
-//   * partial 64x64 blocks are added into an fp32 scratch image of dW with hardware float
-//     atomics; a second kernel applies alpha/beta and converts to the weight type.
+// work sits in one offset (the centre) and its slices serialise on a semaphore.  Here the work of
+// offset r is its LIVE tiles only (reduced mask word, i.e. the forward's mask_output, has bit r),
+// cut into units of QT tiles; a unit makes one partial 64x64 block (per channel block) and adds
+// it into an fp32 scratch image of dW with hardware float atomics; a last kernel applies
+// alpha/beta and converts to the weight type.  Two ways to get there:
+//   * wgrad_prepare_kernel + wgrad_units_kernel (workspace has room for the live-tile lists): the
+//     prepare kernel compacts, per offset, the numbers of its live tiles and zeroes the images;
+//     the unit kernel is a grid of resident workgroups that walk the units of all offsets.  A unit
+//     resolves tile list -> argsort -> pair table for all of its positions at once, packs the
+//     positions that have a pair, and streams their gathered rows through an LDS ring filled by
+//     direct-to-LDS loads; the MFMA operands (contraction = pairs) come out of the row-major
+//     tiles through transposing LDS reads.
+//   * wgrad_atomic_kernel (no room for lists; image zeroed by a memset): a (groups, offsets) grid,
+//     every workgroup scans the reduced mask for its offset itself and surplus workgroups exit;
+//     rows pass through registers and are parked in LDS transposed with 16-bit stores.
 // The sum order is not fixed (fp32 atomics), the partial sums are never rounded to the weight type.
 #pragma once
 #include "common.h"
+#include "lds_dma.h"
 
 namespace cummhip {
 
@@ -33,6 +39,14 @@ struct WgradParams {
   int32_t n_pos, n_idx, rows_x, rows_y;
   int32_t K, C, kv;
   int32_t tiles_per_wg;     // QT
+  // live-tile lists made by wgrad_prepare_kernel (NULL: every workgroup scans the mask itself):
+  // live_cnt[r] = number of tiles whose reduced mask has bit r, live_list[r * num_red + i] = the i-th
+  const int32_t *live_cnt;
+  const int32_t *live_list;
+  // the unit-walking kernel spreads its atomics over `images` copies of the fp32 image, each
+  // image_floats apart; the finalize kernel sums them
+  int32_t images;
+  int64_t image_floats;
 };
 
 constexpr int kWgradMaxPos = 1024;  // positions one workgroup handles at most (QT * mask_width)
@@ -178,6 +192,7 @@ __global__ __launch_bounds__(256) void wgrad_atomic_kernel(const WgradParams p) 
   // holds K indices 4q + x and one C index l16: for a fixed x the 16 lanes of a quarter hit 16
   // consecutive floats (one 64-byte segment per quarter).
   const int64_t ldn = (int64_t)p.kv * p.C;
+  float *image = p.scratch;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -188,10 +203,317 @@ __global__ __launch_bounds__(256) void wgrad_atomic_kernel(const WgradParams p) 
       for (int x = 0; x < 4; ++x) {
         const int mm = kb * 64 + (wm * 2 + i) * 16 + 4 * q + x;
         if (mm < p.K)
-          __hip_atomic_fetch_add(p.scratch + mm * ldn + (int64_t)r * p.C + nn, acc[i][j][x],
+          __hip_atomic_fetch_add(image + mm * ldn + (int64_t)r * p.C + nn, acc[i][j][x],
                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
+  }
+}
+
+// ---- variant that reads the live-tile lists made by wgrad_prepare_kernel: a resident grid whose
+// workgroups walk the units (offset r, channel blocks, share x of the offset's live tiles) u = b,
+// b + G, ...: no workgroup scans the mask, none is launched only to find that it has nothing to do.
+struct WgradPrepareParams {
+  float *scratch;             // zeroed here
+  int64_t scratch_floats;
+  const uint32_t *red_mask;
+  int32_t num_red, kv;
+  uint32_t mask_filter;
+  int32_t *live_cnt;          // [32]
+  int32_t *live_list;         // [kv * num_red]
+};
+
+// workgroup r < kv compacts the tiles of offset r; the others zero the fp32 image
+static __global__ __launch_bounds__(256) void wgrad_prepare_kernel(const WgradPrepareParams p) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if ((int)blockIdx.x >= p.kv) {
+    const int64_t nz = (int64_t)(gridDim.x - p.kv) * 256;   // scratch_floats is a multiple of 4
+    v4f *z = reinterpret_cast<v4f *>(p.scratch);
+    for (int64_t i = (int64_t)(blockIdx.x - p.kv) * 256 + tid; i < p.scratch_floats / 4; i += nz) z[i] = v4f{0, 0, 0, 0};
+    return;
+  }
+  __shared__ int wave_cnt[2][4];
+  const int r = blockIdx.x;
+  const bool on = (p.mask_filter >> r) & 1u;
+  int base = 0;
+  constexpr int U = 8;   // mask words a thread has in flight
+  for (int t0 = 0; t0 < p.num_red; t0 += 256 * U) {
+    uint32_t m[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = t0 + u * 256 + tid;
+      m[u] = t < p.num_red ? p.red_mask[t] : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = t0 + u * 256 + tid;
+      const bool live = on && ((m[u] >> r) & 1u);
+      const uint64_t bal = __ballot(live);
+      if (lane == 0) wave_cnt[u & 1][wave] = __builtin_popcountll(bal);
+      __syncthreads();   // the other set of counters is free again: everybody passed the previous barrier
+      int before = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int c = wave_cnt[u & 1][w];
+        before += w < wave ? c : 0;
+        total += c;
+      }
+      if (live) p.live_list[(int64_t)r * p.num_red + base + before + __builtin_popcountll(bal & ((1ull << lane) - 1ull))] = t;
+      base += total;
+    }
+  }
+  if (tid == 0) p.live_cnt[r] = base;
+}
+
+// a / b for 0 <= a < 2^22, 0 < b < 2^22, without the long integer-division sequence
+__device__ __forceinline__ int fast_div(int a, int b) {
+  int qn = (int)((float)a * __builtin_amdgcn_rcpf((float)b));
+  const int rem = a - qn * b;
+  if (rem < 0) --qn;
+  if (rem >= b) ++qn;
+  return qn;
+}
+
+// inclusive prefix sum over the 64 lanes of a wave with row shifts and row broadcasts
+__device__ __forceinline__ int wave_prefix_sum_dpp(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, true);   // row_bcast:15 into rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, true);   // row_bcast:31 into rows 2, 3
+  return v;
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
+  using E = Elem<T>;
+  constexpr int H = 2;                // 32-pair halves per step
+  constexpr int TK = 32 * H;          // pairs per step
+  constexpr int NS = 4, L = NS - 1;   // ring stages, steps the loads run ahead
+  constexpr int HALF = 8192;          // dOut tile (32 rows x 128 bytes), then the In tile
+  constexpr int STAGE = H * HALF;
+  constexpr int MAXIT = kWgradMaxPos / 256;
+  __shared__ __attribute__((aligned(16))) char ring[NS * STAGE];
+  __shared__ int lds_o[kWgradMaxPos + TK];
+  __shared__ int lds_i[kWgradMaxPos + TK];
+  __shared__ int wave_cnt[MAXIT][4];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, q = lane >> 4;
+
+  const int kblocks = (p.K + 63) / 64, cblocks = (p.C + 63) / 64;
+  const int per_r = kblocks * cblocks;
+  // units of offset r: its workgroups (ceil(live / QT)) times the channel blocks.  Lane r of every
+  // wave holds offset r's numbers (kv <= 32: one mask bit per offset); a prefix sum over the
+  // lanes and a ballot locate a unit without a loop over memory.
+  const int my_live = lane < p.kv ? p.live_cnt[lane] : 0;
+  const v4i y_rsrc = rsrc_words(p.dout, (uint32_t)p.rows_y * (uint32_t)p.K * 2u);
+  const v4i x_rsrc = rsrc_words(p.inp, (uint32_t)p.rows_x * (uint32_t)p.C * 2u);
+  const int mw = p.mask_width;
+
+  // ---- what does not depend on the unit: which chunk of which row of a stage this lane fetches,
+  // where this lane's transposing reads point
+  const int srow = tid >> 3, schunk = tid & 7;
+  auto swz = [](int row) { return 2 * ((row >> 1) & 3); };
+  const uint32_t ring_at = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_addr(ring) + wave * 1024));
+  int y_rd[2][2], x_rd[2][2];   // [half h][16-channel block of this wave]
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int row = q * 8 + h * 4 + (l16 >> 2);
+      const int ycol = (wm * 2 + j) * 16 + 4 * (l16 & 3), xcol = (wn * 2 + j) * 16 + 4 * (l16 & 3);
+      y_rd[h][j] = row * 128 + (((ycol >> 3) ^ swz(row)) * 16) + (ycol & 7) * 2;
+      x_rd[h][j] = HALF / 2 + row * 128 + (((xcol >> 3) ^ swz(row)) * 16) + (xcol & 7) * 2;
+    }
+
+  // (the address arithmetic above runs while the counts are on their way)
+  const int my_wgs = fast_div(my_live + p.tiles_per_wg - 1, p.tiles_per_wg);
+  const int my_units = my_wgs * per_r;
+  const int incl = wave_prefix_sum_dpp(my_units);
+  const int total_units = __builtin_amdgcn_readlane(incl, 31);
+
+  for (int unit = blockIdx.x; unit < total_units; unit += gridDim.x) {
+    const int r = __builtin_amdgcn_readfirstlane(__builtin_popcountll(__ballot(lane < 32 && incl <= unit)));
+    const int u = unit - __builtin_amdgcn_readlane(incl - my_units, r);
+    const int live = __builtin_amdgcn_readlane(my_live, r);
+    const int n_wg = __builtin_amdgcn_readlane(my_wgs, r);
+    int bx = u, cb = 0, kb = 0;
+    if (per_r > 1) {
+      bx = fast_div(u, per_r);
+      const int rest = u - bx * per_r;
+      kb = fast_div(rest, cblocks);
+      cb = rest - kb * cblocks;
+    }
+    // equal shares of the live tiles: the first live % n_wg workgroups take one more
+    const int share = fast_div(live, n_wg), extra = live - share * n_wg;
+    const int lo = bx * share + (bx < extra ? bx : extra);
+    const int n_list = share + (bx < extra ? 1 : 0);
+    const int n_slots = n_list * mw;  // <= kWgradMaxPos (checked on the host)
+
+    // ---- the (dOut row, In row) pairs of this unit's positions: tile list -> argsort -> pair
+    // table, three dependent loads per position, all positions of the unit at once
+    int o_[MAXIT], i_[MAXIT];
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) {
+      const int s = k * 256 + tid;
+      o_[k] = -1;
+      if (s < n_slots) {
+        const int ti = fast_div(s, mw);
+        const int pos = p.live_list[(int64_t)r * p.num_red + lo + ti] * mw + (s - ti * mw);
+        if (pos < p.n_pos) o_[k] = p.argsort[pos];
+        if (o_[k] >= p.rows_y || o_[k] >= p.n_idx) o_[k] = -1;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) {
+      i_[k] = -1;
+      if (o_[k] >= 0) i_[k] = p.indices[(int64_t)r * p.n_idx + o_[k]];
+      if (i_[k] >= p.rows_x) i_[k] = -1;
+    }
+    // Positions without a pair are dropped: the pairs are packed into the front of the LDS lists
+    // (ballot + prefix counts), so that a sparse offset streams only the rows it has.
+    uint64_t bal[MAXIT];
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) {
+      bal[k] = __ballot(i_[k] >= 0);
+      if (lane == 0) wave_cnt[k][wave] = __builtin_popcountll(bal[k]);
+    }
+    __syncthreads();
+    int n_pairs = 0;
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) {
+      int before = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int c = wave_cnt[k][w];
+        before += w < wave ? c : 0;
+        total += c;
+      }
+      if (i_[k] >= 0) {
+        const int dst = n_pairs + before + __builtin_popcountll(bal[k] & ((1ull << lane) - 1ull));
+        lds_o[dst] = o_[k];
+        lds_i[dst] = i_[k];
+      }
+      n_pairs += total;
+    }
+    if (tid < TK) {   // the last step's empty slots
+      lds_o[n_pairs + tid] = -1;
+      lds_i[n_pairs + tid] = -1;
+    }
+    __syncthreads();
+    const int n_steps = (n_pairs + TK - 1) / TK;
+
+    // ---- stream the pairs, 64 per step, through a ring of NS stages.  Each 32-pair half of a
+    // stage holds the gathered dOut and In rows as they are (row = pair, 128 bytes = this block's 64 channels,
+    // 16-byte chunks XOR-permuted by 2*((row/2)%4) against bank conflicts), written by
+    // direct-to-LDS loads: lane l of wave w fetches one 16-byte chunk of row 8w + l/8, so 8
+    // neighbouring lanes read one row's 128 bytes and the permutation is applied by choosing
+    // which chunk a lane fetches.  An empty slot, a channel past the end and a step past the end
+    // are fetched at an offset outside the buffer: zeros arrive, no memory is touched, and the
+    // number of loads in flight stays the same on every path (the waits below count
+    // instructions).  The MFMA operands need 8 consecutive PAIRS of one channel per lane, i.e.
+    // columns of these tiles: ds_read_b64_tr_b16 delivers them (lane s of a 16-lane group points
+    // at row r0 + s/4, channels 4*(s%4)..; lane i receives rows r0 .. r0+3 of channel i).
+    // Step s waits for its own stage, passes the barrier (everybody's loads of step s have
+    // landed, everybody is done with step s-1), reads its operands, refills the stage of step
+    // s-1 with step s+NS-1, computes.
+    const int ych = kb * 64 + (schunk ^ swz(srow)) * 8, xch = cb * 64 + (schunk ^ swz(srow)) * 8;
+    auto offsets = [&](int t, uint32_t (&yoff)[H], uint32_t (&xoff)[H]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int hh = 0; hh < H; ++hh) {
+        yoff[hh] = 0x80000000u;
+        xoff[hh] = 0x80000000u;
+        if (t < n_steps) {
+          const int o = lds_o[t * TK + hh * 32 + srow], i = lds_i[t * TK + hh * 32 + srow];
+          if (o >= 0) {
+            if (ych < p.K) yoff[hh] = (uint32_t)(o * p.K + ych) * 2u;
+            if (xch < p.C) xoff[hh] = (uint32_t)(i * p.C + xch) * 2u;
+          }
+        }
+      }
+    };
+    auto issue = [&](int t, const uint32_t (&yoff)[H], const uint32_t (&xoff)[H]) __attribute__((always_inline)) {
+      const uint32_t dst = ring_at + (uint32_t)__builtin_amdgcn_readfirstlane((t % NS) * STAGE);
+#pragma unroll
+      for (int hh = 0; hh < H; ++hh) {
+        dma_b128(y_rsrc, dst + hh * HALF, yoff[hh], 0);
+        dma_b128(x_rsrc, dst + hh * HALF + HALF / 2, xoff[hh], 0);
+      }
+    };
+
+    v4f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = v4f{0, 0, 0, 0};
+
+    wait_vmcnt<0>();   // the previous unit's atomics: from here on the counter holds ring loads only
+    uint32_t yn[H], xn[H];
+    for (int t = 0; t < L; ++t) {
+      offsets(t, yn, xn);
+      issue(t, yn, xn);
+    }
+    offsets(L, yn, xn);
+    for (int s = 0; s < n_steps; ++s) {
+      wait_vmcnt<2 * H * (L - 1)>();
+      lds_barrier();
+      typedef short v4s __attribute__((ext_vector_type(4)));
+      typedef __attribute__((address_space(3))) v4s *lds_v4s;
+      const char *base = ring + (s % NS) * STAGE;
+      v4i xf[H][2], yf[H][2];
+#pragma unroll
+      for (int hh = 0; hh < H; ++hh)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const char *hb = base + hh * HALF;
+          const v4s ylo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + y_rd[0][j]));
+          const v4s yhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + y_rd[1][j]));
+          const v4s xlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + x_rd[0][j]));
+          const v4s xhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + x_rd[1][j]));
+          yf[hh][j] = __builtin_bit_cast(v4i, __builtin_shufflevector(ylo, yhi, 0, 1, 2, 3, 4, 5, 6, 7));
+          xf[hh][j] = __builtin_bit_cast(v4i, __builtin_shufflevector(xlo, xhi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      issue(s + L, yn, xn);
+      offsets(s + L + 1, yn, xn);
+#pragma unroll
+      for (int hh = 0; hh < H; ++hh)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) acc[i][j] = E::mfma(yf[hh][i], xf[hh][j], acc[i][j]);
+    }
+    wait_vmcnt<0>();   // the fetches past the end
+
+    // ---- add the partial block into an fp32 image.  dOut is the MFMA row operand, so a lane
+    // holds K indices 4q + x and one C index l16: for a fixed x the 16 lanes of a quarter hit 16
+    // consecutive floats (one 64-byte segment per quarter).  Units that follow each other go to
+    // different images, so that the many units of one offset do not all queue on the same
+    // addresses.
+    if (n_steps > 0) {
+      const int64_t ldn = (int64_t)p.kv * p.C;
+      float *image = p.scratch + (int64_t)(unit % p.images) * p.image_floats;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int nn = cb * 64 + (wn * 2 + j) * 16 + l16;
+          if (nn >= p.C) continue;
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            const int mm = kb * 64 + (wm * 2 + i) * 16 + 4 * q + x;
+            if (mm < p.K)
+              __hip_atomic_fetch_add(image + mm * ldn + (int64_t)r * p.C + nn, acc[i][j][x],
+                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+      }
+    }
+    __syncthreads();   // the LDS lists and the ring are rewritten by the next unit
   }
 }
 
@@ -203,21 +525,32 @@ struct WgradFinalizeParams {
   int32_t C, kv;
   uint32_t mask_filter;
   float alpha, beta;
+  int32_t images;  // copies of the image to sum (each `total` floats, rounded up to 64 floats, apart)
+  int64_t image_floats;
 };
 
-// dW = cvt(alpha * scratch + beta * src) for the offsets enabled in mask_filter
+// dW = cvt(alpha * sum of the scratch images + beta * src) for the offsets enabled in mask_filter
+// Four consecutive elements per thread (C is a multiple of 8, so they share their offset).
 template <class T>
 __global__ __launch_bounds__(256) void wgrad_finalize_kernel(const WgradFinalizeParams p) {
   using E = Elem<T>;
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= p.total) return;
   const int r = (int)((i / p.C) % p.kv);
   if (!((p.mask_filter >> r) & 1u)) return;
-  uint16_t *dw = reinterpret_cast<uint16_t *>(p.dw);
-  const uint16_t *src = reinterpret_cast<const uint16_t *>(p.src);
-  float t = p.beta != 0.0f ? __builtin_fmaf(p.alpha, p.scratch[i], p.beta * E::to_float(src[i]))
-                           : p.alpha * p.scratch[i];
-  dw[i] = E::from_float(t);
+  v4f acc = *reinterpret_cast<const v4f *>(p.scratch + i);
+  for (int g = 1; g < p.images; ++g) acc += *reinterpret_cast<const v4f *>(p.scratch + g * p.image_floats + i);
+  typedef uint16_t v4h __attribute__((ext_vector_type(4)));
+  v4h out;
+  if (p.beta != 0.0f) {
+    const v4h src = *reinterpret_cast<const v4h *>(reinterpret_cast<const uint16_t *>(p.src) + i);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) out[x] = E::from_float(__builtin_fmaf(p.alpha, acc[x], p.beta * E::to_float(src[x])));
+  } else {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) out[x] = E::from_float(p.alpha * acc[x]);
+  }
+  *reinterpret_cast<v4h *>(reinterpret_cast<uint16_t *>(p.dw) + i) = out;
 }
 
 }  // namespace cummhip

@@ -207,6 +207,34 @@ def test_backward_weight_balanced_atomic(dtype, shape, strided):
     assert H.rel_err(got, H.as_f32(cur, dtype)) < TOL
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_backward_weight_balanced_atomic_small_workspace(dtype):
+    """Few channels and many tiles: the two fp32 images that split_k_slices = 2 asks for have no
+    room for the live-tile lists (27 * 94 words > 8 * 8 floats per offset), so the kernel that
+    scans the reduced mask itself runs."""
+    c_in, k_out, mask_width = 8, 8, 32
+    print("case backward_weight_atomic small workspace", dtype, flush=True)
+    rng, coords, pt, feat, w, n_in, n_out = _case(15, 3000, c_in, k_out, dtype)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    red = conv_ref.tile_masks(ms, mask_width)
+    assert 4 * 27 * red.shape[0] > 4 * k_out * 27 * c_in
+    dw0 = H.to_storage(rng.normal(0, 1, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    p = ConvParams(3, ConvOpType.BackwardWeight)
+    p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=True)
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(dw0, dtype), H.dev(dout, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(red, "u32"), H.dev(order, "i32")
+    p.mask_width = mask_width
+    p.split_k_slices = 2
+    p.alpha, p.beta = 1.0, 1.0
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref = conv_ref.implicit_gemm_wgrad_ref(
+        dout, feat, dw0, pt.indices_fwd, red, order, mask_width=mask_width, dtype_dout=dtype,
+        dtype_in=dtype, dtype_w=dtype, alpha=1.0, beta=1.0, split_k_slices=1)
+    assert H.rel_err(H.as_f32(H.host(p.weight), dtype), H.as_f32(ref, dtype)) < TOL
+
+
 @pytest.mark.parametrize("tile", [(64, 64), (128, 128), (64, 128)])
 @pytest.mark.parametrize("strided", [False, True])
 def test_int8_inference_bit_exact(tile, strided):

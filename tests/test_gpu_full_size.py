@@ -77,6 +77,31 @@ def test_subm_f16_c64_forward_dgrad_full_size(tile_m):
     assert H.rel_err(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_d, dtype)) < TOL
 
 
+def test_subm_f16_c64_wgrad_full_size():
+    """Backward-weight at the benchmark size with the balanced descriptor and split_k_slices = 32
+    (eight fp32 images), on the reduced masks that the forward pass writes."""
+    print("case full size subm f16 wgrad", flush=True)
+    dtype, tile_m = "f16", 64
+    rng, pt, feat, w, n = _subm_case(20240607, 120000, dtype, 64, 64)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    red = conv_ref.tile_masks(ms, tile_m)
+    dout = H.to_storage(rng.normal(0, 1, size=(n, 64)).astype(np.float32), dtype)
+    dw0 = np.zeros((64, 27, 64), np.float16)
+    p = ConvParams(3, ConvOpType.BackwardWeight)
+    p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=True)
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(dw0, dtype), H.dev(dout, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(red, "u32"), H.dev(order, "i32")
+    p.mask_width = tile_m
+    p.split_k_slices = 32
+    for _ in range(2):   # the second call finds the workspace of the first
+        ConvMainUnitTest.implicit_gemm2(p)
+    ref = conv_ref.implicit_gemm_wgrad_ref(
+        dout, feat, dw0, pt.indices_fwd, red, order, mask_width=tile_m, dtype_dout=dtype,
+        dtype_in=dtype, dtype_w=dtype, split_k_slices=1)
+    assert H.rel_err(H.as_f32(H.host(p.weight), dtype), H.as_f32(ref, dtype)) < TOL
+
+
 def test_s8_stride2_full_size_bit_exact():
     print("case full size s8 stride 2", flush=True)
     rng = np.random.default_rng(20240611)
