@@ -18,7 +18,11 @@ LIB = os.path.join(HERE, "libcummhip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-inline-asm"]   # the direct-to-LDS loads set M0 themselves
+         "-Wno-inline-asm",   # the direct-to-LDS loads set M0 themselves
+         # MFMA accumulators in ordinary VGPRs: with AGPR accumulators the multi-exit step loops
+         # copy every accumulator AGPR -> VGPR -> AGPR once per trip (a quarter of the loop's
+         # vector instructions in the 64x128 kernels)
+         "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 ELEMS = [("F16", "f16"), ("BF16", "bf16"), ("S8", "s8")]
 
