@@ -160,19 +160,33 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   auto swz = [](int row) { return ((row * KS) >> 2) & (LPR - 1); };
   const bool has_gather = p.gather != nullptr;
   // entries: lane l < RPW fetches the entry of tile row wave*RPW + l
+  // A row takes part in kernel offset k only if its own mask word has the bit (the word is
+  // what the pair table was built from: bit clear = entry -1).  Entries and rows of the others
+  // are not fetched at all: the 4-byte entries are scattered over the table, one memory sector
+  // each, and on sparse offsets most rows of a tile have none.
+  auto row_bits = [&](int pos) -> uint32_t {
+    if (p.mask == nullptr) return ~0u;
+    uint32_t w = pos < p.n_pos ? p.mask[pos] : 0u;
+    if (p.reverse_mask) w = __builtin_bitreverse32(w) >> (32 - p.kv);
+    return w;
+  };
   uint32_t key_off = kOob;
+  uint32_t key_bits = 0;
   {
     const int pos = pos_base + wave * RPW + lane;
     int key = -1;
     if (lane < RPW && pos < p.n_pos) key = p.gather_by_pos ? pos : (p.out_rows ? p.out_rows[pos] : pos);
     if (key >= 0 && key < p.n_idx) key_off = (uint32_t)key * 4u;
+    if (lane < RPW) key_bits = row_bits(pos);
   }
   int a_key[IPA];          // without a pair table the gathered row is the key itself
   uint32_t a_col[IPA];     // byte offset of the fetched chunk inside the gathered row, or kOob
+  uint32_t a_bits[IPA];    // mask word of the row
 #pragma unroll
   for (int t = 0; t < IPA; ++t) {
     const int r = (wave * IPA + t) * RPI + lrow;
     const int pos = pos_base + r;
+    a_bits[t] = row_bits(pos);
     int key = -1;
     if (pos < p.n_pos) key = p.gather_by_pos ? pos : (p.out_rows ? p.out_rows[pos] : pos);
     a_key[t] = key >= 0 && key < p.n_idx ? key : -1;
@@ -270,7 +284,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   auto issue_idx = [&](int j, int *slot) {
     const int k = __builtin_amdgcn_readlane(klist, j);
     const v4i rs = rsrc_words(p.gather, k >= 0 ? g_bytes : 0u);
-    dma_b32(rs, lds_addr(slot), key_off, (uint32_t)k * g_k_bytes);
+    dma_b32(rs, lds_addr(slot), (key_bits >> (k & 31)) & 1u ? key_off : kOob, (uint32_t)k * g_k_bytes);
   };
   // entries of this lane's rows out of the wave's slot (its own loads: no barrier needed)
   auto read_idx = [&](const int *slot, int (&dst)[IPA]) {
@@ -286,7 +300,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       // a_col is out of range already for a row without a key or a chunk past the contraction;
       // adding a row offset below 2 GiB keeps it out of range
       const uint32_t v = (uint32_t)src[t];
-      const uint32_t voff = v < (uint32_t)p.rows_a ? v * a_row_bytes + a_col[t] : kOob;
+      const uint32_t voff = v < (uint32_t)p.rows_a && ((a_bits[t] >> (k & 31)) & 1u) ? v * a_row_bytes + a_col[t] : kOob;
       dma_b128(rs_a, lds_addr(st + (wave * IPA + t) * 64), voff, 0u);
     }
     const uint32_t soff = (uint32_t)k * w_k_bytes;   // k = -1 comes with zero records
