@@ -9,7 +9,8 @@
 //     (one request per 64-byte segment), and the data lands in LDS without passing registers
 //     (buffer_load ... lds writes lane l of the instruction at M0 + 16*l);
 //   * the LDS image of a tile is row-major with the 16-byte chunks of a row XOR-permuted by
-//     swz(row) = (row*KS/4) mod 4*KS.  The permutation is applied on the global side (a lane picks
+//     swz(row) = (row*KS/4) mod 4*KS ((row/2) mod 4 for 64-byte rows, two of which share a
+//     128-byte line of banks).  The permutation is applied on the global side (a lane picks
 //     which chunk of its row it fetches), which keeps the global access coalesced, and makes the
 //     MFMA-layout reads (16 lanes = 16 rows, same chunk) hit 16 different bank groups;
 //   * the weight tile is stored in the row order the MFMA fragments want (LDS row wn*NBW*16 +
@@ -157,7 +158,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   // ---- loader role of this lane: rows of the tile it fetches, weight rows it fetches
   const int lrow = lane / LPR;             // row inside a load instruction
   const int lchunk = lane % LPR;           // LDS chunk slot inside the row
-  auto swz = [](int row) { return ((row * KS) >> 2) & (LPR - 1); };
+  auto swz = [](int row) { return KS == 1 ? (row >> 1) & 3 : ((row * KS) >> 2) & (LPR - 1); };
   const bool has_gather = p.gather != nullptr;
   // entries: lane l < RPW fetches the entry of tile row wave*RPW + l
   // A row takes part in kernel offset k only if its own mask word has the bit (the word is

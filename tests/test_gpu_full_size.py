@@ -150,3 +150,24 @@ def test_gather_gemm_scatter_full_size():
     assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
     untouched = np.setdiff1d(np.arange(rows), c_inds)
     np.testing.assert_array_equal(H.host(p.c)[untouched], c0[untouched])   # rows not in c_inds stay as they were
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(2000, 1544, 512, 0.0), (2048, 2048, 1024, 1.0), (3000, 1000, 192, 0.5)])
+def test_dense_gemm_large(dtype, shape):
+    """Plain matmul2 with A [m, k] and B [n, k] at sizes that select the LDS-ring GEMM kernel:
+    ragged m and n, accumulation into C, against a float32 matrix product of the stored values."""
+    m, n, k, beta = shape
+    print("case dense gemm", dtype, shape, flush=True)
+    rng = np.random.default_rng(20240613)
+    a = H.to_storage(rng.normal(0, 1, size=(m, k)).astype(np.float32), dtype)
+    b = H.to_storage(rng.normal(0, 0.1, size=(n, k)).astype(np.float32), dtype)
+    c0 = H.to_storage(rng.normal(0, 1, size=(m, n)).astype(np.float32), dtype)
+    p = GemmParams()
+    p.algo_desp = H.find_gemm_desp(dtype, ShuffleStrideType.NoShuffle, 128, 128, False, True)
+    p.a, p.b, p.c = H.dev(a, dtype), H.dev(b, dtype), H.dev(c0, dtype)
+    p.alpha, p.beta = 1.0, beta
+    GemmMainUnitTest.matmul2(p)
+    ref = gemm_ref.matmul2_ref(a, b, c0, dtype_a=dtype, dtype_b=dtype, dtype_c=dtype, trans_b=True,
+                               alpha=1.0, beta=beta)
+    assert H.rel_err(H.as_f32(H.host(p.c), dtype), H.as_f32(ref, dtype)) < TOL
