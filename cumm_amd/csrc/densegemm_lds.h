@@ -22,17 +22,18 @@
 
 namespace cummhip {
 
-template <class T, int RBW, int NBW, int KS, int NS>
-__global__ __launch_bounds__(256) void densegemm_lds_kernel(const TileGemmParams p, int tiles_m, int tiles_n) {
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS>
+__global__ __launch_bounds__(WM *WN * 64) void densegemm_lds_kernel(const TileGemmParams p, int tiles_m, int tiles_n) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
-  constexpr int TM = 2 * RBW * 16;
-  constexpr int TN = 2 * NBW * 16;
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = WM * RBW * 16;
+  constexpr int TN = WN * NBW * 16;
   constexpr int PV = E::kPerVec;
   constexpr int LPR = 4 * KS;              // 16-byte chunks per row and step
   constexpr int RPI = 64 / LPR;            // rows per load instruction
-  constexpr int IPY = TM * LPR / 256;      // load instructions per wave and step
-  constexpr int IPX = TN * LPR / 256;
+  constexpr int IPY = TM * LPR / NT;       // load instructions per wave and step
+  constexpr int IPX = TN * LPR / NT;
   static_assert(IPY >= 1 && IPX >= 1, "tile too small for the workgroup");
   constexpr int Y_V = TM * LPR;            // 16-byte vectors of the Y part of a stage
   constexpr int STAGE_V = (TM + TN) * LPR;
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(256) void densegemm_lds_kernel(const TileGemmParams
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WN, wn = wave % WN;
   const int m = lane & 15, q = lane >> 4;
 
   // ---- tile of this workgroup

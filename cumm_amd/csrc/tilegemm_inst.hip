@@ -18,31 +18,38 @@ static hipError_t launch_xy(bool xk, bool yk, const TileGemmParams &p, dim3 grid
 }
 
 // Plain GEMM with both operands contiguous along the contraction, two-byte elements, shapes
-// the LDS-ring kernel takes without a remainder in k and with 16-byte output
-// pieces: the LDS-ring kernel; its result does not depend on the tile (one fp32 sum over k in
-// ascending order per element either way).
+// the LDS-ring kernel takes without a remainder in k and with 16-byte output pieces.  Its result
+// does not depend on the tile (one fp32 sum over k in ascending order per element either way).
+// Measured on 4096^3 f16 (TFLOP/s): 256 x 256 x 32 per step with 2 x 4 waves of 128 x 64 and
+// three stages 1089, the same with 4 x 2 waves of 64 x 128 954, with four stages 1066, with 64
+// per step and two stages 1011; 128 x 128 x 64 with 2 x 2 waves and two stages 966; 256 x 128 x 32
+// with three stages 902; the register-staged kernel 583.
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS>
+static hipError_t launch_dense_ring_as(const TileGemmParams &p, hipStream_t s) {
+  constexpr int TM = WM * RBW * 16, TN = WN * NBW * 16;
+  const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
+  hipLaunchKernelGGL((densegemm_lds_kernel<T, WM, WN, RBW, NBW, KS, NS>), dim3((unsigned)(tiles_m * tiles_n)),
+                     dim3(WM * WN * 64), 0, s, p, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
 template <class T>
 static bool launch_dense_ring(const TileGemmParams &p, hipStream_t s, hipError_t *err) {
   if constexpr (Elem<T>::kBytes != 2) {
     return false;
   } else {
-    // 128 x 128 x 64 per step, two stages (64 KB of LDS, two workgroups per CU): the best of
-    // the shapes tried on 4096^3 (966 TFLOP/s; 256 x 128 x 32 with three stages 902, 128 x 256
-    // 895, 256 x 256 x 32 with four stages 813, all against 583 for the register-staged kernel)
-    constexpr int RBW = 4, NBW = 4, KS = 2, NS = 2;
-    constexpr int TM = 2 * RBW * 16, TN = 2 * NBW * 16, BK = KS * 32;
     const auto al16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool ok = p.kv == 1 && p.split_k == 1 && !p.x_gather && !p.y_gather && !p.red_mask &&
-                    p.k >= BK && p.k % BK == 0 && p.n % 8 == 0 && p.ldx % 8 == 0 && p.ldy % 8 == 0 &&
+                    p.k >= 64 && p.k % 64 == 0 && p.n % 8 == 0 && p.ldx % 8 == 0 && p.ldy % 8 == 0 &&
                     p.ldc % 8 == 0 && p.ldd % 8 == 0 && al16(p.X) && al16(p.Y) && al16(p.C) && al16(p.D) &&
-                    (int64_t)p.m * p.n >= (int64_t)TM * TN * 64 &&
                     ((int64_t)(p.m - 1) * p.ldy + p.k) * 2 < ((int64_t)1 << 31) &&
                     ((int64_t)(p.n - 1) * p.ldx + p.k) * 2 < ((int64_t)1 << 31);
     if (!ok) return false;
-    const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
-    hipLaunchKernelGGL((densegemm_lds_kernel<T, RBW, NBW, KS, NS>), dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0,
-                       s, p, tiles_m, tiles_n);
-    *err = hipGetLastError();
+    const int64_t big_tiles = (int64_t)((p.m + 255) / 256) * ((p.n + 255) / 256);
+    const int64_t mid_tiles = (int64_t)((p.m + 127) / 128) * ((p.n + 127) / 128);
+    if (big_tiles >= 256) *err = launch_dense_ring_as<T, 2, 4, 8, 4, 1, 3>(p, s);       // a tile per CU at least
+    else if (mid_tiles >= 64) *err = launch_dense_ring_as<T, 2, 2, 4, 4, 2, 2>(p, s);
+    else return false;
     return true;
   }
 }

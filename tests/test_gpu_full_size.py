@@ -153,10 +153,12 @@ def test_gather_gemm_scatter_full_size():
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("shape", [(2000, 1544, 512, 0.0), (2048, 2048, 1024, 1.0), (3000, 1000, 192, 0.5)])
+@pytest.mark.parametrize("shape", [(2000, 1544, 512, 0.0), (2048, 2048, 1024, 1.0), (3000, 1000, 192, 0.5),
+                                   (4100, 4104, 128, 1.0)])
 def test_dense_gemm_large(dtype, shape):
     """Plain matmul2 with A [m, k] and B [n, k] at sizes that select the LDS-ring GEMM kernel:
-    ragged m and n, accumulation into C, against a float32 matrix product of the stored values."""
+    ragged m and n, accumulation into C, against a float32 matrix product of the stored values
+    (the last shape has a 256 x 256 tile per CU and takes the 8-wave variant)."""
     m, n, k, beta = shape
     print("case dense gemm", dtype, shape, flush=True)
     rng = np.random.default_rng(20240613)
