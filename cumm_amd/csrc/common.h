@@ -81,12 +81,22 @@ __device__ __forceinline__ float apply_act(float x, int act, float act_alpha) {
 // float -> s8: clamp to [-128,127] then round half to even; NaN -> 0
 // (Int8Inference clamp + cvt.rni.sat.s8.f32, cumm/gemm/output_op/linear.py:327-351,
 //  include/tensorview/gemm/math/numeric_convert.h:171-192 of the reference)
+// Three instructions: round half to even, convert (the hardware conversion saturates and turns
+// NaN into 0; written as asm because the C cast is undefined out of range), clamp the integer.
+// Clamping after the rounding equals clamping before it: the bounds are integers.
 __device__ __forceinline__ int f32_to_s8(float t) {
-  if (t < -128.0f) t = -128.0f;
-  if (t > 127.0f) t = 127.0f;
-  float q = __builtin_rintf(t);
-  if (q != q) q = 0.0f;
-  return (int)q;
+  const float q = __builtin_rintf(t);
+  int i;
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(i) : "v"(q));
+  i = i > 127 ? 127 : i;
+  return i < -128 ? -128 : i;
+}
+
+// low bytes of four integers as one dword (three v_perm_b32)
+__device__ __forceinline__ int pack4_bytes(int b0, int b1, int b2, int b3) {
+  const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b1, (uint32_t)b0, 0x0c0c0400u);
+  const uint32_t hi = __builtin_amdgcn_perm((uint32_t)b3, (uint32_t)b2, 0x0c0c0400u);
+  return (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
 }
 
 __device__ __forceinline__ uint32_t wave_or(uint32_t v) {

@@ -122,28 +122,6 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   const int n0 = blockIdx.y * TN;
   const int pos_base = tile * TM;
 
-  // requantisation scale and bias of this lane's output channels (one-byte outputs): requested
-  // now, used in the epilogue; without the int8 epilogue the descriptors have no records
-  float scale_v[E::kBytes == 1 ? 4 * NBW : 1], bias_v[E::kBytes == 1 ? 4 * NBW : 1];
-  if constexpr (E::kBytes == 1) {
-    const uint32_t sb_bytes = p.int8_epilogue ? (uint32_t)p.k_out * 4u : 0u;
-    const __amdgpu_buffer_rsrc_t rs_scale = make_rsrc(p.scale, sb_bytes);
-    const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(p.bias, sb_bytes);
-    const uint32_t off = (uint32_t)(n0 + wn * (NBW * 16) + q * (4 * NBW)) * 4u;
-#pragma unroll
-    for (int g = 0; g < NBW; ++g) {
-      // (whole-vector casts: a per-element cast of the loaded vector was seen to be compiled
-      // into a load of element 0 only)
-      const v4f sv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_scale, off + g * 16, 0, 0));
-      const v4f bv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_bias, off + g * 16, 0, 0));
-#pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        scale_v[g * 4 + x] = sv[x];
-        bias_v[g * 4 + x] = bv[x];
-      }
-    }
-  }
-
   // ---- the tile's mask words are requested first and reduced only after the row keys below have
   // been requested too: one memory round trip for both
   uint32_t mk = 0;
@@ -213,6 +191,29 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       w_voff[t] = e < p.c_in && n < p.k_out
                       ? (uint32_t)(((int64_t)e * p.w_stride_c + n) * E::kBytes)
                       : kOob;
+    }
+  }
+
+  // requantisation scale and bias of this lane's output channels (one-byte outputs): requested
+  // behind the masks and keys (nothing waits for them before the epilogue); without the int8
+  // epilogue the descriptors have no records
+  float scale_v[E::kBytes == 1 ? 4 * NBW : 1], bias_v[E::kBytes == 1 ? 4 * NBW : 1];
+  if constexpr (E::kBytes == 1) {
+    const uint32_t sb_bytes = p.int8_epilogue ? (uint32_t)p.k_out * 4u : 0u;
+    const __amdgpu_buffer_rsrc_t rs_scale = make_rsrc(p.scale, sb_bytes);
+    const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(p.bias, sb_bytes);
+    const uint32_t off = (uint32_t)(n0 + wn * (NBW * 16) + q * (4 * NBW)) * 4u;
+#pragma unroll
+    for (int g = 0; g < NBW; ++g) {
+      // (whole-vector casts: a per-element cast of the loaded vector was seen to be compiled
+      // into a load of element 0 only)
+      const v4f sv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_scale, off + g * 16, 0, 0));
+      const v4f bv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_bias, off + g * 16, 0, 0));
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        scale_v[g * 4 + x] = sv[x];
+        bias_v[g * 4 + x] = bv[x];
+      }
     }
   }
 
@@ -469,7 +470,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
         }
         const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
         vNi outv;
-        int8_t *ob = reinterpret_cast<int8_t *>(&outv);
+        int ob[CPLW];
 #pragma unroll
         for (int x = 0; x < CPLW; ++x) {
           const int a = acc[rb][x >> 2][x & 3];
@@ -483,8 +484,10 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
             t = p.alpha * (float)a;
           }
           t = apply_act(t, ACT, p.act_alpha);
-          ob[x] = (int8_t)f32_to_s8(t);
+          ob[x] = f32_to_s8(t);
         }
+#pragma unroll
+        for (int g = 0; g < ND; ++g) outv[g] = pack4_bytes(ob[4 * g], ob[4 * g + 1], ob[4 * g + 2], ob[4 * g + 3]);
         if constexpr (ND == 4) __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
         else __builtin_amdgcn_raw_buffer_store_b64(outv, rs_c, coff, 0, 0);
       }
