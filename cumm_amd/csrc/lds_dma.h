@@ -51,6 +51,18 @@ __device__ __forceinline__ void dma_b32(v4i rsrc, uint32_t lds, uint32_t voff, u
                :: "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
 }
 
+// A 4-byte buffer load into a register that the compiler does not see as a load: it cannot sink it
+// into a branch (a plain load that feeds only a select is moved behind the select's condition and
+// then waited for there, one round trip per conditional value).  To the compiler the result exists
+// at once: the caller waits by hand (wait_vmcnt) and names the register in keep_after_wait() before
+// the first use, which also keeps the register allocated while the load is in flight.
+__device__ __forceinline__ int load_b32_hidden(v4i rsrc, uint32_t voff) {
+  int r;
+  asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  return r;
+}
+__device__ __forceinline__ void keep_after_wait(int &r) { asm volatile("" : "+v"(r)); }
+
 // Workgroup barrier without the fence of __syncthreads(): the fence would wait for every
 // outstanding direct-to-LDS load, i.e. also for the stages that are being prefetched.  The empty
 // asm statements keep the compiler from moving LDS accesses across the barrier; the caller waits
