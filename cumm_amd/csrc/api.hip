@@ -462,7 +462,8 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
     int images = 0;
     for (int s = 8; s >= 1 && !images; s >>= 1)
       if (s <= a->split_k_slices && a->workspace_bytes >= s * image_bytes + lists_bytes) images = s;
-    const bool fits32 = (int64_t)a->rows_out * a->K * 2 < (int64_t)1 << 31 && (int64_t)a->rows_in * a->C * 2 < (int64_t)1 << 31;
+    const bool fits32 = (int64_t)a->rows_out * a->K * 2 < (int64_t)1 << 31 && (int64_t)a->rows_in * a->C * 2 < (int64_t)1 << 31 &&
+                        (int64_t)kv * a->N * 4 < (int64_t)1 << 31;
     WgradPrepareParams pre;
     std::memset(&pre, 0, sizeof(pre));
     w.images = f.images = 1;

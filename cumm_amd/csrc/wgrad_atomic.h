@@ -311,6 +311,9 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   // wave holds offset r's numbers (kv <= 32: one mask bit per offset); a prefix sum over the
   // lanes and a ballot locate a unit without a loop over memory.
   const int my_live = lane < p.kv ? p.live_cnt[lane] : 0;
+  const v4i rs_list = rsrc_words(p.live_list, (uint32_t)p.kv * (uint32_t)p.num_red * 4u);
+  const v4i rs_sort = rsrc_words(p.argsort, (uint32_t)p.n_pos * 4u);
+  const v4i rs_idx = rsrc_words(p.indices, (uint32_t)p.kv * (uint32_t)p.n_idx * 4u);
   const v4i y_rsrc = rsrc_words(p.dout, (uint32_t)p.rows_y * (uint32_t)p.K * 2u);
   const v4i x_rsrc = rsrc_words(p.inp, (uint32_t)p.rows_x * (uint32_t)p.C * 2u);
   const int mw = p.mask_width;
@@ -356,25 +359,42 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     const int n_slots = n_list * mw;  // <= kWgradMaxPos (checked on the host)
 
     // ---- the (dOut row, In row) pairs of this unit's positions: tile list -> argsort -> pair
-    // table, three dependent loads per position, all positions of the unit at once
-    int o_[MAXIT], i_[MAXIT];
+    // table, three dependent loads per position, all positions of the unit at once.  Each level
+    // is issued for all positions as hidden buffer loads (a position past the end reads 0
+    // through the descriptor and is sorted out with a select) and waited for once: as
+    // conditional C++ loads every one of the twelve got a branch and a wait of its own.
+    int t_[MAXIT], o_[MAXIT], i_[MAXIT], within[MAXIT];
 #pragma unroll
     for (int k = 0; k < MAXIT; ++k) {
       const int s = k * 256 + tid;
-      o_[k] = -1;
-      if (s < n_slots) {
-        const int ti = fast_div(s, mw);
-        const int pos = p.live_list[(int64_t)r * p.num_red + lo + ti] * mw + (s - ti * mw);
-        if (pos < p.n_pos) o_[k] = p.argsort[pos];
-        if (o_[k] >= p.rows_y || o_[k] >= p.n_idx) o_[k] = -1;
-      }
+      const int ti = fast_div(s, mw);
+      within[k] = s - ti * mw;
+      t_[k] = load_b32_hidden(rs_list, s < n_slots ? (uint32_t)(r * p.num_red + lo + ti) * 4u : 0x80000000u);
     }
+    wait_vmcnt<0>();   // (also the previous unit's atomics)
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) keep_after_wait(t_[k]);
+    bool have[MAXIT];
 #pragma unroll
     for (int k = 0; k < MAXIT; ++k) {
-      i_[k] = -1;
-      if (o_[k] >= 0) i_[k] = p.indices[(int64_t)r * p.n_idx + o_[k]];
-      if (i_[k] >= p.rows_x) i_[k] = -1;
+      const int pos = t_[k] * mw + within[k];
+      have[k] = k * 256 + tid < n_slots && pos < p.n_pos;
+      o_[k] = load_b32_hidden(rs_sort, have[k] ? (uint32_t)pos * 4u : 0x80000000u);
     }
+    wait_vmcnt<0>();
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) keep_after_wait(o_[k]);
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) {
+      const int o = o_[k];
+      o_[k] = have[k] && o >= 0 && o < p.rows_y && o < p.n_idx ? o : -1;
+      i_[k] = load_b32_hidden(rs_idx, o_[k] >= 0 ? (uint32_t)(r * p.n_idx + o_[k]) * 4u : 0x80000000u);
+    }
+    wait_vmcnt<0>();
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) keep_after_wait(i_[k]);
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k) i_[k] = o_[k] >= 0 && i_[k] < p.rows_x ? i_[k] : -1;
     // Positions without a pair are dropped: the pairs are packed into the front of the LDS lists
     // (ballot + prefix counts), so that a sparse offset streams only the rows it has.
     uint64_t bal[MAXIT];
