@@ -461,12 +461,15 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
     const size_t lists_bytes = 128 + sizeof(int32_t) * (size_t)kv * w.num_red;
     int images = 0;
     for (int s = 8; s >= 1 && !images; s >>= 1)
-      if (s <= a->split_k_slices && a->workspace_bytes >= s * image_bytes + lists_bytes) images = s;
+      if (s <= a->split_k_slices && a->workspace_bytes >= s * image_bytes + lists_bytes &&
+          (uint64_t)s * image_bytes < ((uint64_t)1 << 32))   // (the finalize kernel reads them through one descriptor)
+        images = s;
     const bool fits32 = (int64_t)a->rows_out * a->K * 2 < (int64_t)1 << 31 && (int64_t)a->rows_in * a->C * 2 < (int64_t)1 << 31 &&
                         (int64_t)kv * a->N * 4 < (int64_t)1 << 31;
     WgradPrepareParams pre;
     std::memset(&pre, 0, sizeof(pre));
     w.images = f.images = 1;
+    w.image_floats = f.image_floats = (int64_t)(image_bytes / sizeof(float));
     // (the unit-walking kernel divides unit numbers with a float reciprocal: exact below 2^22)
     const int64_t unit_bound = ((int64_t)(w.num_red + qt - 1) / qt + 1) * kv * (((int64_t)a->K + 63) / 64) * (((int64_t)a->C + 63) / 64);
     if (images && fits32 && unit_bound < ((int64_t)1 << 22) && w.num_red < (1 << 22)) {

@@ -237,17 +237,22 @@ static __global__ __launch_bounds__(256) void wgrad_prepare_kernel(const WgradPr
   const bool on = (p.mask_filter >> r) & 1u;
   int base = 0;
   constexpr int U = 8;   // mask words a thread has in flight
+  const v4i rs_red = rsrc_words(p.red_mask, (uint32_t)p.num_red * 4u);
   for (int t0 = 0; t0 < p.num_red; t0 += 256 * U) {
-    uint32_t m[U];
+    // (hidden loads, one wait: as conditional loads each of the U got a branch and a wait)
+    int m[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = t0 + u * 256 + tid;
-      m[u] = t < p.num_red ? p.red_mask[t] : 0u;
+      m[u] = load_b32_hidden(rs_red, t < p.num_red ? (uint32_t)t * 4u : 0x80000000u);
     }
+    wait_vmcnt<0>();
+#pragma unroll
+    for (int u = 0; u < U; ++u) keep_after_wait(m[u]);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = t0 + u * 256 + tid;
-      const bool live = on && ((m[u] >> r) & 1u);
+      const bool live = on && (((uint32_t)m[u] >> r) & 1u);
       const uint64_t bal = __ballot(live);
       if (lane == 0) wave_cnt[u & 1][wave] = __builtin_popcountll(bal);
       __syncthreads();   // the other set of counters is free again: everybody passed the previous barrier
@@ -558,8 +563,18 @@ __global__ __launch_bounds__(256) void wgrad_finalize_kernel(const WgradFinalize
   if (i >= p.total) return;
   const int r = (int)((i / p.C) % p.kv);
   if (!((p.mask_filter >> r) & 1u)) return;
-  v4f acc = *reinterpret_cast<const v4f *>(p.scratch + i);
-  for (int g = 1; g < p.images; ++g) acc += *reinterpret_cast<const v4f *>(p.scratch + g * p.image_floats + i);
+  // up to 8 images, all requested at once (a loop over p.images would wait for each): images
+  // past the count are read at an offset outside the descriptor and arrive as zeros
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(p.scratch), 0, (int)((uint32_t)p.images * (uint32_t)p.image_floats * 4u), 0x00020000);
+  v4f part[8];
+#pragma unroll
+  for (int g = 0; g < 8; ++g)
+    part[g] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+        rs, g < p.images ? (uint32_t)((int64_t)g * p.image_floats + i) * 4u : 0x80000000u, 0, 0));
+  v4f acc = part[0];
+#pragma unroll
+  for (int g = 1; g < 8; ++g) acc += part[g];
   typedef uint16_t v4h __attribute__((ext_vector_type(4)));
   v4h out;
   if (p.beta != 0.0f) {
