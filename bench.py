@@ -31,8 +31,8 @@ from cumm_amd.tensorview.gemm import (ConvOpType, ConvParams, GemmParams,  # noq
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per forward launch of the default workload (tile_m = 64), from two rocprofv3 --pmc runs
 # (FETCH_SIZE scaled by the factor 2.000 a copy kernel of known size gives on this part, plus
-# WRITE_SIZE): 2.000 * 16383.6 KiB + 15057.0 KiB.  The counter runs are offline; this is their result.
-MEASURED_TRAFFIC_BYTES = 48971981
+# WRITE_SIZE): 2.000 * 16854.4 KiB + 15057.1 KiB.  The counter runs are offline; this is their result.
+MEASURED_TRAFFIC_BYTES = 49936282
 PEAK_MFMA_F16_TFLOPS = 2516.6
 PEAK_MFMA_I8_TOPS = 5033.2
 GRID = (41, 1600, 1408)
