@@ -154,6 +154,29 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb)
     raw_o_row[rb] = load_b32_hidden(rsw_rows, pos_off(pos_base + (wm * RBW + rb) * 16 + m));
+  // requantisation scale and bias of this lane's output channels (one-byte outputs): requested
+  // behind the masks and keys and landing with them; without the int8 epilogue the descriptors
+  // have no records
+  float scale_v[E::kBytes == 1 ? 4 * NBW : 1], bias_v[E::kBytes == 1 ? 4 * NBW : 1];
+  if constexpr (E::kBytes == 1) {
+    const uint32_t sb_bytes = p.int8_epilogue ? (uint32_t)p.k_out * 4u : 0u;
+    const __amdgpu_buffer_rsrc_t rs_scale = make_rsrc(p.scale, sb_bytes);
+    const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(p.bias, sb_bytes);
+    const uint32_t off = (uint32_t)(n0 + wn * (NBW * 16) + q * (4 * NBW)) * 4u;
+#pragma unroll
+    for (int g = 0; g < NBW; ++g) {
+      // (whole-vector casts: a per-element cast of the loaded vector was seen to be compiled
+      // into a load of element 0 only)
+      const v4f sv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_scale, off + g * 16, 0, 0));
+      const v4f bv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_bias, off + g * 16, 0, 0));
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        scale_v[g * 4 + x] = sv[x];
+        bias_v[g * 4 + x] = bv[x];
+      }
+    }
+  }
+
   wait_vmcnt<0>();
 #pragma unroll
   for (int i = 0; i < MKW; ++i) keep_after_wait(raw_mk[i]);
@@ -194,6 +217,46 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     key_off = key >= 0 && key < p.n_idx ? (uint32_t)key * 4u : kOob;
     key_bits = lane < RPW ? row_bits(raw_key_bits) : 0u;
   }
+  // ---- tile mask: OR over the tile's positions (cumm/conv/kernel.py:844-889 of the reference)
+  uint32_t kmask = 1u;
+  if (has_mask) {
+    kmask = wave_or_dpp(mk) & p.mask_filter;
+    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
+    if (p.exit_on_empty && kmask == 0) return;
+    if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
+    if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
+  }
+  const int n_steps = __builtin_popcount(kmask);
+
+
+  const uint32_t g_k_bytes = (uint32_t)p.n_idx * 4u;
+  const uint32_t g_bytes = has_gather ? p.gather_bytes : 0u;
+
+  // lane j of klist holds the j-th kernel offset of the tile (-1 past the end): lane b pushes
+  // b+1 to the lane of its rank among the set bits, lanes without a bit push into lane 63, which
+  // nobody reads; a lane nobody pushed to reads 0.
+  int klist;
+  {
+    const bool bit = lane < 32 && ((kmask >> lane) & 1u);
+    const int rank = __builtin_popcount(kmask & ((1u << (lane & 31)) - 1u));
+    klist = __builtin_amdgcn_ds_permute(bit ? rank * 4 : 63 * 4, bit ? lane + 1 : 0) - 1;
+  }
+
+  auto issue_idx = [&](int j, int *slot) {
+    const int k = __builtin_amdgcn_readlane(klist, j);
+    const v4i rs = rsrc_words(p.gather, k >= 0 ? g_bytes : 0u);
+    dma_b32(rs, lds_addr(slot), (key_bits >> (k & 31)) & 1u ? key_off : kOob, (uint32_t)k * g_k_bytes);
+  };
+  // The entries of the first offsets are requested now; the address work below (row chunks, weight
+  // rows, fragment slots) overlaps their round trip.
+  if (n_steps > 0) {
+    auto first = [&](auto jc) -> bool {
+      issue_idx(decltype(jc)::value, idx_slot(jc));
+      return false;
+    };
+    run_steps(first, std::make_integer_sequence<int, DI>{});
+  }
+
   int a_key[IPA];          // without a pair table the gathered row is the key itself
   uint32_t a_col[IPA];     // byte offset of the fetched chunk inside the gathered row, or kOob
   uint32_t a_bits[IPA];    // mask word of the row
@@ -230,29 +293,6 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     }
   }
 
-  // requantisation scale and bias of this lane's output channels (one-byte outputs): requested
-  // behind the masks and keys (nothing waits for them before the epilogue); without the int8
-  // epilogue the descriptors have no records
-  float scale_v[E::kBytes == 1 ? 4 * NBW : 1], bias_v[E::kBytes == 1 ? 4 * NBW : 1];
-  if constexpr (E::kBytes == 1) {
-    const uint32_t sb_bytes = p.int8_epilogue ? (uint32_t)p.k_out * 4u : 0u;
-    const __amdgpu_buffer_rsrc_t rs_scale = make_rsrc(p.scale, sb_bytes);
-    const __amdgpu_buffer_rsrc_t rs_bias = make_rsrc(p.bias, sb_bytes);
-    const uint32_t off = (uint32_t)(n0 + wn * (NBW * 16) + q * (4 * NBW)) * 4u;
-#pragma unroll
-    for (int g = 0; g < NBW; ++g) {
-      // (whole-vector casts: a per-element cast of the loaded vector was seen to be compiled
-      // into a load of element 0 only)
-      const v4f sv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_scale, off + g * 16, 0, 0));
-      const v4f bv = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rs_bias, off + g * 16, 0, 0));
-#pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        scale_v[g * 4 + x] = sv[x];
-        bias_v[g * 4 + x] = bv[x];
-      }
-    }
-  }
-
   // ---- reader role: fragment slots (16-byte units) relative to the wave's first row
   int a_rd[KS], w_rd[KS];
 #pragma unroll
@@ -285,17 +325,6 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     out_row[rb] = row_of(pos, raw_o_row[rb]);
   }
 
-  // ---- tile mask: OR over the tile's positions (cumm/conv/kernel.py:844-889 of the reference)
-  uint32_t kmask = 1u;
-  if (has_mask) {
-    kmask = wave_or_dpp(mk) & p.mask_filter;
-    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
-    if (p.exit_on_empty && kmask == 0) return;
-    if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
-    if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
-  }
-  const int n_steps = __builtin_popcount(kmask);
-
   AccV acc[RBW][NBW];
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb)
@@ -304,24 +333,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
 
   const uint32_t a_row_bytes = (uint32_t)p.lda * E::kBytes;
   const uint32_t w_k_bytes = (uint32_t)p.w_stride_k * E::kBytes;
-  const uint32_t g_k_bytes = (uint32_t)p.n_idx * 4u;
-  const uint32_t g_bytes = has_gather ? p.gather_bytes : 0u;
 
-  // lane j of klist holds the j-th kernel offset of the tile (-1 past the end): lane b pushes
-  // b+1 to the lane of its rank among the set bits, lanes without a bit push into lane 63, which
-  // nobody reads; a lane nobody pushed to reads 0.
-  int klist;
-  {
-    const bool bit = lane < 32 && ((kmask >> lane) & 1u);
-    const int rank = __builtin_popcount(kmask & ((1u << (lane & 31)) - 1u));
-    klist = __builtin_amdgcn_ds_permute(bit ? rank * 4 : 63 * 4, bit ? lane + 1 : 0) - 1;
-  }
-
-  auto issue_idx = [&](int j, int *slot) {
-    const int k = __builtin_amdgcn_readlane(klist, j);
-    const v4i rs = rsrc_words(p.gather, k >= 0 ? g_bytes : 0u);
-    dma_b32(rs, lds_addr(slot), (key_bits >> (k & 31)) & 1u ? key_off : kOob, (uint32_t)k * g_k_bytes);
-  };
   // entries of this lane's rows out of the wave's slot (its own loads: no barrier needed)
   auto read_idx = [&](const int *slot, int (&dst)[IPA]) {
 #pragma unroll
@@ -346,13 +358,9 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   };
 
   if (n_steps > 0) {
-    // ---- prologue: entries of offsets 0 .. DI-1, then operands of offsets 0 .. L-1, each
-    // followed by the next entries (the order of a step, so the waits count the same everywhere)
-    auto first = [&](auto jc) -> bool {
-      issue_idx(decltype(jc)::value, idx_slot(jc));
-      return false;
-    };
-    run_steps(first, std::make_integer_sequence<int, DI>{});
+    // ---- prologue (the entries of offsets 0 .. DI-1 are on their way): operands of offsets
+    // 0 .. L-1, each followed by the next entries (the order of a step, so the waits count the
+    // same everywhere)
     auto fill = [&](auto jc) -> bool {
       constexpr int j = decltype(jc)::value;
       wait_vmcnt<DI - 1 + j * (PER_STEP - 1)>();   // entries of offset j have landed
