@@ -157,6 +157,44 @@ def bench_dense_gemm(args):
             "pct_mfma_peak": round(100.0 * tf / PEAK_MFMA_F16_TFLOPS, 3)}
 
 
+def bench_pairs(args, coords):
+    """Input preparation on the GPU for the headline voxel set: hash table + 27 neighbour look-ups
+    per voxel (forward and backward tables, masks), then the stable sort of the masks."""
+    import ctypes as C
+    from cumm_amd import _capi
+    lib = _capi.lib()
+    n = int(coords.shape[0])
+    d_coords = dev(np.ascontiguousarray(coords, np.int32))
+    ind_f, ind_b = tv.empty([27, n], tv.int32, 0), tv.empty([27, n], tv.int32, 0)
+    mask_f, mask_b = tv.empty([n], tv.uint32, 0), tv.empty([n], tv.uint32, 0)
+    smask, order = tv.empty([n], tv.uint32, 0), tv.empty([n], tv.int32, 0)
+    ws1 = tv.empty([int(lib.cumm_hip_subm_pairs_workspace(n))], tv.uint8, 0)
+    ws2 = tv.empty([int(lib.cumm_hip_sort_by_mask_workspace(n))], tv.uint8, 0)
+    arr3 = C.c_int32 * 3
+    shape, ks, dl = arr3(*GRID), arr3(3, 3, 3), arr3(1, 1, 1)
+
+    def pairs_step():
+        _capi.check(lib.cumm_hip_subm_pairs(d_coords.byte_pointer(), n, shape, ks, dl, ind_f.byte_pointer(),
+                                            ind_b.byte_pointer(), mask_f.byte_pointer(), mask_b.byte_pointer(),
+                                            ws1.byte_pointer(), ws1.nbytes, 0))
+
+    def sort_step():
+        _capi.check(lib.cumm_hip_sort_by_mask(mask_f.byte_pointer(), n, 0xFFFFFFFF, smask.byte_pointer(),
+                                              order.byte_pointer(), ws2.byte_pointer(), ws2.nbytes, 0))
+
+    steps, warm = max(5, args.steps // 4), max(2, args.warmup // 4)
+    w1, e1 = timed(pairs_step, steps, warm)
+    w2, e2 = timed(sort_step, steps, warm)
+    bytes1 = n * 16 + 2 * 27 * n * 4 + 2 * n * 4          # coords in; two tables and two masks out
+    bytes2 = 3 * n * 4                                     # masks in; sorted masks and argsort out
+    return {"voxels": n,
+            "subm_pairs": {"ms_per_step": round(w1, 5), "kernel_ms_events": round(e1, 5),
+                           "mvoxels_per_s": round(n / (w1 * 1e-3) / 1e6, 1),
+                           "hbm_frac": round(bytes1 / (e1 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+            "sort_by_mask": {"ms_per_step": round(w2, 5), "kernel_ms_events": round(e2, 5),
+                             "hbm_frac": round(bytes2 / (e2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
+
+
 def bench_s8(args, tile_m):
     """s8 stride-2 SparseConv3d, Cin=64 -> Cout=128, int8 inference epilogue."""
     rng4 = np.random.default_rng(SEED + 4)
@@ -191,7 +229,7 @@ def main():
     ap.add_argument("--tile-m", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
-    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm")
+    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on 512 MiB (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -268,7 +306,7 @@ def main():
     if not args.no_extra:
         extra = {}
         legs = (set(args.extra_only.split(",")) if args.extra_only
-                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm"})
+                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)
         dout = dev(rng.normal(0, 1, size=(n, K)).astype(np.float16))
         if "dgrad" in legs:
@@ -282,6 +320,8 @@ def main():
             extra["gather_gemm_scatter_f16"] = bench_gather_gemm(args)
         if "dense_gemm" in legs:
             extra["dense_gemm_f16_4096"] = bench_dense_gemm(args)
+        if "pairs" in legs:
+            extra["input_preparation_gpu"] = bench_pairs(args, coords)
         result["extra"] = extra
     if not args.no_cpu:
         # CPU baseline: the numpy oracle (per-offset gather -> matmul -> scatter-add) on the

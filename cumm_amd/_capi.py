@@ -86,6 +86,11 @@ SYMBOLS = {
     "cumm_hip_event_synchronize": (C.c_int, [_VP]),
     "cumm_hip_event_elapsed_ms": (C.c_int, [_VP, _VP, C.POINTER(C.c_float)]),
     "cumm_hip_copy_kernel": (C.c_int, [_VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_subm_pairs_workspace": (C.c_size_t, [C.c_int]),
+    "cumm_hip_subm_pairs": (C.c_int, [_VP, C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                      _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_sort_by_mask_workspace": (C.c_size_t, [C.c_int]),
+    "cumm_hip_sort_by_mask": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP, _VP, C.c_size_t, _VP]),
 }
 
 _lib = None

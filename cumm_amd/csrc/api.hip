@@ -623,6 +623,69 @@ __global__ void copy16_kernel(v4i *dst, const v4i *src, size_t n) {
   for (; i < n; i += stride) dst[i] = src[i];
 }
 
+static uint32_t pairs_slots(int n) {
+  uint32_t slots = 1024;
+  while (slots < 2u * (uint32_t)(n > 0 ? n : 0)) slots <<= 1;   // load factor at most one half
+  return slots;
+}
+
+size_t cumm_hip_subm_pairs_workspace(int n) { return (size_t)pairs_slots(n) * 16; }
+
+int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_shape, const int32_t *ksize,
+                        const int32_t *dilation, int32_t *indices_fwd, int32_t *indices_bwd,
+                        uint32_t *mask_fwd, uint32_t *mask_bwd, void *workspace, size_t workspace_bytes,
+                        void *stream) {
+  if (n < 0 || !spatial_shape || !ksize || !dilation) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (n == 0) return CUMM_HIP_OK;
+  if (n > (1 << 30)) return fail(CUMM_HIP_EINVAL, "too many voxels");
+  if (!coords || !indices_fwd || !mask_fwd) return fail(CUMM_HIP_EINVAL, "coords, indices_fwd and mask_fwd must not be empty");
+  if (!aligned16(coords) || !aligned16(workspace)) return fail(CUMM_HIP_EINVAL, "coords and workspace must be 16-byte aligned");
+  const int64_t kv = (int64_t)ksize[0] * ksize[1] * ksize[2];
+  if (ksize[0] < 1 || ksize[1] < 1 || ksize[2] < 1 || kv > 32) return fail(CUMM_HIP_EINVAL, "kernel volume must be 1..32");
+  for (int d = 0; d < 3; ++d)
+    if (spatial_shape[d] < 1 || dilation[d] < 1) return fail(CUMM_HIP_EINVAL, "spatial_shape and dilation must be positive");
+  if (!workspace || workspace_bytes < cumm_hip_subm_pairs_workspace(n))
+    return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", cumm_hip_subm_pairs_workspace(n));
+  SubmPairsParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.coords = coords; p.n = n; p.kv = (int)kv;
+  for (int d = 0; d < 3; ++d) p.shape[d] = spatial_shape[d];
+  for (int k = 0; k < (int)kv; ++k) {
+    const int kz = k / (ksize[1] * ksize[2]), ky = (k / ksize[2]) % ksize[1], kx = k % ksize[2];
+    p.off[k][0] = (kz - ksize[0] / 2) * dilation[0];
+    p.off[k][1] = (ky - ksize[1] / 2) * dilation[1];
+    p.off[k][2] = (kx - ksize[2] / 2) * dilation[2];
+  }
+  p.ind_f = indices_fwd; p.ind_b = indices_bwd; p.mask_f = mask_fwd; p.mask_b = mask_bwd;
+  p.table = workspace; p.slot_mask = pairs_slots(n) - 1u;
+  hipError_t e = launch_subm_pairs(p, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "pair table launch");
+  return CUMM_HIP_OK;
+}
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+size_t cumm_hip_sort_by_mask_workspace(int n) {
+  const size_t words = align256(sizeof(uint32_t) * (size_t)(n > 0 ? n : 1));
+  return 2 * words + align256(sort_by_mask_temp_bytes(n));
+}
+
+int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
+                          int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream) {
+  if (n < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (n == 0) return CUMM_HIP_OK;
+  if (!mask || !sorted_mask || !argsort) return fail(CUMM_HIP_EINVAL, "mask, sorted_mask and argsort must not be empty");
+  if (!workspace || workspace_bytes < cumm_hip_sort_by_mask_workspace(n))
+    return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", cumm_hip_sort_by_mask_workspace(n));
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(CUMM_HIP_EINVAL, "workspace must be 256-byte aligned");
+  const size_t words = align256(sizeof(uint32_t) * (size_t)n);
+  char *base = reinterpret_cast<char *>(workspace);
+  hipError_t e = launch_sort_by_mask(mask, n, mask_filter, sorted_mask, argsort, base, base + words, base + 2 * words,
+                                     workspace_bytes - 2 * words, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "mask sort launch");
+  return CUMM_HIP_OK;
+}
+
 int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes % 16 || !aligned16(dst) || !aligned16(src)) return fail(CUMM_HIP_EINVAL, "copy needs 16-byte alignment");
   const size_t n = bytes / 16;

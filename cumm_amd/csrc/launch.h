@@ -31,4 +31,20 @@ inline bool tilegemm_has_tile(int tm, int tn) {
   return (tm == 64 && tn == 64) || (tm == 128 && tn == 128);
 }
 
+// ---- pair tables of a submanifold convolution and the mask sort (pairs_inst.hip)
+struct SubmPairsParams {
+  const int32_t *coords;   // [n, 4] (batch, z, y, x)
+  int32_t n, kv;
+  int32_t shape[3];
+  int32_t off[32][3];      // (k_zyx - center) * dilation per kernel offset
+  int32_t *ind_f, *ind_b;  // [kv, n]; ind_b may be NULL
+  uint32_t *mask_f, *mask_b;
+  void *table;             // (slot_mask + 1) slots of 16 bytes
+  uint32_t slot_mask;
+};
+hipError_t launch_subm_pairs(const SubmPairsParams &p, hipStream_t s);
+size_t sort_by_mask_temp_bytes(int n);
+hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
+                               void *keys_ws, void *iota_ws, void *temp, size_t temp_bytes, hipStream_t s);
+
 }  // namespace cummhip

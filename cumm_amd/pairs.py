@@ -133,3 +133,62 @@ def sort_by_mask(mask: np.ndarray, mask_filter: int = 0xFFFFFFFF):
     key = mask & np.uint32(mask_filter)
     order = np.argsort(key, kind="stable").astype(np.int32)
     return np.ascontiguousarray(key[order]), order
+
+
+# ---- the same tables built on the GPU (cumm_hip_subm_pairs / cumm_hip_sort_by_mask) ----------
+
+class DevicePairTable(NamedTuple):
+    indices_fwd: "object"   # tv.Tensor [kv, N] int32 on the device
+    indices_bwd: "object"   # tv.Tensor [kv, N] int32
+    mask_fwd: "object"      # tv.Tensor [N] uint32
+    mask_bwd: "object"      # tv.Tensor [N] uint32
+
+
+def subm_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), dilation=(1, 1, 1),
+                      workspace=None, stream: int = 0) -> DevicePairTable:
+    """GPU counterpart of :func:`subm_pairs`: ``coords`` is a device ``tv.Tensor`` [N, 4] int32 of
+    unique (batch, z, y, x); the tables stay on the device.  What the reference's callers take from
+    ``SpconvOps.generate_subm_conv_inds`` (cumm/conv/main_real_spconv.py:91-105 of the reference)."""
+    import ctypes as C
+
+    from . import _capi
+    from . import tensorview as tv
+    if coords.device < 0 or coords.dtype != tv.int32 or coords.ndim != 2 or coords.shape[1] != 4:
+        raise ValueError("coords must be a device int32 tensor of shape [N, 4]")
+    n = int(coords.shape[0])
+    kv = int(ksize[0]) * int(ksize[1]) * int(ksize[2])
+    lib = _capi.lib()
+    need = int(lib.cumm_hip_subm_pairs_workspace(n))
+    if workspace is None or workspace.empty():
+        workspace = tv.empty([max(need, 16)], tv.uint8, 0)
+    ind_f = tv.empty([kv, n], tv.int32, 0)
+    ind_b = tv.empty([kv, n], tv.int32, 0)
+    mask_f = tv.empty([n], tv.uint32, 0)
+    mask_b = tv.empty([n], tv.uint32, 0)
+    arr3 = C.c_int32 * 3
+    _capi.check(lib.cumm_hip_subm_pairs(
+        coords.byte_pointer(), n, arr3(*[int(v) for v in spatial_shape]), arr3(*[int(v) for v in ksize]),
+        arr3(*[int(v) for v in dilation]), ind_f.byte_pointer(), ind_b.byte_pointer(), mask_f.byte_pointer(),
+        mask_b.byte_pointer(), workspace.byte_pointer(), workspace.nbytes, stream))
+    return DevicePairTable(ind_f, ind_b, mask_f, mask_b)
+
+
+def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, stream: int = 0):
+    """GPU counterpart of :func:`sort_by_mask` on a device ``tv.Tensor`` [N] uint32: returns
+    (sorted mask, argsort) device tensors (spconv's sort_1d_by_key[_split], call site
+    cumm/conv/main_real_spconv.py:118-145 of the reference)."""
+    from . import _capi
+    from . import tensorview as tv
+    if mask.device < 0 or mask.dtype != tv.uint32 or mask.ndim != 1:
+        raise ValueError("mask must be a device uint32 vector")
+    n = int(mask.shape[0])
+    lib = _capi.lib()
+    need = int(lib.cumm_hip_sort_by_mask_workspace(n))
+    if workspace is None or workspace.empty():
+        workspace = tv.empty([max(need, 256)], tv.uint8, 0)
+    out_mask = tv.empty([n], tv.uint32, 0)
+    order = tv.empty([n], tv.int32, 0)
+    _capi.check(lib.cumm_hip_sort_by_mask(mask.byte_pointer(), n, int(mask_filter) & 0xFFFFFFFF,
+                                          out_mask.byte_pointer(), order.byte_pointer(),
+                                          workspace.byte_pointer(), workspace.nbytes, stream))
+    return out_mask, order

@@ -165,6 +165,29 @@ int cumm_hip_event_record(void *event, void *stream);
 int cumm_hip_event_synchronize(void *event);
 int cumm_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* host out-param */
 
+/* ---- input preparation for the mask-based kernels (the step before the hot path).
+ * The reference does not do this itself: its callers take pair tables and sorted masks from
+ * spconv (SpconvOps.generate_subm_conv_inds and sort_1d_by_key, call sites
+ * cumm/conv/main_real_spconv.py:91-145); the reference's building block for it is the
+ * linear-probing hash table include/tensorview/hash/linear.cu.h:111-840.
+ *
+ * cumm_hip_subm_pairs: pair tables of a submanifold convolution.
+ *   coords [n, 4] int32 (batch, z, y, x), unique; spatial_shape, ksize (kernel volume <= 32),
+ *   dilation: 3 ints each (host).  Outputs (device): indices_fwd [kv, n] int32 (-1 = none),
+ *   mask_fwd [n] uint32; indices_bwd / mask_bwd may be NULL.  Kernel offset k = (kz*KY + ky)*KX + kx,
+ *   output o gathers the input at coord[o] + (k_zyx - ksize/2) * dilation.
+ *   workspace: at least cumm_hip_subm_pairs_workspace(n) bytes, 16-byte aligned.
+ * cumm_hip_sort_by_mask: sorted = stable ascending sort of (mask & mask_filter), argsort = the
+ *   permutation; workspace at least cumm_hip_sort_by_mask_workspace(n) bytes. */
+size_t cumm_hip_subm_pairs_workspace(int n);
+int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_shape, const int32_t *ksize,
+                        const int32_t *dilation, int32_t *indices_fwd, int32_t *indices_bwd,
+                        uint32_t *mask_fwd, uint32_t *mask_bwd, void *workspace, size_t workspace_bytes,
+                        void *stream);
+size_t cumm_hip_sort_by_mask_workspace(int n);
+int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
+                          int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream);
+
 /* Plain device-to-device copy kernel of `bytes` bytes (16-byte aligned); used to
  * calibrate the HBM traffic counters against a transfer of known size. */
 int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
