@@ -629,7 +629,8 @@ static uint32_t pairs_slots(int n) {
   return slots;
 }
 
-size_t cumm_hip_subm_pairs_workspace(int n) { return (size_t)pairs_slots(n) * 16; }
+// hash table slots (16 bytes each), then one presence word per slot pair
+size_t cumm_hip_subm_pairs_workspace(int n) { return (size_t)pairs_slots(n) * 16 + (size_t)pairs_slots(n) * 4; }
 
 int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_shape, const int32_t *ksize,
                         const int32_t *dilation, int32_t *indices_fwd, int32_t *indices_bwd,
@@ -658,6 +659,9 @@ int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_sha
   }
   p.ind_f = indices_fwd; p.ind_b = indices_bwd; p.mask_f = mask_fwd; p.mask_b = mask_bwd;
   p.table = workspace; p.slot_mask = pairs_slots(n) - 1u;
+  p.filter = reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(workspace) + (size_t)pairs_slots(n) * 16);
+  p.filter_mask = pairs_slots(n) - 1u;
+  p.kx = ksize[2];
   hipError_t e = launch_subm_pairs(p, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "pair table launch");
   return CUMM_HIP_OK;

@@ -41,6 +41,9 @@ struct SubmPairsParams {
   uint32_t *mask_f, *mask_b;
   void *table;             // (slot_mask + 1) slots of 16 bytes
   uint32_t slot_mask;
+  uint32_t *filter;        // (filter_mask + 1) presence words
+  uint32_t filter_mask;
+  int32_t kx;              // offsets along x (kv = kz * ky * kx)
 };
 hipError_t launch_subm_pairs(const SubmPairsParams &p, hipStream_t s);
 size_t sort_by_mask_temp_bytes(int n);
