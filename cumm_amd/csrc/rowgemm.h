@@ -54,6 +54,9 @@ struct RowGemmParams {
   int32_t act;
   int32_t int8_epilogue;  // scale/bias requantisation instead of alpha/beta
   int32_t read_source;    // D is read (beta != 0)
+  // LDS-streaming kernel only: the contraction is walked in 2^chunk_shift chunks of one stage
+  // row each (a step = one kernel offset x one chunk); 0 = the whole contraction fits a row
+  int32_t chunk_shift;
 };
 
 // An offset no buffer contains: every operand is smaller than 2 GiB (checked on the host), and

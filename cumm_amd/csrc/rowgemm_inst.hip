@@ -44,6 +44,24 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   dim3 grid((p.n_pos + TM - 1) / TM, (p.k_out + TN - 1) / TN, 1);
   if (grid.x == 0 || grid.y == 0) return hipSuccess;
   constexpr int chunk_e = 4 * KS * Elem<T>::kPerVec;
+  // A contraction longer than 128 bytes: the LDS-streaming kernel with 128-byte stage rows (three
+  // stages fit, three workgroups per CU) walking the contraction in chunks, rather than
+  // 256-byte rows with two stages or the register-gather kernels.
+  if constexpr (KS == 4) {
+    constexpr int NS2 = lds_stages(TM, TN, 2);
+    if constexpr (NS2 > 0 && (!WT || Elem<T>::kBytes == 2)) {
+      constexpr int chunk2 = 4 * 2 * Elem<T>::kPerVec;
+      const int nch = (p.c_in + chunk2 - 1) / chunk2;
+      int shift = 0;
+      while ((1 << shift) < nch) ++shift;
+      if (shift <= 3 && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
+        RowGemmParams q = p;
+        q.chunk_shift = shift;
+        hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 2, NS2, WT>), grid, dim3(256), 0, s, q);
+        return hipGetLastError();
+      }
+    }
+  }
   constexpr int NS = lds_stages(TM, TN, KS);
   if constexpr (NS > 0 && (!WT || Elem<T>::kBytes == 2)) {
     // the LDS-streaming kernel: 2 x 2 waves, each TM/2 rows by TN/2 channels

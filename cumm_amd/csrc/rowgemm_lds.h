@@ -226,7 +226,8 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
     if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
   }
-  const int n_steps = __builtin_popcount(kmask);
+  // a step = one kernel offset x one chunk of the contraction (one chunk unless chunk_shift)
+  const int n_steps = __builtin_popcount(kmask) << p.chunk_shift;
 
 
   const uint32_t g_k_bytes = (uint32_t)p.n_idx * 4u;
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   }
 
   auto issue_idx = [&](int j, int *slot) {
-    const int k = __builtin_amdgcn_readlane(klist, j);
+    const int k = __builtin_amdgcn_readlane(klist, (j >> p.chunk_shift) & 63);
     const v4i rs = rsrc_words(p.gather, k >= 0 ? g_bytes : 0u);
     dma_b32(rs, lds_addr(slot), (key_bits >> (k & 31)) & 1u ? key_off : kOob, (uint32_t)k * g_k_bytes);
   };
@@ -260,6 +261,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   int a_key[IPA];          // without a pair table the gathered row is the key itself
   uint32_t a_col[IPA];     // byte offset of the fetched chunk inside the gathered row, or kOob
   uint32_t a_bits[IPA];    // mask word of the row
+  int a_cpos[IPA];         // first contraction element of the fetched chunk (in the first chunk of the row)
 #pragma unroll
   for (int t = 0; t < IPA; ++t) {
     const int r = (wave * IPA + t) * RPI + lrow;
@@ -269,9 +271,11 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     const int key = pos < p.n_pos ? (p.gather_by_pos ? pos : row) : -1;
     a_key[t] = key >= 0 && key < p.n_idx ? key : -1;
     const int c = lchunk ^ swz(r);
-    a_col[t] = a_key[t] >= 0 && c * PV < p.c_in ? (uint32_t)c * 16u : kOob;
+    a_cpos[t] = c * PV;
+    a_col[t] = a_key[t] >= 0 ? (uint32_t)c * 16u : kOob;
   }
   uint32_t w_voff[IPW];
+  int w_cpos[IPW];         // contraction element (WT: contraction row) the lane fetches, first chunk
   auto swz_w = [](int e) { return 2 * (((e * LPRW) >> 4) & (LPRW / 2 - 1)); };   // WT: even chunk XOR
 #pragma unroll
   for (int t = 0; t < IPW; ++t) {
@@ -280,16 +284,14 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       const int i = rho & 15, nb = (rho >> 4) % NBW, wq = rho / (16 * NBW);
       const int n = n0 + wq * (16 * NBW) + (i >> 2) * (4 * NBW) + nb * 4 + (i & 3);
       const int c = lchunk ^ swz(rho);
-      w_voff[t] = n < p.k_out && c * PV < p.c_in
-                      ? (uint32_t)((int64_t)n * p.w_stride_n * E::kBytes) + (uint32_t)c * 16u
-                      : kOob;
+      w_cpos[t] = c * PV;
+      w_voff[t] = n < p.k_out ? (uint32_t)((int64_t)n * p.w_stride_n * E::kBytes) + (uint32_t)c * 16u : kOob;
     } else {
       const int e = (wave * IPW + t) * RPIW + lane / LPRW;   // contraction row
       const int c = (lane % LPRW) ^ swz_w(e);                 // chunk of the row this lane fetches
       const int n = n0 + c * PV;
-      w_voff[t] = e < p.c_in && n < p.k_out
-                      ? (uint32_t)(((int64_t)e * p.w_stride_c + n) * E::kBytes)
-                      : kOob;
+      w_cpos[t] = e;
+      w_voff[t] = n < p.k_out ? (uint32_t)(((int64_t)e * p.w_stride_c + n) * E::kBytes) : kOob;
     }
   }
 
@@ -339,8 +341,12 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
 #pragma unroll
     for (int t = 0; t < IPA; ++t) dst[t] = has_gather ? slot[t * RPI + lrow] : a_key[t];
   };
+  constexpr int CHUNK_E = LPR * PV;      // contraction elements of a stage row
   auto issue_operands = [&](int j, const int (&src)[IPA], v4i *st) {
-    const int k = __builtin_amdgcn_readlane(klist, j);
+    const int k = __builtin_amdgcn_readlane(klist, (j >> p.chunk_shift) & 63);
+    const int cc = j & ((1 << p.chunk_shift) - 1);          // chunk of the contraction
+    const int cc_e = cc * CHUNK_E;                           // its first element
+    const uint32_t cc_b = (uint32_t)cc * (LPR * 16u);        // ... as bytes inside a row
     const v4i rs_a = rsrc_words(p.A, k >= 0 ? p.a_bytes : 0u);
     const v4i rs_w = rsrc_words(p.W, k >= 0 ? p.w_bytes : 0u);
 #pragma unroll
@@ -348,13 +354,16 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       // a_col is out of range already for a row without a key or a chunk past the contraction;
       // adding a row offset below 2 GiB keeps it out of range
       const uint32_t v = (uint32_t)src[t];
-      const uint32_t voff = v < (uint32_t)p.rows_a && ((a_bits[t] >> (k & 31)) & 1u) ? v * a_row_bytes + a_col[t] : kOob;
+      const uint32_t voff = v < (uint32_t)p.rows_a && ((a_bits[t] >> (k & 31)) & 1u) && cc_e + a_cpos[t] < p.c_in
+                                ? v * a_row_bytes + a_col[t] + cc_b
+                                : kOob;
       dma_b128(rs_a, lds_addr(st + (wave * IPA + t) * 64), voff, 0u);
     }
-    const uint32_t soff = (uint32_t)k * w_k_bytes;   // k = -1 comes with zero records
+    // k = -1 comes with zero records; a transposed weight tile steps CHUNK_E contraction rows
+    const uint32_t soff = (uint32_t)k * w_k_bytes + (WT ? (uint32_t)cc_e * (uint32_t)p.w_stride_c * E::kBytes : cc_b);
 #pragma unroll
     for (int t = 0; t < IPW; ++t)
-      dma_b128(rs_w, lds_addr(st + A_V + (wave * IPW + t) * 64), w_voff[t], soff);
+      dma_b128(rs_w, lds_addr(st + A_V + (wave * IPW + t) * 64), cc_e + w_cpos[t] < p.c_in ? w_voff[t] : kOob, soff);
   };
 
   if (n_steps > 0) {
