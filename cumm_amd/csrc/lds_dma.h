@@ -62,6 +62,26 @@ __device__ __forceinline__ int load_b32_hidden(v4i rsrc, uint32_t voff) {
   return r;
 }
 __device__ __forceinline__ void keep_after_wait(int &r) { asm volatile("" : "+v"(r)); }
+// The same for 8 and 16 bytes.
+typedef int v2i_hidden __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ v2i_hidden load_b64_hidden(v4i rsrc, uint32_t voff) {
+  v2i_hidden r;
+  asm volatile("buffer_load_dwordx2 %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  return r;
+}
+__device__ __forceinline__ v4i load_b128_hidden(v4i rsrc, uint32_t voff) {
+  v4i r;
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  return r;
+}
+__device__ __forceinline__ void keep_after_wait(v2i_hidden &r) { asm volatile("" : "+v"(r)); }
+__device__ __forceinline__ void keep_after_wait(v4i &r) { asm volatile("" : "+v"(r)); }
+template <int W>
+__device__ __forceinline__ auto load_hidden_words(v4i rsrc, uint32_t voff) {
+  static_assert(W == 2 || W == 4, "8 or 16 bytes");
+  if constexpr (W == 2) return load_b64_hidden(rsrc, voff);
+  else return load_b128_hidden(rsrc, voff);
+}
 
 // Workgroup barrier without the fence of __syncthreads(): the fence would wait for every
 // outstanding direct-to-LDS load, i.e. also for the stages that are being prefetched.  The empty

@@ -177,6 +177,14 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     }
   }
 
+  // Without a mask and with entries addressed by position (gather -> GEMM -> scatter), the first
+  // entries depend on nothing that is loaded here: requested now, they land with the loads above.
+  const bool early_idx = !has_mask && p.gather_by_pos && p.gather != nullptr;
+  if (early_idx) {
+    const bool live = lane < RPW && key_pos < p.n_pos && key_pos < p.n_idx;
+    dma_b32(rsrc_words(p.gather, p.gather_bytes), lds_addr(ix0[wave]), live ? (uint32_t)key_pos * 4u : kOob, 0u);
+  }
+
   wait_vmcnt<0>();
 #pragma unroll
   for (int i = 0; i < MKW; ++i) keep_after_wait(raw_mk[i]);
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   // rows, fragment slots) overlaps their round trip.
   if (n_steps > 0) {
     auto first = [&](auto jc) -> bool {
-      issue_idx(decltype(jc)::value, idx_slot(jc));
+      if (!(early_idx && decltype(jc)::value == 0)) issue_idx(decltype(jc)::value, idx_slot(jc));
       return false;
     };
     run_steps(first, std::make_integer_sequence<int, DI>{});
@@ -325,6 +333,38 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   for (int rb = 0; rb < RBW; ++rb) {
     const int pos = pos_base + (wm * RBW + rb) * 16 + m;
     out_row[rb] = row_of(pos, raw_o_row[rb]);
+  }
+
+  // ---- the rows that the epilogue blends in (beta * D) are requested now, as hidden loads that
+  // the final wait of the step loop covers: their round trip runs under the loop instead of
+  // behind it.  These loads
+  // are older than every operand load of the loop, so the counted waits there only get stricter.
+  constexpr int CPLW = 4 * NBW;            // consecutive output channels of a lane (not WT)
+  constexpr int SRC_W = E::kBytes == 2 ? (WT ? 2 : 4) : CPLW / 4;   // dwords per piece
+  constexpr int SRC_N = E::kBytes == 2 ? (WT ? NBW : CPLW / 8) : 1; // pieces per row
+  static_assert(E::kBytes == 1 || WT || CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
+  const int ch0 = n0 + wn * (NBW * 16) + q * CPLW;
+  auto piece_channel = [&](int i) -> int {
+    if constexpr (E::kBytes == 2 && WT) return n0 + (wn * NBW + i) * 16 + 4 * q;
+    else if constexpr (E::kBytes == 2) return ch0 + i * 8;
+    else return ch0;
+  };
+  typedef int src_vec __attribute__((ext_vector_type(SRC_W)));
+  src_vec src_pre[RBW][SRC_N] = {};
+  if (p.read_source) {
+    const v4i rsw_d = rsrc_words(p.D, p.d_bytes);
+#pragma unroll
+    for (int rb = 0; rb < RBW; ++rb) {
+      const int o = out_row[rb];
+      const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+      for (int i = 0; i < SRC_N; ++i) {
+        const int ch = piece_channel(i);
+        const bool ok = row_ok && ch < p.k_out;
+        src_pre[rb][i] = load_hidden_words<SRC_W>(
+            rsw_d, ok ? (uint32_t)((int64_t)o * p.ldd + ch) * (uint32_t)E::kBytes : kOob);
+      }
+    }
   }
 
   AccV acc[RBW][NBW];
@@ -431,13 +471,14 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   }
 
   wait_vmcnt<0>();   // the loads past the end of the offset list still target this workgroup's LDS
+#pragma unroll
+  for (int rb = 0; rb < RBW; ++rb)
+#pragma unroll
+    for (int i = 0; i < SRC_N; ++i) keep_after_wait(src_pre[rb][i]);
   // ---- epilogue: lane (q, m) holds, for each of its rows, channels ch0 .. ch0 + 4*NBW - 1.
   // The activation and the blend mode are lifted out of the element loops (one straight-line
   // copy per combination): tested per element they cost more issue slots than the arithmetic.
-  constexpr int CPLW = 4 * NBW;
   const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.c_bytes);
-  const __amdgpu_buffer_rsrc_t rs_d = make_rsrc(p.D, p.read_source ? p.d_bytes : 0u);
-  const int ch0 = n0 + wn * (NBW * 16) + q * CPLW;
   // MODE: 0 = alpha*acc, 1 = alpha*acc + beta*src, 2 = scale*acc + bias, 3 = ... + beta*src
   auto store_rows = [&](auto act_c, auto mode_c) {
     constexpr int ACT = decltype(act_c)::value;
@@ -456,10 +497,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
           const bool ok = row_ok && ch < p.k_out;
           const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
           v2i src = {0, 0};
-          if constexpr (SRC) {
-            const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 2u : kOob;
-            src = __builtin_amdgcn_raw_buffer_load_b64(rs_d, doff, 0, 0);
-          }
+          if constexpr (SRC) src = __builtin_bit_cast(v2i, src_pre[rb][nb]);
           const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
           v2i outv;
           uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
@@ -475,7 +513,6 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       }
     } else if constexpr (E::kBytes == 2) {
       constexpr int NG = CPLW / 8;   // 16-byte groups
-      static_assert(CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb) {
         const int o = out_row[rb];
@@ -486,10 +523,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
           const bool ok = row_ok && ch < p.k_out;
           const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
           v4i src = {0, 0, 0, 0};
-          if constexpr (SRC) {
-            const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 2u : kOob;
-            src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
-          }
+          if constexpr (SRC) src = __builtin_bit_cast(v4i, src_pre[rb][g]);
           const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
           v4i outv;
           uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
@@ -514,11 +548,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
         const bool ok = o >= 0 && o < p.rows_c && ch0 < p.k_out;
         const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch0) : kOob;
         vNi src = {};
-        if constexpr (SRC) {
-          const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch0) : kOob;
-          if constexpr (ND == 4) src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
-          else src = __builtin_amdgcn_raw_buffer_load_b64(rs_d, doff, 0, 0);
-        }
+        if constexpr (SRC) src = __builtin_bit_cast(vNi, src_pre[rb][0]);
         const int8_t *sb = reinterpret_cast<const int8_t *>(&src);
         vNi outv;
         int ob[CPLW];
