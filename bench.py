@@ -185,6 +185,30 @@ def bench_pairs(args, coords):
     steps, warm = max(5, args.steps // 4), max(2, args.warmup // 4)
     w1, e1 = timed(pairs_step, steps, warm)
     w2, e2 = timed(sort_step, steps, warm)
+    # regular (strided) convolution on the voxel set of the s8 leg: active output sites (with the
+    # one synchronisation that returns their number), then the tables
+    c4 = synth.clustered_voxels(np.random.default_rng(SEED + 4), 300000, GRID, 60, sigma=15.0, noise_frac=0.10)
+    n4 = int(c4.shape[0])
+    d_c4 = dev(np.ascontiguousarray(c4, np.int32))
+    st, pd = arr3(2, 2, 2), arr3(1, 1, 1)
+    ws3 = tv.empty([int(lib.cumm_hip_conv_pairs_workspace(n4, 1, shape, ks, st, pd, dl))], tv.uint8, 0)
+    out_shape, n_out = arr3(), C.c_int32(0)
+    _capi.check(lib.cumm_hip_conv_pairs_sites(d_c4.byte_pointer(), n4, 1, shape, ks, st, pd, dl, out_shape,
+                                              C.byref(n_out), ws3.byte_pointer(), ws3.nbytes, 0))
+    m4 = int(n_out.value)
+    oc4, f4, b4 = tv.empty([m4, 4], tv.int32, 0), tv.empty([27, m4], tv.int32, 0), tv.empty([27, n4], tv.int32, 0)
+    mf4, mb4 = tv.empty([m4], tv.uint32, 0), tv.empty([n4], tv.uint32, 0)
+
+    def conv_pairs_step():
+        _capi.check(lib.cumm_hip_conv_pairs_sites(d_c4.byte_pointer(), n4, 1, shape, ks, st, pd, dl, out_shape,
+                                                  C.byref(n_out), ws3.byte_pointer(), ws3.nbytes, 0))
+        _capi.check(lib.cumm_hip_conv_pairs_fill(d_c4.byte_pointer(), n4, 1, shape, ks, st, pd, dl, int(n_out.value),
+                                                 oc4.byte_pointer(), f4.byte_pointer(), b4.byte_pointer(),
+                                                 mf4.byte_pointer(), mb4.byte_pointer(), ws3.byte_pointer(),
+                                                 ws3.nbytes, 0))
+
+    w3, e3 = timed(conv_pairs_step, steps, warm)
+    bytes3 = n4 * 16 + 27 * (n4 + m4) * 4 + (n4 + m4) * 4 + m4 * 16   # coords in; tables, masks, coords out
     bytes1 = n * 16 + 2 * 27 * n * 4 + 2 * n * 4          # coords in; two tables and two masks out
     bytes2 = 3 * n * 4                                     # masks in; sorted masks and argsort out
     return {"voxels": n,
@@ -192,7 +216,10 @@ def bench_pairs(args, coords):
                            "mvoxels_per_s": round(n / (w1 * 1e-3) / 1e6, 1),
                            "hbm_frac": round(bytes1 / (e1 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
             "sort_by_mask": {"ms_per_step": round(w2, 5), "kernel_ms_events": round(e2, 5),
-                             "hbm_frac": round(bytes2 / (e2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
+                             "hbm_frac": round(bytes2 / (e2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+            "sparse_conv_pairs_stride2": {"voxels_in": n4, "voxels_out": m4, "ms_per_step": round(w3, 5),
+                                          "mvoxels_per_s": round(n4 / (w3 * 1e-3) / 1e6, 1),
+                                          "hbm_frac": round(bytes3 / (w3 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
 
 
 def bench_s8(args, tile_m):

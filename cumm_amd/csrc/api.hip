@@ -690,6 +690,176 @@ int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uin
   return CUMM_HIP_OK;
 }
 
+// ---- regular (strided) sparse convolution
+namespace {
+struct ConvPairsLayout {
+  bool bitmap;         // small output grid: bitmap + prefix sums instead of hash set + sort
+  unsigned long long n_words;
+  uint32_t slots;
+  size_t bound;        // most output sites n_in inputs can reach
+  size_t off_uniq, off_sorted, off_counters, off_prefix, off_temp, total;
+};
+int gcd_int(int a, int b) { return b == 0 ? a : gcd_int(b, a % b); }
+// out_shape as ConvProblem.calc_output_dims (cumm/conv/params.py:268-292 of the reference)
+const char *conv_pairs_check(int batch_size, const int32_t *spatial_shape, const int32_t *ksize, const int32_t *stride,
+                             const int32_t *padding, const int32_t *dilation, int32_t *out_shape,
+                             unsigned long long *sites) {
+  if (!spatial_shape || !ksize || !stride || !padding || !dilation) return "geometry arrays must not be empty";
+  if (batch_size < 1) return "batch_size must be positive";
+  const int64_t kv = (int64_t)ksize[0] * ksize[1] * ksize[2];
+  if (ksize[0] < 1 || ksize[1] < 1 || ksize[2] < 1 || kv > 32) return "kernel volume must be 1..32";
+  unsigned long long total = (unsigned long long)batch_size;
+  for (int d = 0; d < 3; ++d) {
+    if (spatial_shape[d] < 1 || dilation[d] < 1 || stride[d] < 1 || padding[d] < 0)
+      return "spatial_shape, stride and dilation must be positive, padding not negative";
+    const int64_t span = (int64_t)spatial_shape[d] + 2 * (int64_t)padding[d] - (int64_t)dilation[d] * (ksize[d] - 1) - 1;
+    const int64_t o = span < 0 ? 0 : span / stride[d] + 1;
+    if (o < 1 || o > (1 << 30)) return "empty output shape";
+    out_shape[d] = (int32_t)o;
+    if (total > (1ull << 62) / (unsigned long long)o) return "output grid of more than 2^62 sites";
+    total *= (unsigned long long)o;
+  }
+  *sites = total;
+  return nullptr;
+}
+// An input reaches, per axis, the offsets k with (x + pad - k*dilation) % stride == 0: every
+// stride / gcd(stride, dilation)-th one.
+bool conv_pairs_layout(int n_in, unsigned long long sites, const int32_t *ksize, const int32_t *stride,
+                       const int32_t *dilation, ConvPairsLayout *l) {
+  std::memset(l, 0, sizeof(*l));
+  l->bitmap = sites <= (1ull << 33);
+  if (l->bitmap) {
+    l->n_words = ((sites + 31ull) / 32ull + 3ull) & ~3ull;
+    l->off_prefix = align256((size_t)l->n_words * 4);
+    l->off_temp = l->off_prefix + align256((size_t)l->n_words * 4 + 4);   // (+ the total)
+    l->total = l->off_temp + align256(conv_pairs_scan_temp_bytes((size_t)l->n_words));
+    return true;
+  }
+  int64_t per_input = 1;
+  for (int d = 0; d < 3; ++d) {
+    const int period = stride[d] / gcd_int(stride[d], dilation[d]);
+    per_input *= (ksize[d] + period - 1) / period;
+  }
+  const int64_t bound = per_input * (int64_t)(n_in > 0 ? n_in : 0);
+  if (bound >= ((int64_t)1 << 30)) return false;
+  uint32_t slots = 1024;
+  while ((int64_t)slots < bound + bound / 2) slots <<= 1;   // load factor at most two thirds
+  l->slots = slots;
+  l->bound = (size_t)bound;
+  l->off_uniq = align256((size_t)slots * 16);
+  l->off_sorted = l->off_uniq + align256(l->bound * 8 + 8);
+  l->off_counters = l->off_sorted + align256(l->bound * 8 + 8);
+  l->off_temp = l->off_counters + 256;
+  l->total = l->off_temp + align256(conv_pairs_sort_temp_bytes(l->bound));
+  return true;
+}
+void conv_pairs_params(ConvPairsParams *p, const ConvPairsLayout &l, const int32_t *coords, int n_in, int batch_size,
+                       const int32_t *out_shape, const int32_t *ksize, const int32_t *stride, const int32_t *padding,
+                       const int32_t *dilation, void *workspace) {
+  std::memset(p, 0, sizeof(*p));
+  p->coords = coords; p->n_in = n_in; p->batch = batch_size;
+  p->kv = ksize[0] * ksize[1] * ksize[2];
+  for (int d = 0; d < 3; ++d) { p->out_shape[d] = out_shape[d]; p->stride[d] = stride[d]; p->pad[d] = padding[d]; }
+  for (int k = 0; k < p->kv; ++k) {
+    p->koff[k][0] = (k / (ksize[1] * ksize[2])) * dilation[0];
+    p->koff[k][1] = ((k / ksize[2]) % ksize[1]) * dilation[1];
+    p->koff[k][2] = (k % ksize[2]) * dilation[2];
+  }
+  char *base = reinterpret_cast<char *>(workspace);
+  if (l.bitmap) {
+    p->bits = reinterpret_cast<uint32_t *>(base);
+    p->prefix = reinterpret_cast<uint32_t *>(base + l.off_prefix);
+    p->n_words = l.n_words;
+    return;
+  }
+  p->table = base; p->slot_mask = l.slots - 1u;
+  p->uniq = reinterpret_cast<unsigned long long *>(base + l.off_uniq);
+  p->sorted = reinterpret_cast<unsigned long long *>(base + l.off_sorted);
+  p->counters = reinterpret_cast<unsigned long long *>(base + l.off_counters);
+}
+}  // namespace
+
+size_t cumm_hip_conv_pairs_workspace(int n_in, int batch_size, const int32_t *spatial_shape, const int32_t *ksize,
+                                     const int32_t *stride, const int32_t *padding, const int32_t *dilation) {
+  ConvPairsLayout l;
+  int32_t out_shape[3];
+  unsigned long long sites = 0;
+  if (n_in < 0 || conv_pairs_check(batch_size, spatial_shape, ksize, stride, padding, dilation, out_shape, &sites)) return 0;
+  if (!conv_pairs_layout(n_in, sites, ksize, stride, dilation, &l)) return 0;
+  return l.total;
+}
+
+int cumm_hip_conv_pairs_sites(const int32_t *coords, int n_in, int batch_size, const int32_t *spatial_shape,
+                              const int32_t *ksize, const int32_t *stride, const int32_t *padding,
+                              const int32_t *dilation, int32_t *out_shape, int32_t *n_out, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+  if (n_in < 0 || !out_shape || !n_out) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  unsigned long long sites = 0;
+  if (const char *why = conv_pairs_check(batch_size, spatial_shape, ksize, stride, padding, dilation, out_shape, &sites))
+    return fail(CUMM_HIP_EINVAL, "%s", why);
+  *n_out = 0;
+  if (n_in == 0) return CUMM_HIP_OK;
+  ConvPairsLayout l;
+  if (!conv_pairs_layout(n_in, sites, ksize, stride, dilation, &l)) return fail(CUMM_HIP_EINVAL, "too many voxels");
+  if (!coords || !aligned16(coords)) return fail(CUMM_HIP_EINVAL, "coords must be 16-byte aligned and not empty");
+  if (!workspace || workspace_bytes < l.total) return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", l.total);
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(CUMM_HIP_EINVAL, "workspace must be 256-byte aligned");
+  ConvPairsParams p;
+  conv_pairs_params(&p, l, coords, n_in, batch_size, out_shape, ksize, stride, padding, dilation, workspace);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  char *temp = reinterpret_cast<char *>(workspace) + l.off_temp;
+  // Either way the caller sizes its tables by the number of sites: the one synchronisation of the path.
+  if (l.bitmap) {
+    hipError_t e = launch_conv_pairs_bits(p, temp, l.total - l.off_temp, s);
+    if (e != hipSuccess) return hip_fail(e, "output site launch");
+    uint32_t total = 0;
+    HIP_TRY(hipMemcpyAsync(&total, p.prefix + l.n_words, 4, hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (total >= (1u << 31)) return fail(CUMM_HIP_ERUNTIME, "more than 2^31 output sites");
+    *n_out = (int32_t)total;
+    return CUMM_HIP_OK;
+  }
+  hipError_t e = launch_conv_pairs_sites(p, s);
+  if (e != hipSuccess) return hip_fail(e, "output site launch");
+  unsigned long long counters[2] = {0, 0};
+  HIP_TRY(hipMemcpyAsync(counters, p.counters, sizeof(counters), hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipStreamSynchronize(s));
+  if (counters[0] > l.bound) return fail(CUMM_HIP_ERUNTIME, "more output sites than the geometry allows (duplicate coordinates?)");
+  p.n_out = (int)counters[0];
+  e = launch_conv_pairs_sort(p, counters[1], temp, l.total - l.off_temp, s);
+  if (e != hipSuccess) return hip_fail(e, "output site sort");
+  *n_out = p.n_out;
+  return CUMM_HIP_OK;
+}
+
+int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, const int32_t *spatial_shape,
+                             const int32_t *ksize, const int32_t *stride, const int32_t *padding,
+                             const int32_t *dilation, int n_out, int32_t *out_coords, int32_t *indices_fwd,
+                             int32_t *indices_bwd, uint32_t *mask_fwd, uint32_t *mask_bwd, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+  if (n_in < 0 || n_out < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  int32_t out_shape[3];
+  unsigned long long sites = 0;
+  if (const char *why = conv_pairs_check(batch_size, spatial_shape, ksize, stride, padding, dilation, out_shape, &sites))
+    return fail(CUMM_HIP_EINVAL, "%s", why);
+  if (n_in == 0) return CUMM_HIP_OK;
+  ConvPairsLayout l;
+  if (!conv_pairs_layout(n_in, sites, ksize, stride, dilation, &l)) return fail(CUMM_HIP_EINVAL, "too many voxels");
+  if (!l.bitmap && (size_t)n_out > l.bound) return fail(CUMM_HIP_EINVAL, "n_out is not what cumm_hip_conv_pairs_sites returned");
+  if (!coords || !aligned16(coords)) return fail(CUMM_HIP_EINVAL, "coords must be 16-byte aligned and not empty");
+  if (n_out > 0 && (!out_coords || !indices_fwd || !mask_fwd || !aligned16(out_coords) || !aligned16(indices_fwd)))
+    return fail(CUMM_HIP_EINVAL, "out_coords, indices_fwd (both 16-byte aligned) and mask_fwd must not be empty");
+  if (!workspace || workspace_bytes < l.total) return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", l.total);
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(CUMM_HIP_EINVAL, "workspace must be 256-byte aligned");
+  ConvPairsParams p;
+  conv_pairs_params(&p, l, coords, n_in, batch_size, out_shape, ksize, stride, padding, dilation, workspace);
+  p.n_out = n_out;
+  p.out_coords = out_coords; p.ind_f = indices_fwd; p.ind_b = indices_bwd; p.mask_f = mask_fwd; p.mask_b = mask_bwd;
+  hipError_t e = launch_conv_pairs_fill(p, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "pair table launch");
+  return CUMM_HIP_OK;
+}
+
 int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes % 16 || !aligned16(dst) || !aligned16(src)) return fail(CUMM_HIP_EINVAL, "copy needs 16-byte alignment");
   const size_t n = bytes / 16;

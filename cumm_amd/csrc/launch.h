@@ -46,6 +46,32 @@ struct SubmPairsParams {
   int32_t kx;              // offsets along x (kv = kz * ky * kx)
 };
 hipError_t launch_subm_pairs(const SubmPairsParams &p, hipStream_t s);
+
+// ---- pair tables of a regular (strided) sparse convolution (pairs_inst.hip)
+struct ConvPairsParams {
+  const int32_t *coords;        // [n_in, 4] (batch, z, y, x)
+  int32_t n_in, n_out, kv, batch;
+  int32_t out_shape[3], stride[3], pad[3];
+  int32_t koff[32][3];          // k_zyx * dilation per kernel offset
+  void *table;                  // (slot_mask + 1) slots of 16 bytes: {output site key, output row}
+  uint32_t slot_mask;
+  unsigned long long *uniq;     // output site keys in order of discovery
+  unsigned long long *sorted;   // the same, ascending = output rows
+  unsigned long long *counters; // [0] number of output sites, [1] largest key
+  uint32_t *bits;               // instead of the table, for a small output grid: one bit per site,
+  uint32_t *prefix;             // and the number of active sites before each 32-bit word
+  unsigned long long n_words;   // (0 = hash set and sort)
+  int32_t *out_coords;          // [n_out, 4]
+  int32_t *ind_f, *ind_b;       // [kv, n_out], [kv, n_in] (may be NULL)
+  uint32_t *mask_f, *mask_b;    // [n_out], [n_in] (may be NULL)
+};
+hipError_t launch_conv_pairs_sites(const ConvPairsParams &p, hipStream_t s);
+size_t conv_pairs_sort_temp_bytes(size_t max_sites);
+hipError_t launch_conv_pairs_sort(const ConvPairsParams &p, unsigned long long max_key, void *temp, size_t temp_bytes,
+                                  hipStream_t s);
+hipError_t launch_conv_pairs_fill(const ConvPairsParams &p, hipStream_t s);
+size_t conv_pairs_scan_temp_bytes(size_t n_words);
+hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t temp_bytes, hipStream_t s);
 size_t sort_by_mask_temp_bytes(int n);
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
                                void *keys_ws, void *iota_ws, void *temp, size_t temp_bytes, hipStream_t s);

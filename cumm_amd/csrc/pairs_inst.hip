@@ -24,6 +24,8 @@
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
+#include <rocprim/iterator/transform_iterator.hpp>
 
 #include "launch.h"
 
@@ -139,7 +141,304 @@ __global__ __launch_bounds__(256) void sort_keys_kernel(const uint32_t *mask, ui
   iota[i] = i;
 }
 
+// ---- regular (strided) sparse convolution: an output site is active iff an input falls into
+// its receptive field; output rows are the active sites in ascending (batch, z, y, x) order.
+// (What spconv's generate_conv_inds_mask_stage1 / unique / stage2 give the reference's callers.)
+//   1. every (input, offset) computes its output site; the sites go into a hash set, whose keys
+//      are then gathered into a list (one counter update per 8192 slots);
+//   2. the list is sorted (radix sort over the bits of the largest key): position = output row;
+//   3. the rows are written back into the set, and every (input, offset) looks its site up again:
+//      indices_fwd[k][row] = input, indices_bwd[k][input] = row, the masks by atomic OR.
+// The tables depend on the geometry only: bit-exact against the host builder.
+
+// output site of input c through offset k: (c + pad - k*dilation) / stride where that is exact
+__device__ __forceinline__ bool conv_out_site(const ConvPairsParams &p, const int4 c, int k, unsigned long long *key) {
+  const int in[3] = {c.y, c.z, c.w};
+  if (c.x < 0 || c.x >= p.batch) return false;
+  unsigned long long acc = (unsigned long long)c.x;
+#pragma unroll
+  for (int d = 0; d < 3; ++d) {
+    const int num = in[d] + p.pad[d] - p.koff[k][d];
+    const int q = num / p.stride[d];
+    if (num < 0 || q * p.stride[d] != num || q >= p.out_shape[d]) return false;
+    acc = acc * (unsigned long long)p.out_shape[d] + (unsigned long long)q;
+  }
+  *key = acc;
+  return true;
+}
+
+__global__ __launch_bounds__(256) void conv_pairs_clear_kernel(const ConvPairsParams p) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i <= p.slot_mask) reinterpret_cast<Slot *>(p.table)[i] = Slot{kEmptyKey, -1, 0};
+  if (i < 2) p.counters[i] = 0ull;
+}
+
+__global__ __launch_bounds__(256) void conv_pairs_sites_kernel(const ConvPairsParams p) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int k = blockIdx.y;
+  if (i >= p.n_in) return;
+  Slot *table = reinterpret_cast<Slot *>(p.table);
+  unsigned long long key = 0;
+  if (!conv_out_site(p, reinterpret_cast<const int4 *>(p.coords)[i], k, &key)) return;
+  uint32_t h = (uint32_t)mix64(key) & p.slot_mask;
+  // most candidates repeat a site that is already there: look before the compare-and-swap (a
+  // key never changes once set, so a stale look only costs the swap)
+  for (uint32_t probe = 0; probe <= p.slot_mask; ++probe) {
+    unsigned long long cur = __atomic_load_n(&table[h].key, __ATOMIC_RELAXED);
+    if (cur == kEmptyKey) cur = atomicCAS(&table[h].key, kEmptyKey, key);
+    if (cur == kEmptyKey || cur == key) break;
+    h = (h + 1) & p.slot_mask;
+  }
+}
+
+// The set's keys, gathered into a list in any order (it is sorted next).  A workgroup takes 8192
+// slots and updates the shared counter and the shared maximum once each: updates of one address
+// from all over the chip complete one at a time, about 6 ns each (one per wave of candidates, 250 k
+// of them, took 1.5 ms; one per 2048 slots plus a maximum per wave 96 us).
+constexpr int kCompactPerThread = 32;
+__global__ __launch_bounds__(256) void conv_pairs_compact_kernel(const ConvPairsParams p) {
+  __shared__ uint32_t wave_cnt[4];
+  __shared__ unsigned long long wave_top[4];
+  __shared__ unsigned long long wg_base;
+  const Slot *table = reinterpret_cast<const Slot *>(p.table);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t first = blockIdx.x * (256u * kCompactPerThread);
+  unsigned long long keys[kCompactPerThread];
+  uint32_t mine = 0;
+  unsigned long long top = 0;
+#pragma unroll
+  for (int u = 0; u < kCompactPerThread; ++u) {
+    const uint32_t slot = first + (uint32_t)u * 256u + (uint32_t)tid;
+    keys[u] = slot <= p.slot_mask ? table[slot].key : kEmptyKey;
+  }
+#pragma unroll
+  for (int u = 0; u < kCompactPerThread; ++u) {
+    const bool have = keys[u] != kEmptyKey;
+    mine += (uint32_t)__popcll(__ballot(have));
+    if (have && keys[u] > top) top = keys[u];
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const unsigned long long other = __shfl_xor(top, off);
+    top = other > top ? other : top;
+  }
+  if (lane == 0) {
+    wave_cnt[wave] = mine;
+    wave_top[wave] = top;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    const uint32_t total = wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
+    unsigned long long t = wave_top[0];
+    for (int w = 1; w < 4; ++w) t = wave_top[w] > t ? wave_top[w] : t;
+    wg_base = total ? atomicAdd(&p.counters[0], (unsigned long long)total) : 0ull;
+    if (total) atomicMax(&p.counters[1], t);   // largest key: it bounds the sort's passes
+  }
+  __syncthreads();
+  unsigned long long at = wg_base;
+  for (int w = 0; w < wave; ++w) at += wave_cnt[w];
+#pragma unroll
+  for (int u = 0; u < kCompactPerThread; ++u) {
+    const bool have = keys[u] != kEmptyKey;
+    const unsigned long long found = __ballot(have);
+    if (have) p.uniq[at + __popcll(found & ((1ull << lane) - 1ull))] = keys[u];
+    at += __popcll(found);
+  }
+}
+
+// every (row, offset) starts at -1; the sites get their rows, the coordinates are decoded and the
+// masks zeroed
+__global__ __launch_bounds__(256) void conv_pairs_rows_kernel(const ConvPairsParams p) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  {
+    // the whole forward table starts at -1: 16-byte stores over the flat array, the last thread
+    // writes the odd words at the end
+    const int64_t words = (int64_t)p.kv * p.n_out, quads = words >> 2;
+    const v4i none = {-1, -1, -1, -1};
+    for (int64_t q = j; q < quads; q += (int64_t)gridDim.x * 256) reinterpret_cast<v4i *>(p.ind_f)[q] = none;
+    if (j == 0)
+      for (int64_t w = quads << 2; w < words; ++w) p.ind_f[w] = -1;
+  }
+  if (j < p.n_in && p.mask_b) p.mask_b[j] = 0u;
+  if (j >= p.n_out) return;
+  Slot *table = reinterpret_cast<Slot *>(p.table);
+  unsigned long long key = p.sorted[j];
+  uint32_t h = (uint32_t)mix64(key) & p.slot_mask;
+  for (uint32_t probe = 0; probe <= p.slot_mask; ++probe) {
+    if (table[h].key == key) {
+      table[h].row = j;
+      break;
+    }
+    h = (h + 1) & p.slot_mask;
+  }
+  int4 c;
+  c.w = (int)(key % (unsigned long long)p.out_shape[2]); key /= (unsigned long long)p.out_shape[2];
+  c.z = (int)(key % (unsigned long long)p.out_shape[1]); key /= (unsigned long long)p.out_shape[1];
+  c.y = (int)(key % (unsigned long long)p.out_shape[0]); key /= (unsigned long long)p.out_shape[0];
+  c.x = (int)key;
+  reinterpret_cast<int4 *>(p.out_coords)[j] = c;
+  p.mask_f[j] = 0u;
+}
+
+template <bool BITS>
+__global__ __launch_bounds__(256) void conv_pairs_fill_kernel(const ConvPairsParams p) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int k = blockIdx.y;
+  if (i >= p.n_in) return;
+  unsigned long long key = 0;
+  int row = -1;
+  if (conv_out_site(p, reinterpret_cast<const int4 *>(p.coords)[i], k, &key)) {
+    if constexpr (BITS) {
+      const uint32_t word = p.bits[key >> 5], b = (uint32_t)key & 31u;
+      if ((word >> b) & 1u) row = (int)(p.prefix[key >> 5] + (uint32_t)__popc(word & ((1u << b) - 1u)));
+    } else {
+      const Slot *table = reinterpret_cast<const Slot *>(p.table);
+      uint32_t h = (uint32_t)mix64(key) & p.slot_mask;
+      Slot s = table[h];
+      for (uint32_t probe = 0; s.key != key && s.key != kEmptyKey && probe <= p.slot_mask; ++probe) {
+        h = (h + 1) & p.slot_mask;
+        s = table[h];
+      }
+      if (s.key == key) row = s.row;
+    }
+  }
+  if (p.ind_b) p.ind_b[(int64_t)k * p.n_in + i] = row;
+  if (row >= 0 && row < p.n_out) {
+    p.ind_f[(int64_t)k * p.n_out + row] = i;
+    atomicOr(&p.mask_f[row], 1u << k);
+    if (p.mask_b) atomicOr(&p.mask_b[i], 1u << k);
+  }
+}
+
+// ---- the same with a bitmap of the output grid in place of the hash set (grids of up to 2^33
+// sites): a site's row is the number of set bits before it - a prefix sum over the words' bit
+// counts -, so neither the list, nor the sort, nor any probing is needed.
+__global__ __launch_bounds__(256) void conv_bits_clear_kernel(const ConvPairsParams p) {
+  const v4i zero = {0, 0, 0, 0};   // (n_words is a multiple of 4)
+  for (unsigned long long q = blockIdx.x * 256ull + threadIdx.x; q < p.n_words / 4; q += gridDim.x * 256ull)
+    reinterpret_cast<v4i *>(p.bits)[q] = zero;
+}
+
+__global__ __launch_bounds__(256) void conv_bits_sites_kernel(const ConvPairsParams p) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int k = blockIdx.y;
+  if (i >= p.n_in) return;
+  unsigned long long key = 0;
+  if (!conv_out_site(p, reinterpret_cast<const int4 *>(p.coords)[i], k, &key)) return;
+  const uint32_t bit = 1u << ((uint32_t)key & 31u);
+  // a third of the candidates repeat a site: look first (a set bit stays set)
+  if (!(__atomic_load_n(&p.bits[key >> 5], __ATOMIC_RELAXED) & bit)) atomicOr(&p.bits[key >> 5], bit);
+}
+
+// number of active sites, behind the prefix sums (one 4-byte copy to the host instead of two)
+__global__ void conv_bits_total_kernel(const ConvPairsParams p) {
+  p.prefix[p.n_words] = p.prefix[p.n_words - 1] + (uint32_t)__popc(p.bits[p.n_words - 1]);
+}
+
+struct BitCount {
+  __host__ __device__ uint32_t operator()(uint32_t w) const { return (uint32_t)__builtin_popcount(w); }
+};
+
+// table prefill, masks, and the coordinates of the active sites, word by word
+__global__ __launch_bounds__(256) void conv_bits_rows_kernel(const ConvPairsParams p) {
+  const unsigned long long j = blockIdx.x * 256ull + threadIdx.x, step = gridDim.x * 256ull;
+  {
+    const unsigned long long words = (unsigned long long)p.kv * p.n_out, quads = words >> 2;
+    const v4i none = {-1, -1, -1, -1};
+    for (unsigned long long q = j; q < quads; q += step) reinterpret_cast<v4i *>(p.ind_f)[q] = none;
+    if (j == 0)
+      for (unsigned long long w = quads << 2; w < words; ++w) p.ind_f[w] = -1;
+  }
+  if (p.mask_b)
+    for (unsigned long long i = j; i < (unsigned long long)p.n_in; i += step) p.mask_b[i] = 0u;
+  for (unsigned long long o = j; o < (unsigned long long)p.n_out; o += step) p.mask_f[o] = 0u;
+  for (unsigned long long w = j; w < p.n_words; w += step) {
+    uint32_t word = p.bits[w];
+    uint32_t row = p.prefix[w];
+    while (word != 0u) {
+      const int b = __ffs((int)word) - 1;
+      word &= word - 1u;
+      unsigned long long site = w * 32ull + (unsigned long long)b;
+      int4 c;
+      c.w = (int)(site % (unsigned long long)p.out_shape[2]); site /= (unsigned long long)p.out_shape[2];
+      c.z = (int)(site % (unsigned long long)p.out_shape[1]); site /= (unsigned long long)p.out_shape[1];
+      c.y = (int)(site % (unsigned long long)p.out_shape[0]); site /= (unsigned long long)p.out_shape[0];
+      c.x = (int)site;
+      if (row < (uint32_t)p.n_out) reinterpret_cast<int4 *>(p.out_coords)[row] = c;
+      ++row;
+    }
+  }
+}
+
 }  // namespace
+
+hipError_t launch_conv_pairs_sites(const ConvPairsParams &p, hipStream_t s) {
+  hipLaunchKernelGGL(conv_pairs_clear_kernel, dim3((p.slot_mask + 256u) / 256u), dim3(256), 0, s, p);
+  if (p.n_in > 0) {
+    hipLaunchKernelGGL(conv_pairs_sites_kernel, dim3((p.n_in + 255) / 256, p.kv), dim3(256), 0, s, p);
+    const uint32_t per_wg = 256u * kCompactPerThread;
+    hipLaunchKernelGGL(conv_pairs_compact_kernel, dim3((p.slot_mask + per_wg) / per_wg), dim3(256), 0, s, p);
+  }
+  return hipGetLastError();
+}
+
+size_t conv_pairs_sort_temp_bytes(size_t max_sites) {
+  size_t bytes = 0;
+  (void)rocprim::radix_sort_keys(nullptr, bytes, (const unsigned long long *)nullptr, (unsigned long long *)nullptr,
+                                 max_sites > 0 ? max_sites : 1, 0, 64);
+  return bytes;
+}
+
+hipError_t launch_conv_pairs_sort(const ConvPairsParams &p, unsigned long long max_key, void *temp, size_t temp_bytes,
+                                  hipStream_t s) {
+  if (p.n_out <= 0) return hipSuccess;
+  int end_bit = 1;
+  while (end_bit < 64 && (max_key >> end_bit) != 0ull) ++end_bit;
+  return rocprim::radix_sort_keys(temp, temp_bytes, (const unsigned long long *)p.uniq, p.sorted, (size_t)p.n_out, 0,
+                                  end_bit, s);
+}
+
+hipError_t launch_conv_pairs_fill(const ConvPairsParams &p, hipStream_t s) {
+  const int most = p.n_out > p.n_in ? p.n_out : p.n_in;
+  if (most <= 0) return hipSuccess;
+  if (p.n_words != 0ull) {
+    unsigned long long wgs = (p.n_words + 255ull) / 256ull;
+    if (wgs < (unsigned long long)(most + 255) / 256) wgs = (unsigned long long)(most + 255) / 256;
+    if (wgs > 16384ull) wgs = 16384ull;
+    hipLaunchKernelGGL(conv_bits_rows_kernel, dim3((unsigned)wgs), dim3(256), 0, s, p);
+    if (p.n_in > 0)
+      hipLaunchKernelGGL(conv_pairs_fill_kernel<true>, dim3((p.n_in + 255) / 256, p.kv), dim3(256), 0, s, p);
+    return hipGetLastError();
+  }
+  hipLaunchKernelGGL(conv_pairs_rows_kernel, dim3((most + 255) / 256), dim3(256), 0, s, p);
+  if (p.n_in > 0)
+    hipLaunchKernelGGL(conv_pairs_fill_kernel<false>, dim3((p.n_in + 255) / 256, p.kv), dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+size_t conv_pairs_scan_temp_bytes(size_t n_words) {
+  size_t bytes = 0;
+  (void)rocprim::exclusive_scan(nullptr, bytes, rocprim::make_transform_iterator((const uint32_t *)nullptr, BitCount()),
+                                (uint32_t *)nullptr, 0u, n_words > 0 ? n_words : 1, rocprim::plus<uint32_t>());
+  return bytes;
+}
+
+// bitmap of the active output sites and its prefix sums
+hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t temp_bytes, hipStream_t s) {
+  unsigned long long wgs = (p.n_words / 4 + 255ull) / 256ull;
+  if (wgs > 16384ull) wgs = 16384ull;
+  if (wgs == 0ull) wgs = 1ull;
+  hipLaunchKernelGGL(conv_bits_clear_kernel, dim3((unsigned)wgs), dim3(256), 0, s, p);
+  if (p.n_in > 0)
+    hipLaunchKernelGGL(conv_bits_sites_kernel, dim3((p.n_in + 255) / 256, p.kv), dim3(256), 0, s, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  e = rocprim::exclusive_scan(temp, temp_bytes, rocprim::make_transform_iterator((const uint32_t *)p.bits, BitCount()),
+                              p.prefix, 0u, (size_t)p.n_words, rocprim::plus<uint32_t>(), s);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(conv_bits_total_kernel, dim3(1), dim3(1), 0, s, p);
+  return hipGetLastError();
+}
 
 hipError_t launch_subm_pairs(const SubmPairsParams &p, hipStream_t s) {
   if (p.n <= 0) return hipSuccess;

@@ -173,6 +173,55 @@ def subm_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), dil
     return DevicePairTable(ind_f, ind_b, mask_f, mask_b)
 
 
+class DeviceConvPairTable(NamedTuple):
+    indices_fwd: "object"   # tv.Tensor [kv, N_out] int32 on the device
+    indices_bwd: "object"   # tv.Tensor [kv, N_in] int32
+    mask_fwd: "object"      # tv.Tensor [N_out] uint32
+    mask_bwd: "object"      # tv.Tensor [N_in] uint32
+    out_coords: "object"    # tv.Tensor [N_out, 4] int32
+    out_shape: Tuple[int, ...]
+
+
+def sparse_conv_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), stride=(2, 2, 2),
+                             padding=(1, 1, 1), dilation=(1, 1, 1), batch_size: int = 1, workspace=None,
+                             stream: int = 0) -> DeviceConvPairTable:
+    """GPU counterpart of :func:`sparse_conv_pairs`: ``coords`` is a device ``tv.Tensor`` [N, 4]
+    int32 of unique (batch, z, y, x); the tables stay on the device.  Two library calls with one
+    stream synchronisation between them (the number of active output sites sizes the tables), as
+    with spconv's generate_conv_inds_mask_stage1 / stage2.  Batch indices are 0 .. batch_size-1."""
+    import ctypes as C
+
+    from . import _capi
+    from . import tensorview as tv
+    if coords.device < 0 or coords.dtype != tv.int32 or coords.ndim != 2 or coords.shape[1] != 4:
+        raise ValueError("coords must be a device int32 tensor of shape [N, 4]")
+    n_in = int(coords.shape[0])
+    kv = int(ksize[0]) * int(ksize[1]) * int(ksize[2])
+    lib = _capi.lib()
+    arr3 = C.c_int32 * 3
+    geo = [arr3(*[int(v) for v in a]) for a in (spatial_shape, ksize, stride, padding, dilation)]
+    need = int(lib.cumm_hip_conv_pairs_workspace(n_in, int(batch_size), *geo))
+    if need == 0:
+        raise ValueError("bad geometry (kernel volume 1..32, non-empty output grid) or too many voxels")
+    if workspace is None or workspace.empty():
+        workspace = tv.empty([max(need, 256)], tv.uint8, 0)
+    out_shape = arr3()
+    n_out = C.c_int32(0)
+    _capi.check(lib.cumm_hip_conv_pairs_sites(coords.byte_pointer(), n_in, int(batch_size), *geo, out_shape, C.byref(n_out),
+                                              workspace.byte_pointer(), workspace.nbytes, stream))
+    n = int(n_out.value)
+    out_coords = tv.empty([n, 4], tv.int32, 0)
+    ind_f = tv.empty([kv, n], tv.int32, 0)
+    ind_b = tv.empty([kv, n_in], tv.int32, 0)
+    mask_f = tv.empty([n], tv.uint32, 0)
+    mask_b = tv.empty([n_in], tv.uint32, 0)
+    _capi.check(lib.cumm_hip_conv_pairs_fill(
+        coords.byte_pointer(), n_in, int(batch_size), *geo, n, out_coords.byte_pointer(), ind_f.byte_pointer(),
+        ind_b.byte_pointer(), mask_f.byte_pointer(), mask_b.byte_pointer(), workspace.byte_pointer(),
+        workspace.nbytes, stream))
+    return DeviceConvPairTable(ind_f, ind_b, mask_f, mask_b, out_coords, tuple(int(v) for v in out_shape))
+
+
 def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, stream: int = 0):
     """GPU counterpart of :func:`sort_by_mask` on a device ``tv.Tensor`` [N] uint32: returns
     (sorted mask, argsort) device tensors (spconv's sort_1d_by_key[_split], call site

@@ -188,6 +188,35 @@ size_t cumm_hip_sort_by_mask_workspace(int n);
 int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
                           int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Pair tables of a regular (strided) sparse convolution, in two calls like spconv's
+ * generate_conv_inds_mask_stage1 / stage2 (the reference's callers take them from there; its own
+ * building block is the same hash table, include/tensorview/hash/linear.cu.h:111-840).  Output
+ * shape as ConvProblem.calc_output_dims (cumm/conv/params.py:268-292).  An output site is active
+ * iff an input falls into its receptive field; output rows are the active sites in ascending
+ * (batch, z, y, x) order; output o gathers the input at o*stride - padding + k_zyx*dilation.
+ *
+ * cumm_hip_conv_pairs_sites finds the active sites: writes out_shape[3] and *n_out (host) and
+ *   SYNCHRONISES the stream once to do so (the caller sizes its tables by n_out).
+ * cumm_hip_conv_pairs_fill, with the same coords, geometry and workspace (untouched in between)
+ *   and that n_out: out_coords [n_out, 4], indices_fwd [kv, n_out] (both 16-byte aligned), mask_fwd [n_out];
+ *   indices_bwd [kv, n_in] / mask_bwd [n_in] may be NULL (indices_bwd[k][i] = the output row that
+ *   input i feeds through offset k, -1 = none).
+ * batch_size: the batch indices of coords are 0 .. batch_size-1 (others are ignored).  Output
+ *   grids of up to 2^33 sites (batch included) are handled with a bitmap of the grid (an eighth
+ *   of a byte per site, twice), larger ones with a hash set and a sort: same results.
+ * workspace: at least cumm_hip_conv_pairs_workspace(...) bytes (0 = bad geometry), 256-byte aligned. */
+size_t cumm_hip_conv_pairs_workspace(int n_in, int batch_size, const int32_t *spatial_shape, const int32_t *ksize,
+                                     const int32_t *stride, const int32_t *padding, const int32_t *dilation);
+int cumm_hip_conv_pairs_sites(const int32_t *coords, int n_in, int batch_size, const int32_t *spatial_shape,
+                              const int32_t *ksize, const int32_t *stride, const int32_t *padding,
+                              const int32_t *dilation, int32_t *out_shape, int32_t *n_out, void *workspace,
+                              size_t workspace_bytes, void *stream);
+int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, const int32_t *spatial_shape,
+                             const int32_t *ksize, const int32_t *stride, const int32_t *padding,
+                             const int32_t *dilation, int n_out, int32_t *out_coords, int32_t *indices_fwd,
+                             int32_t *indices_bwd, uint32_t *mask_fwd, uint32_t *mask_bwd, void *workspace,
+                             size_t workspace_bytes, void *stream);
+
 /* Plain device-to-device copy kernel of `bytes` bytes (16-byte aligned); used to
  * calibrate the HBM traffic counters against a transfer of known size. */
 int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);

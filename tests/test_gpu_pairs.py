@@ -64,3 +64,95 @@ def test_pairs_argument_errors():
         pairs.subm_pairs_device(c, (4, 4, 4), ksize=(3, 3, 5))        # kernel volume 45 > 32
     with pytest.raises(RuntimeError):
         pairs.subm_pairs_device(c, (4, 4, 4), workspace=tv.zeros([64], tv.uint8, 0))   # too small
+
+
+# ---- regular (strided) sparse convolution -------------------------------------------------------
+
+def _check_conv_case(coords, shape, ksize=(3, 3, 3), stride=(2, 2, 2), padding=(1, 1, 1), dilation=(1, 1, 1),
+                     batch_size=2):
+    ref = pairs.sparse_conv_pairs(coords, shape, ksize, stride, padding, dilation)
+    got = pairs.sparse_conv_pairs_device(H.dev(np.ascontiguousarray(coords, np.int32), "i32"), shape, ksize,
+                                         stride, padding, dilation, batch_size=batch_size)
+    assert tuple(got.out_shape) == tuple(ref.out_shape)
+    np.testing.assert_array_equal(H.host(got.out_coords), ref.out_coords)
+    np.testing.assert_array_equal(H.host(got.indices_fwd), ref.indices_fwd)
+    np.testing.assert_array_equal(H.host(got.indices_bwd), ref.indices_bwd)
+    np.testing.assert_array_equal(H.host(got.mask_fwd), ref.mask_fwd)
+    np.testing.assert_array_equal(H.host(got.mask_bwd), ref.mask_bwd)
+    return ref, got
+
+
+def _random_coords(rng, n, shape, batches=2):
+    total = batches * shape[0] * shape[1] * shape[2]
+    cells = rng.choice(total, size=min(n, total), replace=False)
+    return np.stack(np.unravel_index(cells, (batches,) + tuple(shape)), axis=1).astype(np.int32)
+
+
+@pytest.mark.parametrize("n,shape", [(1, (4, 4, 4)), (65, (6, 10, 10)), (3000, (12, 40, 40)), (5000, (9, 17, 33))])
+def test_sparse_conv_pairs_small(n, shape):
+    print("case sparse conv pairs", n, shape, flush=True)
+    _check_conv_case(_random_coords(np.random.default_rng(200 + n), n, shape), shape)
+
+
+def test_sparse_conv_pairs_geometries():
+    """Strides, paddings, dilations and kernel shapes other than 3x3x3 / 2 / 1 / 1, also a stride
+    that shares a factor with the dilation and a stride-1 convolution (every offset reaches)."""
+    rng = np.random.default_rng(7)
+    shape = (10, 21, 18)
+    coords = _random_coords(rng, 2500, shape)
+    for ksize, stride, padding, dilation in [
+            ((3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+            ((3, 3, 3), (2, 2, 2), (0, 0, 0), (1, 1, 1)),
+            ((2, 2, 2), (2, 2, 2), (0, 0, 0), (1, 1, 1)),
+            ((3, 3, 3), (2, 2, 2), (2, 2, 2), (2, 2, 2)),
+            ((1, 3, 3), (1, 2, 3), (0, 1, 2), (1, 1, 2)),
+            ((3, 2, 4), (3, 1, 2), (1, 0, 1), (1, 2, 1))]:
+        print("case sparse conv geometry", ksize, stride, padding, dilation, flush=True)
+        _check_conv_case(coords, shape, ksize, stride, padding, dilation)
+
+
+def test_sparse_conv_pairs_dense_block():
+    """Every voxel of a block: every output site has all of its in-range inputs."""
+    g = np.stack(np.meshgrid(np.arange(8), np.arange(9), np.arange(10), indexing="ij"), -1).reshape(-1, 3)
+    coords = np.zeros((g.shape[0], 4), np.int32)
+    coords[:, 1:] = g
+    coords = coords[np.random.default_rng(5).permutation(coords.shape[0])]
+    _check_conv_case(coords, (8, 9, 10))
+
+
+def test_sparse_conv_pairs_huge_grid_hash_path():
+    """An output grid of 2 x 2048^3 = 2^34 sites is beyond the bitmap: hash set and sort.  Clusters
+    of neighbours so that output sites are shared; also a 3-batch case with a kernel that every
+    input reaches 27 times."""
+    print("case sparse conv pairs hash path", flush=True)
+    rng = np.random.default_rng(11)
+    shape = (4096, 4096, 4096)
+    centres = rng.integers(8, 4088, size=(400, 3))
+    pts = (centres[:, None, :] + rng.integers(-3, 4, size=(400, 40, 3))).reshape(-1, 3)
+    b = rng.integers(0, 2, size=(pts.shape[0], 1))
+    coords = np.unique(np.concatenate([b, pts], axis=1), axis=0).astype(np.int32)
+    coords = coords[rng.permutation(coords.shape[0])]
+    _check_conv_case(coords, shape)
+    _check_conv_case(coords, shape, stride=(1, 1, 1), batch_size=3)
+
+
+def test_sparse_conv_pairs_full_size():
+    """The stride-2 benchmark geometry (300 k voxels in 41 x 1600 x 1408, about 650 k outputs)."""
+    print("case sparse conv pairs full size", flush=True)
+    rng = np.random.default_rng(20240607 + 1)
+    grid = (41, 1600, 1408)
+    coords = synth.clustered_voxels(rng, 300000, grid, 60, sigma=15.0, noise_frac=0.10)
+    ref, got = _check_conv_case(coords, grid, batch_size=1)
+    assert ref.out_coords.shape[0] > coords.shape[0]
+
+
+def test_sparse_conv_pairs_empty_and_errors():
+    got = pairs.sparse_conv_pairs_device(tv.zeros([0, 4], tv.int32, 0), (8, 8, 8))
+    assert got.out_coords.shape[0] == 0 and tuple(got.out_shape) == (4, 4, 4)
+    c = tv.zeros([8, 4], tv.int32, 0)
+    with pytest.raises(ValueError):
+        pairs.sparse_conv_pairs_device(c, (4, 4, 4), ksize=(3, 3, 5))        # kernel volume 45 > 32
+    with pytest.raises(ValueError):
+        pairs.sparse_conv_pairs_device(c, (2, 2, 2), ksize=(3, 3, 3), padding=(0, 0, 0))   # no output
+    with pytest.raises(RuntimeError):
+        pairs.sparse_conv_pairs_device(c, (4, 4, 4), workspace=tv.zeros([256], tv.uint8, 0))   # too small
