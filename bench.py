@@ -141,6 +141,29 @@ def bench_gather_gemm(args):
             "hbm_frac": round(nbytes / (e_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
 
+def bench_gather_scatter(args):
+    """Stand-alone GatherAll.gather and ScatterAll.scatter: 1 M rows of 64 f16 (128 bytes), random
+    permutation.  Gather moves rows in + rows out + indices; scatter-add reads the destination too."""
+    from cumm_amd.gemm.gather import GatherAll, ScatterAll
+    rng5 = np.random.default_rng(SEED + 5)
+    n, c = 1_000_000, 64
+    a = dev(rng5.normal(0, 1, size=(n, c)).astype(np.float16))
+    perm = dev(rng5.permutation(n).astype(np.int32))
+    out = tv.zeros([n, c], tv.float16, 0)
+    g, sc = GatherAll(), ScatterAll()
+    steps, warm = max(5, args.steps // 4), max(2, args.warmup // 4)
+    w1, e1 = timed(lambda: g.gather(out, a, perm), steps, warm)
+    w2, e2 = timed(lambda: sc.scatter(out, a, perm), steps, warm)
+    b1, b2 = n * (2 * c * 2 + 4), n * (3 * c * 2 + 4)
+    return {"rows": n, "row_bytes": c * 2,
+            "gather": {"ms_per_step": round(w1, 5), "kernel_ms_events": round(e1, 5),
+                       "gbytes_per_s": round(b1 / (e1 * 1e-3) / 1e9, 1),
+                       "hbm_frac": round(b1 / (e1 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+            "scatter_add": {"ms_per_step": round(w2, 5), "kernel_ms_events": round(e2, 5),
+                            "gbytes_per_s": round(b2 / (e2 * 1e-3) / 1e9, 1),
+                            "hbm_frac": round(b2 / (e2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
+
+
 def bench_dense_gemm(args):
     """Plain matmul2, 4096^3 f16 (the only MFMA-bound shape of the path)."""
     rng3 = np.random.default_rng(SEED + 3)
@@ -256,7 +279,7 @@ def main():
     ap.add_argument("--tile-m", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
-    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs")
+    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs,gather")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on 512 MiB (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -333,7 +356,7 @@ def main():
     if not args.no_extra:
         extra = {}
         legs = (set(args.extra_only.split(",")) if args.extra_only
-                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs"})
+                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)
         dout = dev(rng.normal(0, 1, size=(n, K)).astype(np.float16))
         if "dgrad" in legs:
@@ -349,6 +372,8 @@ def main():
             extra["dense_gemm_f16_4096"] = bench_dense_gemm(args)
         if "pairs" in legs:
             extra["input_preparation_gpu"] = bench_pairs(args, coords)
+        if "gather" in legs:
+            extra["gather_scatter_rows"] = bench_gather_scatter(args)
         result["extra"] = extra
     if not args.no_cpu:
         # CPU baseline: the numpy oracle (per-offset gather -> matmul -> scatter-add) on the

@@ -96,6 +96,8 @@ SYMBOLS = {
                                   [C.POINTER(C.c_int32), C.POINTER(C.c_int32), _VP, C.c_size_t, _VP]),
     "cumm_hip_conv_pairs_fill": (C.c_int, [_VP, C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5 +
                                  [C.c_int, _VP, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_gather_rows": (C.c_int, [_VP, _VP, _VP, C.c_int, C.c_int, C.c_size_t, _VP]),
+    "cumm_hip_scatter_add_rows": (C.c_int, [_VP, _VP, _VP, C.c_int, C.c_int, C.c_int, C.c_int, _VP]),
 }
 
 _lib = None

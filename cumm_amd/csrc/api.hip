@@ -860,6 +860,59 @@ int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, co
   return CUMM_HIP_OK;
 }
 
+// ---- stand-alone gather / scatter-add
+namespace {
+bool row_move_params(RowMoveParams *p, void *dst, const void *src, const int32_t *indices, int m, int rows_other,
+                     size_t row_bytes, bool *wide) {
+  *wide = row_bytes % 16 == 0 && aligned16(dst) && aligned16(src);
+  const size_t piece = *wide ? 16 : 4;
+  if (row_bytes / piece > 0xffffffffull) return false;
+  p->src = src; p->dst = dst; p->indices = indices;
+  p->per_row = (uint32_t)(row_bytes / piece);
+  p->pieces = (uint64_t)m * p->per_row;
+  p->shift = -1;
+  for (int b = 0; b < 32; ++b)
+    if (p->per_row == (1u << b)) p->shift = b;
+  p->rows_other = rows_other;
+  return true;
+}
+}  // namespace
+
+int cumm_hip_gather_rows(void *output, const void *input, const int32_t *indices, int m, int rows_in,
+                         size_t row_bytes, void *stream) {
+  if (m < 0 || rows_in < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (row_bytes % 4) return fail(CUMM_HIP_ERUNTIME, "not supported. use supported() to check first");
+  if (m == 0 || row_bytes == 0) return CUMM_HIP_OK;
+  if (!output || !indices || (!input && rows_in > 0)) return fail(CUMM_HIP_EINVAL, "output, input and indices must not be empty");
+  if ((reinterpret_cast<uintptr_t>(output) | reinterpret_cast<uintptr_t>(input)) & 3u)
+    return fail(CUMM_HIP_EINVAL, "tensors must be 4-byte aligned");
+  RowMoveParams p;
+  bool wide = false;
+  if (!row_move_params(&p, output, input, indices, m, rows_in, row_bytes, &wide)) return fail(CUMM_HIP_EINVAL, "rows too long");
+  hipError_t e = launch_gather_rows(p, wide, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "gather launch");
+  return CUMM_HIP_OK;
+}
+
+int cumm_hip_scatter_add_rows(void *output, const void *input, const int32_t *indices, int m, int rows_out,
+                              int channels, int dtype, void *stream) {
+  if (m < 0 || rows_out < 0 || channels < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (dtype != CUMM_HIP_F32 && dtype != CUMM_HIP_F16 && dtype != CUMM_HIP_BF16)
+    return fail(CUMM_HIP_ERUNTIME, "can't find a suitable scatter: dtype must be f32, f16 or bf16");
+  const size_t row_bytes = (size_t)channels * (dtype == CUMM_HIP_F32 ? 4 : 2);
+  if (row_bytes % 4) return fail(CUMM_HIP_ERUNTIME, "not supported. use supported() to check first");
+  if (m == 0 || row_bytes == 0 || rows_out == 0) return CUMM_HIP_OK;
+  if (!output || !input || !indices) return fail(CUMM_HIP_EINVAL, "output, input and indices must not be empty");
+  if ((reinterpret_cast<uintptr_t>(output) | reinterpret_cast<uintptr_t>(input)) & 3u)
+    return fail(CUMM_HIP_EINVAL, "tensors must be 4-byte aligned");
+  RowMoveParams p;
+  bool wide = false;
+  if (!row_move_params(&p, output, input, indices, m, rows_out, row_bytes, &wide)) return fail(CUMM_HIP_EINVAL, "rows too long");
+  hipError_t e = launch_scatter_add_rows(p, dtype, wide, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "scatter launch");
+  return CUMM_HIP_OK;
+}
+
 int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes % 16 || !aligned16(dst) || !aligned16(src)) return fail(CUMM_HIP_EINVAL, "copy needs 16-byte alignment");
   const size_t n = bytes / 16;

@@ -76,4 +76,17 @@ size_t sort_by_mask_temp_bytes(int n);
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
                                void *keys_ws, void *iota_ws, void *temp, size_t temp_bytes, hipStream_t s);
 
+// ---- stand-alone row gather / scatter-add (gather_inst.hip)
+struct RowMoveParams {
+  const void *src;
+  void *dst;
+  const int32_t *indices;   // [m]
+  uint64_t pieces;          // m * per_row
+  uint32_t per_row;         // pieces (16 or 4 bytes) per row
+  int32_t shift;            // log2(per_row) when that is a power of two, else -1
+  int32_t rows_other;       // rows of the indexed tensor (gather: source, scatter-add: destination)
+};
+hipError_t launch_gather_rows(const RowMoveParams &p, bool wide, hipStream_t s);
+hipError_t launch_scatter_add_rows(const RowMoveParams &p, int dtype, bool wide, hipStream_t s);
+
 }  // namespace cummhip

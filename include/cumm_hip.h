@@ -217,6 +217,20 @@ int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, co
                              int32_t *indices_bwd, uint32_t *mask_fwd, uint32_t *mask_bwd, void *workspace,
                              size_t workspace_bytes, void *stream);
 
+/* ---- stand-alone row gather / scatter-add (the "native" per-offset path around a plain GEMM)
+ * cumm_hip_gather_rows: output[i, :] = input[indices[i], :] for i < m; rows of row_bytes bytes
+ *   (a multiple of 4), any dtype; an index outside [0, rows_in) gives a row of zeros.
+ *   Replaces GatherAll.gather / Gather.gather (cumm/gemm/gather.py:224-256, 482-497).
+ * cumm_hip_scatter_add_rows: output[indices[i], :] += input[i, :] for i < m, indices unique; dtype
+ *   CUMM_HIP_F32 (the reference's only one), CUMM_HIP_F16 or CUMM_HIP_BF16 (sum formed in fp32,
+ *   rounded once); channels * itemsize a multiple of 4; a row whose index is outside
+ *   [0, rows_out) is dropped.  Replaces ScatterAll.scatter / Scatter.scatter
+ *   (cumm/gemm/gather.py:356-389, 603-617). */
+int cumm_hip_gather_rows(void *output, const void *input, const int32_t *indices, int m, int rows_in,
+                         size_t row_bytes, void *stream);
+int cumm_hip_scatter_add_rows(void *output, const void *input, const int32_t *indices, int m, int rows_out,
+                              int channels, int dtype, void *stream);
+
 /* Plain device-to-device copy kernel of `bytes` bytes (16-byte aligned); used to
  * calibrate the HBM traffic counters against a transfer of known size. */
 int cumm_hip_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);

@@ -16,6 +16,8 @@ Pinning status (how each part is anchored other than by re-typing itself):
 * int8 epilogue                           - exhaustive check of round-half-even + saturation
 * bf16 rounding                           - torch.bfloat16 conversion on random + tie values
 * descriptor names / workspace / mnk      - the reference's own headers compiled into oracle/_ref
+* stand-alone gather / scatter-add         - permutation + inverse, identity index, one-hot matrix
+  product, index counts, f16 tie rounding; tests/test_oracle_gather.py
 * pair tables (SubM and strided)          - PARITY UNPINNED against spconv (not part of the
   reference tree); pinned only against a brute-force dictionary search, and the
   row order of strided outputs / argsort tie-breaking are this build's conventions.
