@@ -279,7 +279,7 @@ def main():
     ap.add_argument("--tile-m", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
-    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs,gather")
+    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs,gather,tuner")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on 512 MiB (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -356,7 +356,7 @@ def main():
     if not args.no_extra:
         extra = {}
         legs = (set(args.extra_only.split(",")) if args.extra_only
-                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather"})
+                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather", "tuner"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)
         dout = dev(rng.normal(0, 1, size=(n, K)).astype(np.float16))
         if "dgrad" in legs:
@@ -374,6 +374,16 @@ def main():
             extra["input_preparation_gpu"] = bench_pairs(args, coords)
         if "gather" in legs:
             extra["gather_scatter_rows"] = bench_gather_scatter(args)
+        if "tuner" in legs:
+            # the timing-based descriptor choice on the headline problem (after the timed region)
+            from cumm_amd import tuner
+            keep = p.conv_algo_desp
+            res = tuner.Tuner(steps=20, warmup=3).tune_conv(p)
+            extra["tuner_forward"] = {"chosen_tile": list(res.desp.tile_shape[:2]),
+                                      "ms_by_tile": {"%dx%d" % (d[0], d[1]): round(ms, 5) for d, ms in
+                                                     zip([c.tile_shape for c in tuner.conv_candidates(p)],
+                                                         [ms for _, ms in res.tried])}}
+            p.conv_algo_desp = keep
         result["extra"] = extra
     if not args.no_cpu:
         # CPU baseline: the numpy oracle (per-offset gather -> matmul -> scatter-add) on the
