@@ -164,6 +164,81 @@ def bench_gather_scatter(args):
                             "hbm_frac": round(b2 / (e2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
 
 
+def bench_stack(args):
+    """bf16 sparse stack layers at 1 M voxels (200 clusters on 64 x 2048 x 2048): one SubMConv3d 3x3x3
+    C = 128 layer (bias + ReLU epilogue) forward / backward-input / backward-weight, the stride-2
+    SparseConv3d 128 -> 256 forward, and the GPU input preparation; descriptors chosen by the tuner."""
+    from cumm_amd import tuner
+    from cumm_amd.tensorview.gemm import Activation
+    grid = (64, 2048, 2048)
+    rng6 = np.random.default_rng(SEED + 6)
+    coords = synth.clustered_voxels(rng6, 1_000_000, grid, 200, sigma=15.0, noise_frac=0.10)
+    n, c = int(coords.shape[0]), 128
+    d_coords = dev(coords)
+
+    def bf16(shape, scale):
+        v = rng6.integers(-127, 128, size=shape, dtype=np.int8).astype(np.float32) * np.float32(scale)
+        return tv.from_numpy(np.ascontiguousarray(synth.f32_to_bf16_bits(v))).type_view(tv.bfloat16).cuda()
+
+    t0 = time.perf_counter()
+    table = pairs.subm_pairs_device(d_coords, grid)
+    ms_tv, order_tv = pairs.sort_by_mask_device(table.mask_fwd)
+    table2 = pairs.sparse_conv_pairs_device(d_coords, grid, batch_size=1)
+    ms2_tv, order2_tv = pairs.sort_by_mask_device(table2.mask_fwd)
+    ConvMainUnitTest_sync()
+    prep_ms = (time.perf_counter() - t0) * 1e3          # first call, allocations included
+    n_out2 = int(table2.indices_fwd.dim(1))
+    pairs1 = int((table.indices_fwd.cpu().numpy() >= 0).sum())
+    pairs2 = int((table2.indices_fwd.cpu().numpy() >= 0).sum())
+    x, w, b = bf16((n, c), 1 / 64), bf16((c, 27, c), 1 / 2048), bf16((c,), 1 / 512)
+    dout = bf16((n, c), 1 / 64)
+    w2, b2 = bf16((256, 27, c), 1 / 2048), bf16((256,), 1 / 512)
+    tn = tuner.Tuner(steps=3, warmup=1)
+    steps, warm = max(5, args.steps // 10), max(2, args.warmup // 10)
+    res = {"voxels": n, "pairs": pairs1, "voxels_out_stride2": n_out2, "pairs_stride2": pairs2,
+           "input_preparation_first_call_ms": round(prep_ms, 3)}
+
+    def leg(name, p, flops):
+        r = tn.tune_conv(p)
+        wms, ems = timed(lambda: ConvMainUnitTest.implicit_gemm2(p), steps, warm)
+        res[name] = {"tile": list(r.desp.tile_shape[:2]), "ms_per_step": round(wms, 5),
+                     "tflops": round(flops / (wms * 1e-3) / 1e12, 2)}
+
+    pf = ConvParams(3, ConvOpType.Forward)
+    pf.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 128, 128)
+    pf.input, pf.weight, pf.bias, pf.output = x, w, b, tv.zeros([n, c], tv.bfloat16, 0)
+    pf.indices, pf.mask, pf.mask_argsort = table.indices_fwd, ms_tv, order_tv
+    pf.beta, pf.act_type = 1.0, Activation.ReLU
+    leg("subm_c128_forward", pf, 2.0 * pairs1 * c * c)
+    pd = ConvParams(3, ConvOpType.BackwardInput)
+    pd.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.BackwardInput, 128, 128)
+    pd.input, pd.weight, pd.output = tv.zeros([n, c], tv.bfloat16, 0), w, dout
+    pd.indices, pd.mask, pd.mask_argsort = table.indices_bwd, ms_tv, order_tv
+    pd.reverse_mask = True
+    leg("subm_c128_backward_input", pd, 2.0 * pairs1 * c * c)
+    red = tv.zeros([(n + 63) // 64], tv.uint32, 0)
+    pm = ConvParams(3, ConvOpType.Forward)        # a forward call with 64-row tiles writes the reduced masks
+    pm.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 64, 128)
+    pm.input, pm.weight, pm.output = x, w, tv.zeros([n, c], tv.bfloat16, 0)
+    pm.indices, pm.mask, pm.mask_argsort, pm.mask_output = table.indices_fwd, ms_tv, order_tv, red
+    ConvMainUnitTest.implicit_gemm2(pm)
+    pw = ConvParams(3, ConvOpType.BackwardWeight)
+    pw.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.BackwardWeight, 64, 64, parallel=True)
+    pw.input, pw.weight, pw.output = x, tv.zeros([c, 27, c], tv.bfloat16, 0), dout
+    pw.indices, pw.mask, pw.mask_argsort = table.indices_fwd, red, order_tv
+    pw.mask_width, pw.split_k_slices = 64, 32
+    wms, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), steps, warm)
+    res["subm_c128_backward_weight_balanced"] = {"ms_per_step": round(wms, 5),
+                                                 "tflops": round(2.0 * pairs1 * c * c / (wms * 1e-3) / 1e12, 2)}
+    p2 = ConvParams(3, ConvOpType.Forward)
+    p2.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 128, 128)
+    p2.input, p2.weight, p2.bias, p2.output = x, w2, b2, tv.zeros([n_out2, 256], tv.bfloat16, 0)
+    p2.indices, p2.mask, p2.mask_argsort = table2.indices_fwd, ms2_tv, order2_tv
+    p2.beta, p2.act_type = 1.0, Activation.ReLU
+    leg("stride2_c128_c256_forward", p2, 2.0 * pairs2 * c * 256)
+    return res
+
+
 def bench_dense_gemm(args):
     """Plain matmul2, 4096^3 f16 (the only MFMA-bound shape of the path)."""
     rng3 = np.random.default_rng(SEED + 3)
@@ -279,7 +354,7 @@ def main():
     ap.add_argument("--tile-m", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
-    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs,gather,tuner")
+    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs,gather,tuner,stack")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on 512 MiB (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
@@ -356,7 +431,7 @@ def main():
     if not args.no_extra:
         extra = {}
         legs = (set(args.extra_only.split(",")) if args.extra_only
-                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather", "tuner"})
+                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather", "tuner", "stack"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)
         dout = dev(rng.normal(0, 1, size=(n, K)).astype(np.float16))
         if "dgrad" in legs:
@@ -374,6 +449,8 @@ def main():
             extra["input_preparation_gpu"] = bench_pairs(args, coords)
         if "gather" in legs:
             extra["gather_scatter_rows"] = bench_gather_scatter(args)
+        if "stack" in legs:
+            extra["bf16_stack_1m"] = bench_stack(args)
         if "tuner" in legs:
             # the timing-based descriptor choice on the headline problem (after the timed region)
             from cumm_amd import tuner
