@@ -1,0 +1,212 @@
+"""torch.Tensor <-> tv.Tensor without copies, and autograd functions around the mask-based sparse
+convolution (forward = implicit_gemm2 Forward, backward = BackwardInput + BackwardWeight).
+
+``torch2tensor`` / ``tensor2torch`` stand where the reference's ``PyTorchTools.torch2tensor`` /
+``tensor2torch`` do (cumm/bindings.py:53-86 over include/tensorview/torch_utils.h).  torch is
+plumbing here: it owns activations, parameters and the stream; every kernel that runs is this
+library's.  Imported on demand: nothing else in the package needs torch.
+"""
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import pairs, tuner
+from . import tensorview as tv
+from .conv.main import ConvMainUnitTest
+from .tensorview.gemm import Activation, ConvOpType, ConvParams
+
+_TORCH_TO_TV = {torch.float32: tv.float32, torch.float16: tv.float16, torch.bfloat16: tv.bfloat16,
+                torch.int32: tv.int32, torch.int8: tv.int8, torch.uint8: tv.uint8, torch.int64: tv.int64,
+                torch.int16: tv.int16, torch.float64: tv.float64, torch.bool: tv.bool_}
+_TV_TO_TORCH = {v: k for k, v in _TORCH_TO_TV.items()}
+# torch has no full unsigned support: tensor2torch(cast_uint_to_int=True) views them as signed
+_UINT_AS_INT = {tv.uint32: torch.int32, tv.uint16: torch.int16, tv.uint64: torch.int64}
+_TYPESTR = {torch.float32: "<f4", torch.float16: "<f2", torch.int32: "<i4", torch.int8: "|i1", torch.uint8: "|u1",
+            torch.int64: "<i8", torch.int16: "<i2", torch.float64: "<f8", torch.bool: "|b1"}
+
+
+def torch2tensor(t: torch.Tensor) -> tv.Tensor:
+    """A tv.Tensor over the storage of ``t`` (any strides); ``t`` is kept alive by the view."""
+    if t.dtype not in _TORCH_TO_TV:
+        raise ValueError("unsupported torch dtype %s" % t.dtype)
+    device = t.device.index if t.is_cuda else -1
+    if t.is_cuda and device is None:
+        device = torch.cuda.current_device()
+    return tv.from_blob_strided(t.data_ptr(), list(t.shape), list(t.stride()), _TORCH_TO_TV[t.dtype], device,
+                                keepalive=t)
+
+
+class _DeviceArray:
+    """What torch.as_tensor needs to wrap device memory in place."""
+
+    def __init__(self, ten: tv.Tensor, typestr: str, itemsize: int):
+        self._keep = ten
+        self.__cuda_array_interface__ = {
+            "shape": tuple(ten.shape), "typestr": typestr, "data": (ten.byte_pointer(), False), "version": 2,
+            "strides": tuple(s * itemsize for s in ten.stride)}
+
+
+def tensor2torch(ten: tv.Tensor, clone: bool = True, cast_uint_to_int: bool = False) -> torch.Tensor:
+    """The reference's signature (clone=True copies; clone=False shares the memory and keeps ``ten``
+    alive)."""
+    dt = ten.dtype
+    if dt in _UINT_AS_INT:
+        if not cast_uint_to_int:
+            raise ValueError("torch has no such unsigned type: pass cast_uint_to_int=True")
+        tdt = _UINT_AS_INT[dt]
+    elif dt in _TV_TO_TORCH:
+        tdt = _TV_TO_TORCH[dt]
+    else:
+        raise ValueError("unsupported tv dtype %d" % dt)
+    if ten.empty():
+        return torch.empty(list(ten.shape), dtype=tdt, device="cuda" if ten.device >= 0 else "cpu")
+    if ten.device < 0:
+        arr = ten.numpy_view()
+        res = torch.from_numpy(arr).view(tdt) if tdt != torch.bfloat16 else torch.from_numpy(arr).view(torch.bfloat16)
+    else:
+        carrier = torch.int16 if tdt == torch.bfloat16 else tdt
+        res = torch.as_tensor(_DeviceArray(ten, _TYPESTR[carrier], ten.itemsize), device="cuda:%d" % ten.device)
+        if tdt == torch.bfloat16:
+            res = res.view(torch.bfloat16)
+    return res.clone() if clone else res
+
+
+def current_stream() -> int:
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+_TUNER = tuner.Tuner(steps=3, warmup=1)
+
+
+def _desp_like(dtype, op, parallel=False):
+    for d in ConvMainUnitTest.get_all_conv_algo_desp():
+        if (d.dtype_a == dtype and ConvOpType(d.op_type) == op and not d.is_int8_inference and
+                bool(d.split_k_parallel) == parallel and d.mask_sparse):
+            return d
+    raise RuntimeError("can't find any suitable algo for your parameters.")
+
+
+class SparseConvGeometry:
+    """Pair tables, masks and sorts of one convolution geometry, built on the GPU once and shared by
+    every layer (and every pass) that uses it."""
+
+    def __init__(self, coords: torch.Tensor, spatial_shape: Sequence[int], ksize=(3, 3, 3), stride=None,
+                 padding=(1, 1, 1), dilation=(1, 1, 1), batch_size: int = 1):
+        if coords.dtype != torch.int32 or not coords.is_cuda or coords.dim() != 2 or coords.shape[1] != 4:
+            raise ValueError("coords must be a cuda int32 tensor [N, 4] of (batch, z, y, x)")
+        coords = coords.contiguous()
+        stream = current_stream()
+        c_tv = torch2tensor(coords)
+        self.subm = stride is None
+        self.n_in = int(coords.shape[0])
+        self.kv = int(ksize[0]) * int(ksize[1]) * int(ksize[2])
+        if self.subm:
+            t = pairs.subm_pairs_device(c_tv, spatial_shape, ksize, dilation, stream=stream)
+            self.out_coords, self.out_shape = coords, tuple(int(s) for s in spatial_shape)
+        else:
+            t = pairs.sparse_conv_pairs_device(c_tv, spatial_shape, ksize, stride, padding, dilation,
+                                               batch_size=batch_size, stream=stream)
+            self.out_coords, self.out_shape = tensor2torch(t.out_coords, clone=False), t.out_shape
+        self.indices_fwd, self.indices_bwd = t.indices_fwd, t.indices_bwd
+        self.n_out = int(t.indices_fwd.dim(1))
+        self.mask_fwd, self.order_fwd = pairs.sort_by_mask_device(t.mask_fwd, stream=stream)
+        if self.subm:      # the forward masks serve the backward-input pass, bit-reversed in the kernel
+            self.mask_bwd, self.order_bwd = self.mask_fwd, self.order_fwd
+        else:
+            self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, stream=stream)
+        self._reduced = {}
+
+    def reduced_mask(self, width: int) -> tv.Tensor:
+        """OR of the sorted forward masks over runs of ``width`` positions (backward-weight)."""
+        if width not in self._reduced:
+            m = tensor2torch(self.mask_fwd, clone=False, cast_uint_to_int=True)
+            tiles = (self.n_out + width - 1) // width
+            padded = torch.zeros(tiles * width, dtype=torch.int32, device=m.device)
+            padded[: self.n_out] = m
+            red = padded.view(tiles, width)
+            while red.shape[1] > 1:
+                half = red.shape[1] // 2
+                red = torch.bitwise_or(red[:, :half], red[:, half:2 * half]) if red.shape[1] % 2 == 0 else \
+                    torch.cat([torch.bitwise_or(red[:, :half], red[:, half:2 * half]), red[:, 2 * half:]], dim=1)
+            red = red.reshape(tiles).contiguous()
+            self._reduced[width] = (torch2tensor(red).type_view(tv.uint32), red)
+        return self._reduced[width][0]
+
+
+class _SparseConvFunction(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, features, weight, bias, geometry: SparseConvGeometry, relu: bool):
+        features, weight = features.contiguous(), weight.contiguous()
+        dtype = _TORCH_TO_TV[features.dtype]
+        out = torch.empty((geometry.n_out, weight.shape[0]), dtype=features.dtype, device=features.device)
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = _desp_like(dtype, ConvOpType.Forward)
+        p.input, p.weight, p.output = torch2tensor(features), torch2tensor(weight), torch2tensor(out)
+        p.indices, p.mask, p.mask_argsort = geometry.indices_fwd, geometry.mask_fwd, geometry.order_fwd
+        if bias is not None:
+            p.bias, p.beta = torch2tensor(bias.contiguous()), 1.0
+        if relu:
+            p.act_type = Activation.ReLU
+        p.stream = current_stream()
+        _TUNER.tune_conv(p)
+        ConvMainUnitTest.implicit_gemm2(p)
+        ctx.geometry, ctx.relu, ctx.has_bias = geometry, relu, bias is not None
+        ctx.save_for_backward(features, weight, out if relu else None)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        features, weight, out = ctx.saved_tensors
+        g: SparseConvGeometry = ctx.geometry
+        grad_out = grad_out.contiguous()
+        if ctx.relu:
+            grad_out = grad_out * (out > 0).to(grad_out.dtype)
+        dtype = _TORCH_TO_TV[features.dtype]
+        stream = current_stream()
+        grad_in = grad_w = grad_b = None
+        if ctx.needs_input_grad[0]:
+            grad_in = torch.empty_like(features)
+            p = ConvParams(3, ConvOpType.BackwardInput)
+            p.conv_algo_desp = _desp_like(dtype, ConvOpType.BackwardInput)
+            p.input, p.weight, p.output = torch2tensor(grad_in), torch2tensor(weight), torch2tensor(grad_out)
+            p.indices, p.mask, p.mask_argsort = g.indices_bwd, g.mask_bwd, g.order_bwd
+            p.reverse_mask = g.subm
+            p.stream = stream
+            _TUNER.tune_conv(p)
+            ConvMainUnitTest.implicit_gemm2(p)
+        if ctx.needs_input_grad[1]:
+            grad_w = torch.empty_like(weight)
+            p = ConvParams(3, ConvOpType.BackwardWeight)
+            p.conv_algo_desp = _desp_like(dtype, ConvOpType.BackwardWeight, parallel=True)
+            p.input, p.weight, p.output = torch2tensor(features), torch2tensor(grad_w), torch2tensor(grad_out)
+            p.indices, p.mask, p.mask_argsort = g.indices_fwd, g.reduced_mask(64), g.order_fwd
+            p.mask_width, p.split_k_slices = 64, 32
+            p.stream = stream
+            ConvMainUnitTest.implicit_gemm2(p)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            grad_b = grad_out.float().sum(0).to(grad_out.dtype)
+        return grad_in, grad_w, grad_b, None, None
+
+
+def sparse_conv(features: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                geometry: SparseConvGeometry, relu: bool = False) -> torch.Tensor:
+    """features [N_in, C], weight [K, kv, C] (f16 / bf16, cuda) -> [N_out, K]; differentiable in
+    features, weight and bias."""
+    return _SparseConvFunction.apply(features, weight, bias, geometry, relu)
+
+
+class SparseConv3d(torch.nn.Module):
+    """A layer over :func:`sparse_conv`: submanifold when its geometry was built without a stride."""
+
+    def __init__(self, in_channels: int, out_channels: int, ksize=(3, 3, 3), bias: bool = True, relu: bool = False,
+                 dtype=torch.float16, device="cuda"):
+        super().__init__()
+        kv = int(ksize[0]) * int(ksize[1]) * int(ksize[2])
+        w = torch.randn(out_channels, kv, in_channels, device=device) * (2.0 / (kv * in_channels)) ** 0.5
+        self.weight = torch.nn.Parameter(w.to(dtype))
+        self.bias = torch.nn.Parameter(torch.zeros(out_channels, dtype=dtype, device=device)) if bias else None
+        self.relu = relu
+
+    def forward(self, features: torch.Tensor, geometry: SparseConvGeometry) -> torch.Tensor:
+        return sparse_conv(features, self.weight, self.bias, geometry, self.relu)
