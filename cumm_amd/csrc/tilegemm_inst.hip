@@ -91,10 +91,15 @@ hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const
     hipLaunchKernelGGL(wgrad_prepare_kernel, dim3(p.kv + 256), dim3(256), 0, s, pre);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
+    // With several 64 x 64 channel blocks a unit either takes one of them (more units: small
+    // inputs) or walks them all on one set of pair lists (the centre offset alone then gives
+    // `groups` units: enough when that fills the device).
+    WgradParams q = p;
+    q.merge_blocks = kblocks * cblocks > 1 && groups >= resident ? 1 : 0;
     // never more workgroups than units can exist
-    const long long max_units = ((long long)groups * p.kv + p.kv) * kblocks * cblocks;
+    const long long max_units = ((long long)groups * p.kv + p.kv) * (q.merge_blocks ? 1 : kblocks * cblocks);
     hipLaunchKernelGGL((wgrad_units_kernel<T>), dim3((unsigned)(max_units < resident ? max_units : resident)),
-                       dim3(256), 0, s, p);
+                       dim3(256), 0, s, q);
   } else {
     dim3 grid(groups, p.kv * kblocks * cblocks, 1);
     hipLaunchKernelGGL((wgrad_atomic_kernel<T>), grid, dim3(256), 0, s, p);

@@ -47,6 +47,9 @@ struct WgradParams {
   // image_floats apart; the finalize kernel sums them
   int32_t images;
   int64_t image_floats;
+  // one unit walks all 64 x 64 channel blocks of its positions in turn (the pair lists are made
+  // once) instead of one block per unit; set by the launcher when the units are many anyway
+  int32_t merge_blocks;
 };
 
 constexpr int kWgradMaxPos = 1024;  // positions one workgroup handles at most (QT * mask_width)
@@ -311,7 +314,8 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   const int l16 = lane & 15, q = lane >> 4;
 
   const int kblocks = (p.K + 63) / 64, cblocks = (p.C + 63) / 64;
-  const int per_r = kblocks * cblocks;
+  const int per_r = p.merge_blocks ? 1 : kblocks * cblocks;
+  const int combos = p.merge_blocks ? kblocks * cblocks : 1;
   // units of offset r: its workgroups (ceil(live / QT)) times the channel blocks.  Lane r of every
   // wave holds offset r's numbers (kv <= 32: one mask bit per offset); a prefix sum over the
   // lanes and a ballot locate a unit without a loop over memory.
@@ -447,6 +451,11 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     // Step s waits for its own stage, passes the barrier (everybody's loads of step s have
     // landed, everybody is done with step s-1), reads its operands, refills the stage of step
     // s-1 with step s+NS-1, computes.
+    for (int combo = 0; combo < combos; ++combo) {
+    if (p.merge_blocks) {
+      kb = fast_div(combo, cblocks);
+      cb = combo - kb * cblocks;
+    }
     const int ych = kb * 64 + (schunk ^ swz(srow)) * 8, xch = cb * 64 + (schunk ^ swz(srow)) * 8;
     auto offsets = [&](int t, uint32_t (&yoff)[H], uint32_t (&xoff)[H]) __attribute__((always_inline)) {
 #pragma unroll
@@ -538,6 +547,8 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
         }
       }
     }
+    lds_barrier();     // every wave is done with the ring before the next block's loads land in it
+    }  // channel blocks
     __syncthreads();   // the LDS lists and the ring are rewritten by the next unit
   }
 }
