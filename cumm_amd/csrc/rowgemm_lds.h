@@ -118,8 +118,27 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     else return ix3[wave];
   };
 
-  const int tile = (int)gridDim.x - 1 - (int)blockIdx.x;  // heaviest tiles first (masks sorted ascending)
-  const int n0 = blockIdx.y * TN;
+  // Workgroups are dispatched in the order of their linear number, round-robin over the 8 XCDs.
+  // With several column blocks per row tile, the workgroups of one row tile are given numbers 8
+  // apart - neighbours in time on one XCD - so that the rows one of them gathers are in that
+  // XCD's L2 for the others (as grid.y they would run a whole grid.x apart).
+  int tile_rank = (int)blockIdx.x, col = 0;
+  if (gridDim.y > 1) {
+    const int gx = (int)gridDim.x, gy = (int)gridDim.y;
+    const int lin = (int)blockIdx.y * gx + (int)blockIdx.x;
+    const int gx8 = gx & ~7;
+    if (lin < gx8 * gy) {
+      const int slot = lin >> 3;
+      tile_rank = (slot / gy) * 8 + (lin & 7);
+      col = slot % gy;
+    } else {
+      const int rest = lin - gx8 * gy;
+      tile_rank = gx8 + rest / gy;
+      col = rest % gy;
+    }
+  }
+  const int tile = (int)gridDim.x - 1 - tile_rank;  // heaviest tiles first (masks sorted ascending)
+  const int n0 = col * TN;
   const int pos_base = tile * TM;
 
   // ---- the tile's mask words are requested first and reduced only after the row keys below have
@@ -229,7 +248,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   uint32_t kmask = 1u;
   if (has_mask) {
     kmask = wave_or_dpp(mk) & p.mask_filter;
-    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
+    if (p.mask_out != nullptr && tid == 0 && col == 0) p.mask_out[tile] = kmask;
     if (p.exit_on_empty && kmask == 0) return;
     if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
     if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
