@@ -12,6 +12,7 @@ the forward kernel and a CPU baseline (the numpy oracle) timed on the host cores
 """
 import argparse
 import json
+import re
 import os
 import sys
 import time
@@ -134,9 +135,14 @@ def bench_gather_gemm(args):
     pg.a_inds = dev(rng2.permutation(rows)[:m].astype(np.int32))
     pg.c_inds = dev(rng2.permutation(rows)[:m].astype(np.int32))
     pg.alpha, pg.beta = 1.0, 1.0
+    from cumm_amd import tuner
+    best = tuner.Tuner(steps=10, warmup=2).tune_gemm(pg)     # the caller's descriptor choice, by timing
     w_ms, e_ms = timed(lambda: GemmMainUnitTest.matmul2(pg), args.steps, args.warmup)
     nbytes = m * k * 2 + 2 * m * n * 2 + k * n * 2 + 2 * m * 4
-    return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
+    return {"tile": list(best.desp.tile_shape[:2]),
+            "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
+                           for nm, ms in best.tried},
+            "ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
             "tflops": round(2.0 * m * n * k / (w_ms * 1e-3) / 1e12, 3),
             "hbm_frac": round(nbytes / (e_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
@@ -336,10 +342,15 @@ def bench_s8(args, tile_m):
     p4.scale = dev(rng4.uniform(0.001, 0.01, size=(128,)).astype(np.float32))
     p4.bias = dev(rng4.normal(0, 1, size=(128,)).astype(np.float32))
     p4.indices, p4.mask, p4.mask_argsort = dev(pt4.indices_fwd), dev(ms4), dev(as4)
+    from cumm_amd import tuner
+    best = tuner.Tuner(steps=10, warmup=2).tune_conv(p4)     # the caller's descriptor choice, by timing
     w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(p4), args.steps, args.warmup)
     ops4 = 2.0 * P4 * 64 * 128
     bytes4 = n_in4 * 64 + n_out4 * 128 + 27 * 64 * 128 + 27 * n_out4 * 4 + n_out4 * 8 + 2 * 128 * 4
     return {"voxels_in": n_in4, "voxels_out": n_out4, "active_pairs": P4,
+            "tile": list(best.desp.tile_shape[:2]),
+            "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
+                           for nm, ms in best.tried},
             "ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
             "tops": round(ops4 / (w_ms * 1e-3) / 1e12, 3),
             "pct_mfma_i8_peak": round(100.0 * ops4 / (w_ms * 1e-3) / 1e12 / PEAK_MFMA_I8_TOPS, 3),
