@@ -283,3 +283,73 @@ def test_ragged_and_empty():
         ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64,
                                                 dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
         assert H.rel_err(H.as_f32(H.host(p.output), dtype), H.as_f32(ref, dtype)) < TOL
+
+
+@pytest.mark.parametrize("geometry", [
+    ("subm", (1, 3, 3), None, None),
+    ("subm", (3, 1, 1), None, None),
+    ("subm", (1, 1, 1), None, None),
+    ("strided", (2, 2, 2), (2, 2, 2), (0, 0, 0)),
+    ("strided", (2, 4, 4), (1, 2, 2), (0, 1, 1)),          # kernel volume 32: every mask bit in use
+    ("strided", (3, 3, 3), (1, 1, 1), (1, 1, 1)),          # stride 1: a regular convolution on all sites
+])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_kernel_volumes_forward_and_backward(dtype, geometry):
+    """Kernel volumes other than 27 (1 to 32 offsets) through all three passes."""
+    kind, ksize, stride, padding = geometry
+    print("case kernel volume", dtype, geometry, flush=True)
+    rng = np.random.default_rng(31)
+    grid = (10, 24, 20)
+    coords = synth.clustered_voxels(rng, 2200, grid, 5, sigma=3.0)
+    if kind == "subm":
+        pt = pairs.subm_pairs(coords, grid, ksize)
+    else:
+        pt = pairs.sparse_conv_pairs(coords, grid, ksize, stride, padding)
+    kv = ksize[0] * ksize[1] * ksize[2]
+    n_in, n_out = coords.shape[0], pt.indices_fwd.shape[1]
+    c_in, k_out, tile = 64, 96, (64, 64)
+    feat = H.to_storage(rng.normal(0, 1, size=(n_in, c_in)).astype(np.float32), dtype)
+    w = H.to_storage(rng.normal(0, 0.1, size=(k_out, kv, c_in)).astype(np.float32), dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    zero_out = H.to_storage(np.zeros((n_out, k_out), np.float32), dtype)
+
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, *tile)
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(zero_out, dtype)
+    p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_fwd, "i32"), H.dev(ms, "u32"), H.dev(order, "i32")
+    p.mask_output = tv.zeros([(n_out + 63) // 64], tv.uint32, 0)
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, zero_out, pt.indices_fwd, ms, order, tile_m=64,
+                                                 dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+    assert H.rel_err(H.as_f32(H.host(p.output), dtype), H.as_f32(ref, dtype)) < TOL
+    np.testing.assert_array_equal(H.host(p.mask_output), ref_mo)
+
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    zero_in = H.to_storage(np.zeros((n_in, c_in), np.float32), dtype)
+    if kind == "subm":
+        msb, orderb, reverse = ms, order, True
+    else:
+        msb, orderb = pairs.sort_by_mask(pt.mask_bwd)
+        reverse = False
+    pd = ConvParams(3, ConvOpType.BackwardInput)
+    pd.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, *tile)
+    pd.input, pd.weight, pd.output = H.dev(zero_in, dtype), p.weight, H.dev(dout, dtype)
+    pd.indices, pd.mask, pd.mask_argsort = H.dev(pt.indices_bwd, "i32"), H.dev(msb, "u32"), H.dev(orderb, "i32")
+    pd.reverse_mask = reverse
+    ConvMainUnitTest.implicit_gemm2(pd)
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, zero_in, pt.indices_bwd, msb, orderb, tile_m=64, dtype_in=dtype,
+                                             dtype_w=dtype, dtype_out=dtype, reverse_mask=reverse)
+    assert H.rel_err(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_d, dtype)) < TOL
+
+    red = conv_ref.tile_masks(ms, 64)
+    zero_w = H.to_storage(np.zeros((k_out, kv, c_in), np.float32), dtype)
+    ref_w = conv_ref.implicit_gemm_wgrad_ref(dout, feat, zero_w, pt.indices_fwd, red, order, mask_width=64,
+                                             dtype_dout=dtype, dtype_in=dtype, dtype_w=dtype, split_k_slices=1)
+    for parallel in (True, False):
+        pw = ConvParams(3, ConvOpType.BackwardWeight)
+        pw.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=parallel)
+        pw.input, pw.weight, pw.output = p.input, H.dev(zero_w, dtype), pd.output
+        pw.indices, pw.mask, pw.mask_argsort = p.indices, H.dev(red, "u32"), p.mask_argsort
+        pw.mask_width, pw.split_k_slices = 64, 4 if parallel else 1
+        ConvMainUnitTest.implicit_gemm2(pw)
+        assert H.rel_err(H.as_f32(H.host(pw.weight), dtype), H.as_f32(ref_w, dtype)) < TOL
