@@ -353,3 +353,56 @@ def test_kernel_volumes_forward_and_backward(dtype, geometry):
         pw.mask_width, pw.split_k_slices = 64, 4 if parallel else 1
         ConvMainUnitTest.implicit_gemm2(pw)
         assert H.rel_err(H.as_f32(H.host(pw.weight), dtype), H.as_f32(ref_w, dtype)) < TOL
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("act,act_alpha", [(Activation.Sigmoid, 0.0), (Activation.LeakyReLU, 0.1),
+                                           (Activation.LeakyReLU, 0.0)])
+def test_forward_sigmoid_and_leaky_relu(dtype, act, act_alpha):
+    """The other two activations of the epilogue (UnaryActivation, cumm/gemm/gemmmath/__init__.py:181-214),
+    with a bias, on the LDS-streaming kernel (64 channels) and on the chunked one (160 channels)."""
+    print("case activation", dtype, act, act_alpha, flush=True)
+    for c_in, k_out, tile in ((64, 64, (64, 64)), (160, 96, (128, 128))):
+        rng, coords, pt, feat, w, n_in, n_out = _case(41, 2500, c_in, k_out, dtype)
+        bias = H.to_storage(rng.normal(0, 0.5, size=(k_out,)).astype(np.float32), dtype)
+        ms, order = pairs.sort_by_mask(pt.mask_fwd)
+        out0 = H.to_storage(np.zeros((n_out, k_out), np.float32), dtype)
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, *tile)
+        p.input, p.weight, p.output, p.bias = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype), H.dev(bias, dtype)
+        p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_fwd, "i32"), H.dev(ms, "u32"), H.dev(order, "i32")
+        p.beta, p.act_type, p.act_alpha = 1.0, act, act_alpha
+        ConvMainUnitTest.implicit_gemm2(p)
+        ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=tile[0],
+                                                dtype_in=dtype, dtype_w=dtype, dtype_out=dtype, bias=bias, beta=1.0,
+                                                act=act.value, act_alpha=act_alpha)
+        got, want = H.as_f32(H.host(p.output), dtype), H.as_f32(ref, dtype)
+        assert H.rel_err(got, want) < TOL
+        if act == Activation.Sigmoid:
+            assert 0.0 <= got.min() and got.max() <= 1.0 and 0.3 < got.mean() < 0.7
+        elif act_alpha == 0.1:
+            assert got.min() < 0.0       # negative values pass, scaled
+
+
+@pytest.mark.parametrize("act_alpha", [0.1, 0.25])
+def test_int8_inference_leaky_relu_bit_exact(act_alpha):
+    print("case int8 leaky relu", act_alpha, flush=True)
+    c_in, k_out = 64, 128
+    rng, coords, pt, feat, w, n_in, n_out = _case(43, 3000, c_in, k_out, "s8", strided=True)
+    scale = rng.uniform(0.001, 0.01, size=(k_out,)).astype(np.float32)
+    bias = rng.normal(0, 1, size=(k_out,)).astype(np.float32)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    out0 = np.zeros((n_out, k_out), np.int8)
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = H.find_conv_desp("s8", ConvOpType.Forward, 64, 128, int8_inference=True)
+    p.input, p.weight, p.output = H.dev(feat, "s8"), H.dev(w, "s8"), H.dev(out0, "s8")
+    p.scale, p.bias = H.dev(scale, "f32"), H.dev(bias, "f32")
+    p.act_type, p.act_alpha = Activation.LeakyReLU, act_alpha
+    p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_fwd, "i32"), H.dev(ms, "u32"), H.dev(order, "i32")
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in="s8",
+                                            dtype_w="s8", dtype_out="s8", scale=scale, bias=bias,
+                                            act=Activation.LeakyReLU.value, act_alpha=act_alpha, int8_inference=True)
+    got = H.host(p.output)
+    np.testing.assert_array_equal(got, ref)
+    assert (got < 0).any() and (got > 0).any()
