@@ -71,20 +71,25 @@ hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const
                                                      const WgradFinalizeParams &f, hipStream_t s) {
   using T = CUMM_ELEM;
   const int groups = (p.num_red + p.tiles_per_wg - 1) / p.tiles_per_wg;
-  const int kblocks = (p.K + 63) / 64, cblocks = (p.C + 63) / 64;
+  // both channel counts above 64: units of 128 x 128 channels (one gather of the full rows)
+  const bool wide = p.live_list != nullptr && p.K > 64 && p.C > 64;
+  const int cpu_ = wide ? 128 : 64;   // channels per unit block
+  const int kblocks = (p.K + cpu_ - 1) / cpu_, cblocks = (p.C + cpu_ - 1) / cpu_;
   if (groups == 0 || p.kv == 0) return hipSuccess;
   hipError_t e;
   if (p.live_list != nullptr) {
     // lists + zeroed image, then a resident grid that walks the units
-    static int resident_of[16] = {};
+    static int resident_of[2][16] = {};
     int dev = 0;
     e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    int &resident = resident_of[dev & 15];
+    int &resident = resident_of[wide ? 1 : 0][dev & 15];
     if (resident == 0) {
       int cus = 0, per_cu = 0;
       e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-      if (e == hipSuccess) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wgrad_units_kernel<T>, 256, 0);
+      if (e == hipSuccess)
+        e = wide ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wgrad_units_kernel<T, 2, 2, 1>, 256, 0)
+                 : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wgrad_units_kernel<T, 1, 1, 2>, 256, 0);
       if (e != hipSuccess) return e;
       resident = cus * per_cu > 0 ? cus * per_cu : 1;
     }
@@ -98,8 +103,9 @@ hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const
     q.merge_blocks = kblocks * cblocks > 1 && groups >= resident ? 1 : 0;
     // never more workgroups than units can exist
     const long long max_units = ((long long)groups * p.kv + p.kv) * (q.merge_blocks ? 1 : kblocks * cblocks);
-    hipLaunchKernelGGL((wgrad_units_kernel<T>), dim3((unsigned)(max_units < resident ? max_units : resident)),
-                       dim3(256), 0, s, q);
+    const dim3 units_grid((unsigned)(max_units < resident ? max_units : resident));
+    if (wide) hipLaunchKernelGGL((wgrad_units_kernel<T, 2, 2, 1>), units_grid, dim3(256), 0, s, q);
+    else hipLaunchKernelGGL((wgrad_units_kernel<T, 1, 1, 2>), units_grid, dim3(256), 0, s, q);
   } else {
     dim3 grid(groups, p.kv * kblocks * cblocks, 1);
     hipLaunchKernelGGL((wgrad_atomic_kernel<T>), grid, dim3(256), 0, s, p);

@@ -293,15 +293,22 @@ __device__ __forceinline__ int wave_prefix_sum_dpp(int v) {
   return v;
 }
 
-template <class T>
+// KB, CB = 64-channel blocks of dOut (K) and of In (C) that a unit multiplies in one pass, H =
+// 32-pair halves per step.  <1, 1, 2> is the unit described above.  <2, 2, 1> takes 128 x 128
+// channels: the full 256-byte rows of a pair are gathered once instead of one 128-byte half per
+// 64 x 64 block (four gathers of each pair at C = K = 128, where the launch is bound by that
+// traffic once dOut and In no longer fit the last-level cache); its stage holds 32 pairs (16 KB,
+// four stages, still two workgroups per CU) and a wave accumulates 64 x 64.
+template <class T, int KB, int CB, int H>
 __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   using E = Elem<T>;
-  constexpr int H = 2;                // 32-pair halves per step
   constexpr int TK = 32 * H;          // pairs per step
   constexpr int NS = 4, L = NS - 1;   // ring stages, steps the loads run ahead
-  constexpr int HALF = 8192;          // dOut tile (32 rows x 128 bytes), then the In tile
+  constexpr int PART = 4096;          // one tile: 32 rows x 128 bytes
+  constexpr int HALF = (KB + CB) * PART;   // the dOut tiles, then the In tiles
   constexpr int STAGE = H * HALF;
   constexpr int MAXIT = kWgradMaxPos / 256;
+  constexpr int NJ = 2 * KB, NI = 2 * CB;   // 16-channel blocks of dOut / In per wave
   __shared__ __attribute__((aligned(16))) char ring[NS * STAGE];
   __shared__ int lds_o[kWgradMaxPos + TK];
   __shared__ int lds_i[kWgradMaxPos + TK];
@@ -313,7 +320,7 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   const int wm = wave >> 1, wn = wave & 1;
   const int l16 = lane & 15, q = lane >> 4;
 
-  const int kblocks = (p.K + 63) / 64, cblocks = (p.C + 63) / 64;
+  const int kblocks = (p.K + 64 * KB - 1) / (64 * KB), cblocks = (p.C + 64 * CB - 1) / (64 * CB);
   const int per_r = p.merge_blocks ? 1 : kblocks * cblocks;
   const int combos = p.merge_blocks ? kblocks * cblocks : 1;
   // units of offset r: its workgroups (ceil(live / QT)) times the channel blocks.  Lane r of every
@@ -332,16 +339,23 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   const int srow = tid >> 3, schunk = tid & 7;
   auto swz = [](int row) { return 2 * ((row >> 1) & 3); };
   const uint32_t ring_at = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_addr(ring) + wave * 1024));
-  int y_rd[2][2], x_rd[2][2];   // [half h][16-channel block of this wave]
+  int y_rd[2][NJ], x_rd[2][NI];   // [4-row group h of a read pair][16-channel block of this wave]
 #pragma unroll
-  for (int h = 0; h < 2; ++h)
+  for (int h = 0; h < 2; ++h) {
+    const int row = q * 8 + h * 4 + (l16 >> 2);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int row = q * 8 + h * 4 + (l16 >> 2);
-      const int ycol = (wm * 2 + j) * 16 + 4 * (l16 & 3), xcol = (wn * 2 + j) * 16 + 4 * (l16 & 3);
-      y_rd[h][j] = row * 128 + (((ycol >> 3) ^ swz(row)) * 16) + (ycol & 7) * 2;
-      x_rd[h][j] = HALF / 2 + row * 128 + (((xcol >> 3) ^ swz(row)) * 16) + (xcol & 7) * 2;
+    for (int j = 0; j < NJ; ++j) {
+      const int g = wm * NJ + j;   // 16-channel block among the unit's 4 * KB: tile g / 4, column block g % 4
+      const int ycol = (g & 3) * 16 + 4 * (l16 & 3);
+      y_rd[h][j] = (g >> 2) * PART + row * 128 + (((ycol >> 3) ^ swz(row)) * 16) + (ycol & 7) * 2;
     }
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int g = wn * NI + j;
+      const int xcol = (g & 3) * 16 + 4 * (l16 & 3);
+      x_rd[h][j] = (KB + (g >> 2)) * PART + row * 128 + (((xcol >> 3) ^ swz(row)) * 16) + (xcol & 7) * 2;
+    }
+  }
 
   // (the address arithmetic above runs while the counts are on their way)
   const int my_wgs = fast_div(my_live + p.tiles_per_wg - 1, p.tiles_per_wg);
@@ -456,70 +470,82 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
       kb = fast_div(combo, cblocks);
       cb = combo - kb * cblocks;
     }
-    const int ych = kb * 64 + (schunk ^ swz(srow)) * 8, xch = cb * 64 + (schunk ^ swz(srow)) * 8;
-    auto offsets = [&](int t, uint32_t (&yoff)[H], uint32_t (&xoff)[H]) __attribute__((always_inline)) {
+    const int ych = kb * (64 * KB) + (schunk ^ swz(srow)) * 8, xch = cb * (64 * CB) + (schunk ^ swz(srow)) * 8;
+    auto offsets = [&](int t, uint32_t (&yoff)[H][KB], uint32_t (&xoff)[H][CB]) __attribute__((always_inline)) {
 #pragma unroll
       for (int hh = 0; hh < H; ++hh) {
-        yoff[hh] = 0x80000000u;
-        xoff[hh] = 0x80000000u;
+#pragma unroll
+        for (int pp = 0; pp < KB; ++pp) yoff[hh][pp] = 0x80000000u;
+#pragma unroll
+        for (int pp = 0; pp < CB; ++pp) xoff[hh][pp] = 0x80000000u;
         if (t < n_steps) {
           const int o = lds_o[t * TK + hh * 32 + srow], i = lds_i[t * TK + hh * 32 + srow];
           if (o >= 0) {
-            if (ych < p.K) yoff[hh] = (uint32_t)(o * p.K + ych) * 2u;
-            if (xch < p.C) xoff[hh] = (uint32_t)(i * p.C + xch) * 2u;
+#pragma unroll
+            for (int pp = 0; pp < KB; ++pp)
+              if (ych + pp * 64 < p.K) yoff[hh][pp] = (uint32_t)(o * p.K + ych + pp * 64) * 2u;
+#pragma unroll
+            for (int pp = 0; pp < CB; ++pp)
+              if (xch + pp * 64 < p.C) xoff[hh][pp] = (uint32_t)(i * p.C + xch + pp * 64) * 2u;
           }
         }
       }
     };
-    auto issue = [&](int t, const uint32_t (&yoff)[H], const uint32_t (&xoff)[H]) __attribute__((always_inline)) {
+    auto issue = [&](int t, const uint32_t (&yoff)[H][KB], const uint32_t (&xoff)[H][CB]) __attribute__((always_inline)) {
       const uint32_t dst = ring_at + (uint32_t)__builtin_amdgcn_readfirstlane((t % NS) * STAGE);
 #pragma unroll
       for (int hh = 0; hh < H; ++hh) {
-        dma_b128(y_rsrc, dst + hh * HALF, yoff[hh], 0);
-        dma_b128(x_rsrc, dst + hh * HALF + HALF / 2, xoff[hh], 0);
+#pragma unroll
+        for (int pp = 0; pp < KB; ++pp) dma_b128(y_rsrc, dst + hh * HALF + pp * PART, yoff[hh][pp], 0);
+#pragma unroll
+        for (int pp = 0; pp < CB; ++pp) dma_b128(x_rsrc, dst + hh * HALF + (KB + pp) * PART, xoff[hh][pp], 0);
       }
     };
 
-    v4f acc[2][2];
+    v4f acc[NJ][NI];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NJ; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = v4f{0, 0, 0, 0};
+      for (int j = 0; j < NI; ++j) acc[i][j] = v4f{0, 0, 0, 0};
 
     wait_vmcnt<0>();   // the previous unit's atomics: from here on the counter holds ring loads only
-    uint32_t yn[H], xn[H];
+    uint32_t yn[H][KB], xn[H][CB];
     for (int t = 0; t < L; ++t) {
       offsets(t, yn, xn);
       issue(t, yn, xn);
     }
     offsets(L, yn, xn);
     for (int s = 0; s < n_steps; ++s) {
-      wait_vmcnt<2 * H * (L - 1)>();
+      wait_vmcnt<(KB + CB) * H * (L - 1)>();
       lds_barrier();
       typedef short v4s __attribute__((ext_vector_type(4)));
       typedef __attribute__((address_space(3))) v4s *lds_v4s;
       const char *base = ring + (s % NS) * STAGE;
-      v4i xf[H][2], yf[H][2];
+      v4i xf[H][NI], yf[H][NJ];
 #pragma unroll
-      for (int hh = 0; hh < H; ++hh)
+      for (int hh = 0; hh < H; ++hh) {
+        const char *hb = base + hh * HALF;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const char *hb = base + hh * HALF;
+        for (int j = 0; j < NJ; ++j) {
           const v4s ylo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + y_rd[0][j]));
           const v4s yhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + y_rd[1][j]));
+          yf[hh][j] = __builtin_bit_cast(v4i, __builtin_shufflevector(ylo, yhi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
           const v4s xlo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + x_rd[0][j]));
           const v4s xhi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(hb + x_rd[1][j]));
-          yf[hh][j] = __builtin_bit_cast(v4i, __builtin_shufflevector(ylo, yhi, 0, 1, 2, 3, 4, 5, 6, 7));
           xf[hh][j] = __builtin_bit_cast(v4i, __builtin_shufflevector(xlo, xhi, 0, 1, 2, 3, 4, 5, 6, 7));
         }
+      }
       issue(s + L, yn, xn);
       offsets(s + L + 1, yn, xn);
 #pragma unroll
       for (int hh = 0; hh < H; ++hh)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < NJ; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = E::mfma(yf[hh][i], xf[hh][j], acc[i][j]);
+          for (int j = 0; j < NI; ++j) acc[i][j] = E::mfma(yf[hh][i], xf[hh][j], acc[i][j]);
     }
     wait_vmcnt<0>();   // the fetches past the end
 
@@ -532,14 +558,14 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
       const int64_t ldn = (int64_t)p.kv * p.C;
       float *image = p.scratch + (int64_t)(unit % p.images) * p.image_floats;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < NJ; ++i) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int nn = cb * 64 + (wn * 2 + j) * 16 + l16;
+        for (int j = 0; j < NI; ++j) {
+          const int nn = cb * (64 * CB) + (wn * NI + j) * 16 + l16;
           if (nn >= p.C) continue;
 #pragma unroll
           for (int x = 0; x < 4; ++x) {
-            const int mm = kb * 64 + (wm * 2 + i) * 16 + 4 * q + x;
+            const int mm = kb * (64 * KB) + (wm * NJ + i) * 16 + 4 * q + x;
             if (mm < p.K)
               __hip_atomic_fetch_add(image + mm * ldn + (int64_t)r * p.C + nn, acc[i][j][x],
                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

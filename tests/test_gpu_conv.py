@@ -175,7 +175,8 @@ def test_backward_weight(dtype, tile, split_k):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("shape", [(64, 64, 64), (64, 96, 128), (40, 72, 32)])
+@pytest.mark.parametrize("shape", [(64, 64, 64), (64, 96, 128), (40, 72, 32), (128, 128, 64), (72, 136, 64),
+                                   (160, 200, 32)])
 @pytest.mark.parametrize("strided", [False, True])
 def test_backward_weight_balanced_atomic(dtype, shape, strided):
     """The split_k_parallel descriptor: work balanced over live tiles, fp32 atomic partial sums;
