@@ -662,6 +662,9 @@ int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_sha
   p.filter = reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(workspace) + (size_t)pairs_slots(n) * 16);
   p.filter_mask = pairs_slots(n) - 1u;
   p.kx = ksize[2];
+  p.center_k = -1;
+  for (int k = 0; k < (int)kv; ++k)
+    if (p.off[k][0] == 0 && p.off[k][1] == 0 && p.off[k][2] == 0) p.center_k = k;
   hipError_t e = launch_subm_pairs(p, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "pair table launch");
   return CUMM_HIP_OK;

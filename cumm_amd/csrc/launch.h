@@ -44,6 +44,7 @@ struct SubmPairsParams {
   uint32_t *filter;        // (filter_mask + 1) presence words
   uint32_t filter_mask;
   int32_t kx;              // offsets along x (kv = kz * ky * kx)
+  int32_t center_k;        // the offset (0, 0, 0), whose pair is the voxel itself; -1 if there is none
 };
 hipError_t launch_subm_pairs(const SubmPairsParams &p, hipStream_t s);
 

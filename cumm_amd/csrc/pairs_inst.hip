@@ -55,8 +55,10 @@ __global__ __launch_bounds__(256) void pairs_clear_kernel(const SubmPairsParams 
   if (i <= p.slot_mask) reinterpret_cast<Slot *>(p.table)[i] = Slot{kEmptyKey, -1, 0};
   if (i <= p.filter_mask) p.filter[i] = 0u;
   if (i < (uint32_t)p.n) {
-    p.mask_f[i] = 0u;
-    if (p.mask_b) p.mask_b[i] = 0u;
+    // every voxel pairs with itself through the centre offset: that bit is set here, and the
+    // look-up kernel neither probes the table nor touches the masks for it
+    p.mask_f[i] = p.center_k >= 0 ? 1u << p.center_k : 0u;
+    if (p.mask_b) p.mask_b[i] = p.center_k >= 0 ? 1u << (p.kv - 1 - p.center_k) : 0u;
   }
 }
 
@@ -104,6 +106,11 @@ __global__ __launch_bounds__(256) void pairs_lookup_kernel(const SubmPairsParams
   uint32_t have_index = ~0u, word = 0;
   for (int kx = 0; kx < p.kx; ++kx) {
     const int k = zy * p.kx + kx;
+    if (k == p.center_k) {
+      p.ind_f[(int64_t)k * p.n + i] = i;
+      if (p.ind_b) p.ind_b[(int64_t)(p.kv - 1 - k) * p.n + i] = i;
+      continue;
+    }
     const int z = c.y + p.off[k][0], y = c.z + p.off[k][1], x = c.w + p.off[k][2];
     int row = -1;
     if (z >= 0 && z < p.shape[0] && y >= 0 && y < p.shape[1] && x >= 0 && x < p.shape[2]) {
