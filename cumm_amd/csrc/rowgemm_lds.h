@@ -340,7 +340,11 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
 #pragma unroll
         for (int nb = 0; nb < NBW; ++nb) {
           const int e = s * 32 + q * 8 + h * 4 + (m >> 2);
-          const int col = (wn * NBW + nb) * 16 + 4 * (m & 3);          // first channel (tile local)
+          // first channel (tile local) of the four this address lane points at.  Block nb takes
+          // channels 4*nb .. 4*nb+3 of every run of 4*NBW: the lane that holds rows 4q .. 4q+3 of
+          // the MFMA result then holds 4*NBW consecutive channels over its blocks (16-byte stores),
+          // like the fragment order of the untransposed weights
+          const int col = wn * (NBW * 16) + (m & 3) * (4 * NBW) + nb * 4;
           const int chunk = (col / PV) ^ swz_w(e);
           wt_rd[s][h][nb] = A_V * 16 + e * (LPRW * 16) + chunk * 16 + (col % PV) * E::kBytes;
         }
@@ -359,13 +363,12 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   // behind it.  These loads
   // are older than every operand load of the loop, so the counted waits there only get stricter.
   constexpr int CPLW = 4 * NBW;            // consecutive output channels of a lane (not WT)
-  constexpr int SRC_W = E::kBytes == 2 ? (WT ? 2 : 4) : CPLW / 4;   // dwords per piece
-  constexpr int SRC_N = E::kBytes == 2 ? (WT ? NBW : CPLW / 8) : 1; // pieces per row
-  static_assert(E::kBytes == 1 || WT || CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
+  constexpr int SRC_W = E::kBytes == 2 ? 4 : CPLW / 4;          // dwords per piece
+  constexpr int SRC_N = E::kBytes == 2 ? CPLW / 8 : 1;          // pieces per row
+  static_assert(E::kBytes == 1 || CPLW % 8 == 0, "two-byte outputs need NBW >= 2");
   const int ch0 = n0 + wn * (NBW * 16) + q * CPLW;
   auto piece_channel = [&](int i) -> int {
-    if constexpr (E::kBytes == 2 && WT) return n0 + (wn * NBW + i) * 16 + 4 * q;
-    else if constexpr (E::kBytes == 2) return ch0 + i * 8;
+    if constexpr (E::kBytes == 2) return ch0 + i * 8;
     else return ch0;
   };
   typedef int src_vec __attribute__((ext_vector_type(SRC_W)));
@@ -503,34 +506,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     constexpr int ACT = decltype(act_c)::value;
     constexpr int MODE = decltype(mode_c)::value;
     constexpr bool SRC = (MODE & 1) != 0;
-    if constexpr (E::kBytes == 2 && WT) {
-      // channels nb*16 + 4q .. +3 of each block: 8-byte pieces
-      typedef int v2i __attribute__((ext_vector_type(2)));
-#pragma unroll
-      for (int rb = 0; rb < RBW; ++rb) {
-        const int o = out_row[rb];
-        const bool row_ok = o >= 0 && o < p.rows_c;
-#pragma unroll
-        for (int nb = 0; nb < NBW; ++nb) {
-          const int ch = n0 + (wn * NBW + nb) * 16 + 4 * q;
-          const bool ok = row_ok && ch < p.k_out;
-          const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 2u : kOob;
-          v2i src = {0, 0};
-          if constexpr (SRC) src = __builtin_bit_cast(v2i, src_pre[rb][nb]);
-          const uint16_t *sh = reinterpret_cast<const uint16_t *>(&src);
-          v2i outv;
-          uint16_t *oh = reinterpret_cast<uint16_t *>(&outv);
-#pragma unroll
-          for (int x = 0; x < 4; ++x) {
-            const float a = acc[rb][nb][x];
-            float t = SRC ? __builtin_fmaf(p.alpha, a, p.beta * E::to_float(sh[x])) : p.alpha * a;
-            t = apply_act(t, ACT, p.act_alpha);
-            oh[x] = E::from_float(t);
-          }
-          __builtin_amdgcn_raw_buffer_store_b64(outv, rs_c, coff, 0, 0);
-        }
-      }
-    } else if constexpr (E::kBytes == 2) {
+    if constexpr (E::kBytes == 2) {
       constexpr int NG = CPLW / 8;   // 16-byte groups
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb) {
