@@ -207,7 +207,10 @@ def bench_stack(args):
     def leg(name, p, flops):
         r = tn.tune_conv(p)
         wms, ems = timed(lambda: ConvMainUnitTest.implicit_gemm2(p), steps, warm)
-        res[name] = {"tile": list(r.desp.tile_shape[:2]), "ms_per_step": round(wms, 5),
+        res[name] = {"tile": list(r.desp.tile_shape[:2]),
+                     "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
+                                    for nm, ms in r.tried},
+                     "ms_per_step": round(wms, 5),
                      "tflops": round(flops / (wms * 1e-3) / 1e12, 2)}
 
     pf = ConvParams(3, ConvOpType.Forward)
