@@ -82,6 +82,15 @@ __device__ __forceinline__ auto load_hidden_words(v4i rsrc, uint32_t voff) {
   if constexpr (W == 2) return load_b64_hidden(rsrc, voff);
   else return load_b128_hidden(rsrc, voff);
 }
+// The same into a variable that already has a value (a conditional load: the variable keeps its
+// value on the other path).  The register is read-write to the compiler, so both paths end in
+// the same register and no copy - which would copy too early - is needed where they meet.
+__device__ __forceinline__ void load_hidden_into(v2i_hidden &r, v4i rsrc, uint32_t voff) {
+  asm volatile("buffer_load_dwordx2 %0, %1, %2, 0 offen" : "+v"(r) : "v"(voff), "s"(rsrc) : "memory");
+}
+__device__ __forceinline__ void load_hidden_into(v4i &r, v4i rsrc, uint32_t voff) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "+v"(r) : "v"(voff), "s"(rsrc) : "memory");
+}
 
 // Workgroup barrier without the fence of __syncthreads(): the fence would wait for every
 // outstanding direct-to-LDS load, i.e. also for the stages that are being prefetched.  The empty

@@ -383,8 +383,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       for (int i = 0; i < SRC_N; ++i) {
         const int ch = piece_channel(i);
         const bool ok = row_ok && ch < p.k_out;
-        src_pre[rb][i] = load_hidden_words<SRC_W>(
-            rsw_d, ok ? (uint32_t)((int64_t)o * p.ldd + ch) * (uint32_t)E::kBytes : kOob);
+        load_hidden_into(src_pre[rb][i], rsw_d, ok ? (uint32_t)((int64_t)o * p.ldd + ch) * (uint32_t)E::kBytes : kOob);
       }
     }
   }
