@@ -358,7 +358,20 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   }
 
   // (the address arithmetic above runs while the counts are on their way)
-  const int my_wgs = fast_div(my_live + p.tiles_per_wg - 1, p.tiles_per_wg);
+  // Tiles per unit: as few as still leave every workgroup of the grid at most one unit - shorter
+  // units end sooner, and the longest unit is the launch's critical path -, at most what the LDS
+  // lists hold.  (Every offset may add a partly filled unit: kv * per_r workgroups are set aside.)
+  int tiles_per_unit = p.tiles_per_wg;
+  {
+    const int total_live = __builtin_amdgcn_readlane(wave_prefix_sum_dpp(my_live), 31);
+    const int room = (int)gridDim.x - p.kv * per_r;
+    if (room > 0) {
+      int fewest = fast_div(total_live * per_r + room - 1, room);
+      fewest = fewest < 2 ? 2 : fewest;
+      tiles_per_unit = fewest < tiles_per_unit ? fewest : tiles_per_unit;
+    }
+  }
+  const int my_wgs = fast_div(my_live + tiles_per_unit - 1, tiles_per_unit);
   const int my_units = my_wgs * per_r;
   const int incl = wave_prefix_sum_dpp(my_units);
   const int total_units = __builtin_amdgcn_readlane(incl, 31);
