@@ -303,7 +303,15 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   }
   uint32_t w_voff[IPW];
   int w_cpos[IPW];         // contraction element (WT: contraction row) the lane fetches, first chunk
-  auto swz_w = [](int e) { return 2 * (((e * LPRW) >> 4) & (LPRW / 2 - 1)); };   // WT: even chunk XOR
+  // WT: chunk XOR of contraction row e.  A transposing read has, per 16 lanes, four rows e .. e+3
+  // and four chunks 4*NBW/8 apart (see wt_rd below), 8 bytes of each.  Rows of 128 bytes (TN = 64)
+  // alternate between the halves of the 256 bytes the banks span, so rows e and e+2 must use
+  // different chunks: bit 2 follows bit 1 of e.  Rows of 256 bytes (TN = 128) all start at bank 0
+  // and the four chunks are two apart: bits 0 and 3 follow bits 0 and 1 of e.
+  auto swz_w = [](int e) {
+    return LPRW == 8 ? 4 * ((e >> 1) & 1) | 2 * ((e >> 2) & 1) : (e & 1) | 8 * ((e >> 1) & 1) | 2 * ((e >> 2) & 1);
+  };
+  static_assert(!WT || LPRW == 8 || LPRW == 16, "weight tiles of 64 or 128 channels");
 #pragma unroll
   for (int t = 0; t < IPW; ++t) {
     if constexpr (!WT) {
