@@ -196,14 +196,6 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     }
   }
 
-  // Without a mask and with entries addressed by position (gather -> GEMM -> scatter), the first
-  // entries depend on nothing that is loaded here: requested now, they land with the loads above.
-  const bool early_idx = !has_mask && p.gather_by_pos && p.gather != nullptr;
-  if (early_idx) {
-    const bool live = lane < RPW && key_pos < p.n_pos && key_pos < p.n_idx;
-    dma_b32(rsrc_words(p.gather, p.gather_bytes), lds_addr(ix0[wave]), live ? (uint32_t)key_pos * 4u : kOob, 0u);
-  }
-
   wait_vmcnt<0>();
 #pragma unroll
   for (int i = 0; i < MKW; ++i) keep_after_wait(raw_mk[i]);
@@ -279,7 +271,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   // rows, fragment slots) overlaps their round trip.
   if (n_steps > 0) {
     auto first = [&](auto jc) -> bool {
-      if (!(early_idx && decltype(jc)::value == 0)) issue_idx(decltype(jc)::value, idx_slot(jc));
+      issue_idx(decltype(jc)::value, idx_slot(jc));
       return false;
     };
     run_steps(first, std::make_integer_sequence<int, DI>{});
