@@ -194,6 +194,13 @@ def bench_stack(args):
     ConvMainUnitTest_sync()
     prep_ms = (time.perf_counter() - t0) * 1e3          # first call, allocations included
     n_out2 = int(table2.indices_fwd.dim(1))
+    prep = {}
+    for name, fn in (("subm_pairs", lambda: pairs.subm_pairs_device(d_coords, grid)),
+                     ("sort_by_mask", lambda: pairs.sort_by_mask_device(table.mask_fwd)),
+                     ("sparse_conv_pairs_stride2", lambda: pairs.sparse_conv_pairs_device(d_coords, grid, batch_size=1)),
+                     ("sort_by_mask_stride2", lambda: pairs.sort_by_mask_device(table2.mask_fwd))):
+        wms, _ = timed(fn, 5, 2)     # (wall clock: allocation of the result tensors included)
+        prep[name] = round(wms, 4)
     pairs1 = int((table.indices_fwd.cpu().numpy() >= 0).sum())
     pairs2 = int((table2.indices_fwd.cpu().numpy() >= 0).sum())
     x, w, b = bf16((n, c), 1 / 64), bf16((c, 27, c), 1 / 2048), bf16((c,), 1 / 512)
@@ -202,7 +209,7 @@ def bench_stack(args):
     tn = tuner.Tuner(steps=3, warmup=1)
     steps, warm = max(5, args.steps // 10), max(2, args.warmup // 10)
     res = {"voxels": n, "pairs": pairs1, "voxels_out_stride2": n_out2, "pairs_stride2": pairs2,
-           "input_preparation_first_call_ms": round(prep_ms, 3)}
+           "input_preparation_first_call_ms": round(prep_ms, 3), "input_preparation_ms": prep}
 
     def leg(name, p, flops):
         r = tn.tune_conv(p)
