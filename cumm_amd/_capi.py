@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcummhip.so")
 
 OK, EINVAL, ERUNTIME, ENOALGO = 0, 1, 2, 3
+STATIC_WORKSPACE_BYTES = 8 << 20   # CUMM_HIP_STATIC_WORKSPACE_BYTES
 
 
 class GemmDesc(C.Structure):
@@ -62,6 +63,7 @@ _VP, _PVP = C.c_void_p, C.POINTER(C.c_void_p)
 SYMBOLS = {
     "cumm_hip_gemm": (C.c_int, [C.POINTER(GemmDesc), C.POINTER(GemmArgs), _VP]),
     "cumm_hip_sparse_conv": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(SparseConvArgs), _VP]),
+    "cumm_hip_sparse_conv_static_ws": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(SparseConvArgs), _VP]),
     "cumm_hip_list_gemm_algos": (C.c_int, [C.POINTER(GemmDesc), C.c_int]),
     "cumm_hip_list_conv_algos": (C.c_int, [C.POINTER(ConvDesc), C.c_int]),
     "cumm_hip_gemm_supported": (C.c_int, [C.POINTER(GemmDesc)]),

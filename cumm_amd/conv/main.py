@@ -58,11 +58,24 @@ class ConvMainUnitTest:
                                        mask_sparse))
 
     @staticmethod
+    def implicit_gemm2_static_workspace(params: ConvParams) -> None:
+        """``implicit_gemm2`` for callers that must not allocate device memory: the workspace a
+        backward-weight call needs is an array of ``_capi.STATIC_WORKSPACE_BYTES`` bytes inside
+        the library (``cumm_hip_sparse_conv_static_ws``); ``params.workspace`` is ignored and
+        never assigned.  A problem that needs more raises ValueError.  Calls that overlap in
+        time on one GPU share that array and race."""
+        ConvMainUnitTest._implicit_gemm2(params, True)
+
+    @staticmethod
     def implicit_gemm2(params: ConvParams) -> None:
+        ConvMainUnitTest._implicit_gemm2(params, False)
+
+    @staticmethod
+    def _implicit_gemm2(params: ConvParams, static_ws: bool) -> None:
         desp = params.conv_algo_desp
         # A call whose parameter object has not changed since it was last validated goes
         # straight to the C ABI with the argument block prepared then.
-        prep = params.__dict__.get("_prepared")
+        prep = params.__dict__.get("_prepared_static" if static_ws else "_prepared")
         if prep is not None and prep[0] == (params._version, desp._version, desp.tile_shape[0],
                                             desp.tile_shape[1], desp.tile_shape[2]):
             status = prep[1](prep[2], prep[3], params.stream)
@@ -153,14 +166,17 @@ class ConvMainUnitTest:
 
         workspace_size = desp.query_conv_workspace_size(mnk[0], mnk[1], mnk[2], split_k_slices,
                                                         kernel_volume)
-        if workspace_size > 0:
-            if not params.workspace.empty():
-                if params.workspace.nbytes < workspace_size:
-                    raise RuntimeError("workspace at least %d bytes." % workspace_size)
-            else:
-                # as in the reference the allocation stays in the caller's params object
-                params.workspace = empty([workspace_size], uint8, 0)
-        workspace = params.workspace
+        if static_ws:
+            workspace = Tensor()
+        else:
+            if workspace_size > 0:
+                if not params.workspace.empty():
+                    if params.workspace.nbytes < workspace_size:
+                        raise RuntimeError("workspace at least %d bytes." % workspace_size)
+                else:
+                    # as in the reference the allocation stays in the caller's params object
+                    params.workspace = empty([workspace_size], uint8, 0)
+            workspace = params.workspace
 
         args = _capi.SparseConvArgs()
         args.ptr_A, args.ptr_B, args.ptr_C = _ptr(a_ten), _ptr(b_ten), _ptr(c_ten)
@@ -192,7 +208,7 @@ class ConvMainUnitTest:
         name = repr(desp) if params.timer.enable else ""
         if name:
             params.timer.record(name, params.stream)
-        fn = _capi.lib().cumm_hip_sparse_conv
+        fn = _capi.lib().cumm_hip_sparse_conv_static_ws if static_ws else _capi.lib().cumm_hip_sparse_conv
         status = fn(ctypes.byref(cdesc), ctypes.byref(args), params.stream)
         if name:
             params.timer.record(name, params.stream)
@@ -200,6 +216,6 @@ class ConvMainUnitTest:
         if not name:
             # remember the validated argument block (the tensors it points into stay referenced
             # by params; any later assignment to params or the descriptor invalidates it)
-            params.__dict__["_prepared"] = (
+            params.__dict__["_prepared_static" if static_ws else "_prepared"] = (
                 (params._version, desp._version, desp.tile_shape[0], desp.tile_shape[1],
                  desp.tile_shape[2]), fn, ctypes.byref(cdesc), ctypes.byref(args), cdesc, args)

@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -147,6 +148,56 @@ void fill_gemm_desc(CummHipGemmDesc &d, int dt, int ta, int tb, int tc, int tm, 
   d.split_k_serial = splitk;
   d.split_k_parallel = 0;
 }
+
+// Zeroes `words` 4-byte words.  Used instead of hipMemsetAsync for semaphores and partial-sum
+// images so that a caller may record these entry points into a HIP graph.
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *dst, size_t words, int wide) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t done = 0;
+  if (wide) {   // 16-byte aligned: whole quads first
+    const size_t quads = words / 4;
+    for (size_t q = i; q < quads; q += stride) reinterpret_cast<v4i *>(dst)[q] = v4i{0, 0, 0, 0};
+    done = quads * 4;
+  }
+  for (size_t w = done + i; w < words; w += stride) dst[w] = 0u;
+}
+
+hipError_t zero_device(void *ptr, size_t bytes, hipStream_t s) {
+  const size_t words = (bytes + 3) / 4;   // (every size zeroed here is a multiple of 4)
+  if (words == 0) return hipSuccess;
+  const int wide = aligned16(ptr) ? 1 : 0;
+  size_t blocks = ((wide ? words / 4 + 3 : words) + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)blocks), dim3(256), 0, s, reinterpret_cast<uint32_t *>(ptr), words, wide);
+  return hipGetLastError();
+}
+
+// ---- the library's own scratch memory for cumm_hip_sparse_conv_static_ws: one array per GPU,
+// held until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels and fills take the address that call returns for the current device.
+static __device__ __align__(256) unsigned char scratch[CUMM_HIP_STATIC_WORKSPACE_BYTES];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void **out) {
+  int dev = -1;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(CUMM_HIP_ERUNTIME, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) return fail(CUMM_HIP_ERUNTIME, "hipGetSymbolAddress returned no address for the scratch array");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return CUMM_HIP_OK;
+}
+
+int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a, void *stream_, void *workspace,
+                     size_t workspace_bytes, size_t workspace_cap);
 
 }  // namespace
 
@@ -348,7 +399,8 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
     const size_t need = sizeof(int32_t) * grid.x * grid.y;
     if (!a->workspace || a->workspace_bytes < need)
       return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
-    HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
+    if (reinterpret_cast<uintptr_t>(a->workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
+    HIP_TRY(zero_device(a->workspace, need, stream));
     p.sem = reinterpret_cast<int32_t *>(a->workspace);
   }
   hipError_t e = launch_tilegemm(dt, tm, tn, xk, yk, p, grid, stream);
@@ -359,6 +411,23 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
 // ---------------------------------------------------------------------------------------------
 int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a, void *stream_) {
   if (!desc || !a) return fail(CUMM_HIP_EINVAL, "null descriptor or arguments");
+  return sparse_conv_impl(desc, a, stream_, a->workspace, a->workspace_bytes, 0);
+}
+
+int cumm_hip_sparse_conv_static_ws(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a, void *stream_) {
+  if (!desc || !a) return fail(CUMM_HIP_EINVAL, "null descriptor or arguments");
+  void *ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  return sparse_conv_impl(desc, a, stream_, ws, CUMM_HIP_STATIC_WORKSPACE_BYTES, CUMM_HIP_STATIC_WORKSPACE_BYTES);
+}
+
+}  // extern "C"
+
+namespace {
+// workspace_cap != 0: the workspace is the library's own array of that size, and a problem that
+// needs more is an argument error (the caller cannot make it larger)
+int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a, void *stream_, void *workspace,
+                     size_t workspace_bytes, size_t workspace_cap) {
   const CummHipConvDesc &c = *desc;
   const CummHipGemmDesc &d = c.gemm;
   const int fam = conv_family(c);
@@ -434,12 +503,14 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
   if (a->mask_width <= 0 || a->mask_width % tk) return fail(CUMM_HIP_ERUNTIME, "mask_width must be a positive multiple of tile k");
   if (fam == 3 && a->split_k_slices > 1 && a->mask_width <= kWgradMaxPos) {
     const size_t need = sizeof(float) * (size_t)a->K * kv * a->C;
-    if (!a->workspace || a->workspace_bytes < need)
+    if (workspace_cap && need > workspace_cap)
+      return fail(CUMM_HIP_EINVAL, "this problem needs %zu bytes of workspace, the static one holds %zu", need, workspace_cap);
+    if (!workspace || workspace_bytes < need)
       return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
-    if (reinterpret_cast<uintptr_t>(a->workspace) & 15u) return fail(CUMM_HIP_EINVAL, "workspace must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u) return fail(CUMM_HIP_EINVAL, "workspace must be 16-byte aligned");
     WgradParams w;
     std::memset(&w, 0, sizeof(w));
-    w.dout = a->ptr_A; w.inp = a->ptr_B; w.scratch = reinterpret_cast<float *>(a->workspace);
+    w.dout = a->ptr_A; w.inp = a->ptr_B; w.scratch = reinterpret_cast<float *>(workspace);
     w.argsort = a->mask_argsort_ptr; w.indices = a->indice_ptr; w.red_mask = a->mask_ptr;
     w.num_red = (a->N + a->mask_width - 1) / a->mask_width; w.mask_width = a->mask_width;
     w.mask_filter = a->mask_filter;
@@ -461,7 +532,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
     const size_t lists_bytes = 128 + sizeof(int32_t) * (size_t)kv * w.num_red;
     int images = 0;
     for (int s = 8; s >= 1 && !images; s >>= 1)
-      if (s <= a->split_k_slices && a->workspace_bytes >= s * image_bytes + lists_bytes &&
+      if (s <= a->split_k_slices && workspace_bytes >= s * image_bytes + lists_bytes &&
           (uint64_t)s * image_bytes < ((uint64_t)1 << 32))   // (the finalize kernel reads them through one descriptor)
         images = s;
     const bool fits32 = (int64_t)a->rows_out * a->K * 2 < (int64_t)1 << 31 && (int64_t)a->rows_in * a->C * 2 < (int64_t)1 << 31 &&
@@ -473,7 +544,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
     // (the unit-walking kernel divides unit numbers with a float reciprocal: exact below 2^22)
     const int64_t unit_bound = ((int64_t)(w.num_red + qt - 1) / qt + 1) * kv * (((int64_t)a->K + 63) / 64) * (((int64_t)a->C + 63) / 64);
     if (images && fits32 && unit_bound < ((int64_t)1 << 22) && w.num_red < (1 << 22)) {
-      char *base = reinterpret_cast<char *>(a->workspace);
+      char *base = reinterpret_cast<char *>(workspace);
       const size_t lists_at = images * image_bytes;
       pre.scratch = w.scratch; pre.scratch_floats = (int64_t)(lists_at / sizeof(float));
       pre.red_mask = w.red_mask; pre.num_red = w.num_red; pre.kv = kv; pre.mask_filter = w.mask_filter;
@@ -483,7 +554,7 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
       w.images = f.images = images;
       w.image_floats = f.image_floats = (int64_t)(image_bytes / sizeof(float));
     } else {
-      HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
+      HIP_TRY(zero_device(workspace, need, stream));
     }
     hipError_t e = dt == CUMM_HIP_F16 ? launch_wgrad_atomic_f16(w, pre, f, stream) : launch_wgrad_atomic_bf16(w, pre, f, stream);
     if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
@@ -512,15 +583,21 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
   dim3 grid((a->K + tm - 1) / tm, n_tiles * kv, p.split_k);
   if (p.split_k > 1) {
     const size_t need = sizeof(int32_t) * grid.x * grid.y;
-    if (!a->workspace || a->workspace_bytes < need)
+    if (workspace_cap && need > workspace_cap)
+      return fail(CUMM_HIP_EINVAL, "this problem needs %zu bytes of workspace, the static one holds %zu", need, workspace_cap);
+    if (!workspace || workspace_bytes < need)
       return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
-    HIP_TRY(hipMemsetAsync(a->workspace, 0, need, stream));
-    p.sem = reinterpret_cast<int32_t *>(a->workspace);
+    if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
+    HIP_TRY(zero_device(workspace, need, stream));
+    p.sem = reinterpret_cast<int32_t *>(workspace);
   }
   hipError_t e = launch_tilegemm(dt, tm, tn, false, false, p, grid, stream);
   if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
   return CUMM_HIP_OK;
 }
+}  // namespace
+
+extern "C" {
 
 // ---------------------------------------------------------------------------------------------
 int cumm_hip_device_count(int *count) {

@@ -127,6 +127,20 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *args, void
 int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArgs *args,
                          void *stream);
 
+/* cumm_hip_sparse_conv for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc) and so cannot provide the
+ * workspace that backward-weight needs (split-K semaphores; fp32 partial-sum images and live-tile
+ * lists of the split_k_parallel descriptors).  No counterpart in the reference, whose
+ * implicit_gemm2 allocates a missing workspace itself (cumm/conv/nvrtc_code.py:183-192).
+ * args->workspace / workspace_bytes are ignored: the workspace is an array of
+ * CUMM_HIP_STATIC_WORKSPACE_BYTES bytes inside the library, one per GPU, kept until the process
+ * ends.  A problem that needs more returns CUMM_HIP_EINVAL.  The call allocates nothing and
+ * clears what it needs with kernels (no memset nodes).  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams) race. */
+#define CUMM_HIP_STATIC_WORKSPACE_BYTES (8u << 20)
+int cumm_hip_sparse_conv_static_ws(const CummHipConvDesc *desc, const CummHipSparseConvArgs *args,
+                                   void *stream);
+
 /* GemmMainUnitTest.get_all_algo_desp / ConvMainUnitTest.get_all_conv_algo_desp
  * (cumm/gemm/main.py:914-965, cumm/conv/main.py:467-481): the descriptors this
  * build has kernels for.  Writes at most cap entries, returns the total. */
