@@ -10,9 +10,9 @@ import ctypes
 from typing import List, Tuple
 
 from .. import _capi
-from ..gemm.main import (INT_MAX, _check_device, _check_shape, _enum_int, _ptr, desp_from_c,
-                         desp_to_c)
-from ..tensorview import Tensor, empty, uint8
+from ..gemm.main import (INT_MAX, _check_device, _check_dtype, _check_shape, _enum_int, _ptr,
+                         desp_from_c, desp_to_c)
+from ..tensorview import Tensor, empty, float32, int32, uint8, uint32
 from ..tensorview.gemm import (ConvAlgoDesp, ConvOpType, ConvParams, gemm_abc_012_to_iwo,
                                implicit_gemm_mnk)
 
@@ -105,6 +105,21 @@ class ConvMainUnitTest:
             raise RuntimeError("error")
         _check_device(inp, weight, output, bias, scale, output_add, indices, mask, mask_argsort,
                       mask_output)
+        # The reference takes every operand through data_ptr<T>(), which throws on another
+        # element type (include/tensorview/tensor.h:1497, 2027): the kernels derive all extents
+        # from the descriptor's element sizes.
+        _check_dtype(inp, desp.dtype_input, "input")
+        _check_dtype(weight, desp.dtype_weight, "weight")
+        _check_dtype(output, desp.dtype_output, "output")
+        _check_dtype(indices, int32, "indices")
+        _check_dtype(mask_argsort, int32, "mask_argsort")
+        _check_dtype(mask, uint32, "mask")
+        _check_dtype(mask_output, uint32, "mask_output")
+        if desp.is_int8_inference:
+            _check_dtype(bias, float32, "bias")
+            _check_dtype(scale, float32, "scale")
+        else:
+            _check_dtype(bias, desp.dtype_output, "bias")
         inv = gemm_abc_012_to_iwo(op_type)
         iwo = [inp, weight, output]
         a_ten, b_ten, c_ten = iwo[inv[0]], iwo[inv[1]], iwo[inv[2]]

@@ -720,6 +720,10 @@ int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_sha
   if (!aligned16(coords) || !aligned16(workspace)) return fail(CUMM_HIP_EINVAL, "coords and workspace must be 16-byte aligned");
   const int64_t kv = (int64_t)ksize[0] * ksize[1] * ksize[2];
   if (ksize[0] < 1 || ksize[1] < 1 || ksize[2] < 1 || kv > 32) return fail(CUMM_HIP_EINVAL, "kernel volume must be 1..32");
+  // indices_bwd[k] = indices_fwd[kv-1-k] and the bit-reversed masks hold only when offset kv-1-k is
+  // the negative of offset k, i.e. for odd kernel sizes
+  if (!(ksize[0] & 1) || !(ksize[1] & 1) || !(ksize[2] & 1))
+    return fail(CUMM_HIP_EINVAL, "submanifold convolution needs odd kernel sizes");
   for (int d = 0; d < 3; ++d)
     if (spatial_shape[d] < 1 || dilation[d] < 1) return fail(CUMM_HIP_EINVAL, "spatial_shape and dilation must be positive");
   if (!workspace || workspace_bytes < cumm_hip_subm_pairs_workspace(n))

@@ -10,7 +10,7 @@ import ctypes
 from typing import Dict, List, Tuple
 
 from .. import _capi
-from ..tensorview import Tensor, empty, uint8
+from ..tensorview import Tensor, empty, int32, uint8
 from ..tensorview.gemm import (Activation, GemmAlgoDesp, GemmParams, ShuffleStrideType)
 
 INT_MAX = 2 ** 31 - 1
@@ -67,6 +67,12 @@ def _check_shape(t: Tensor, shape, what="shape"):
 
 def _ptr(t: Tensor):
     return None if t.empty() else t.byte_pointer()
+
+
+def _check_dtype(t: Tensor, dtype: int, what: str):
+    """template_dtype_check of the reference's data_ptr<T>() (include/tensorview/tensor.h:1497)."""
+    if not t.empty() and t.dtype != int(dtype):
+        raise RuntimeError("%s has dtype %d, expected %d" % (what, t.dtype, int(dtype)))
 
 
 def _check_device(*tens):
@@ -182,6 +188,12 @@ class GemmMainUnitTest:
         _check_shape(b, [-1, -1])
         _check_shape(c, [-1, -1])
         _check_device(a, b, c, d, params.a_inds, params.b_inds, params.c_inds)
+        _check_dtype(a, desp.dtype_a, "a")
+        _check_dtype(b, desp.dtype_b, "b")
+        _check_dtype(c, desp.dtype_c, "c")
+        _check_dtype(d, desp.dtype_c, "d")
+        for name in ("a_inds", "b_inds", "c_inds"):
+            _check_dtype(getattr(params, name), int32, name)
         a_ten, b_ten = a, b
         trans_a, trans_b, trans_c = desp.trans_a, desp.trans_b, desp.trans_c
         if trans_c:

@@ -57,9 +57,17 @@ def calc_output_dims(in_shape, ksize, padding, stride, dilation):
                  for i, k, p, s, d in zip(in_shape, ksize, padding, stride, dilation))
 
 
+def _check_odd_ksize(ksize):
+    if any(int(k) < 1 or int(k) % 2 == 0 for k in ksize):
+        raise ValueError("submanifold convolution needs odd kernel sizes, got %s" % (list(ksize),))
+
+
 def subm_pairs(coords: np.ndarray, spatial_shape: Sequence[int], ksize=(3, 3, 3),
                dilation=(1, 1, 1)) -> PairTable:
-    """Submanifold convolution: outputs sit on the input sites."""
+    """Submanifold convolution: outputs sit on the input sites.  Kernel sizes must be odd: only
+    then is offset kv-1-k the negative of offset k, which the backward table (the forward one
+    reversed) and the bit-reversed backward masks rely on."""
+    _check_odd_ksize(ksize)
     coords = np.ascontiguousarray(coords, dtype=np.int32)
     n = coords.shape[0]
     offs = _offsets(ksize)
@@ -155,6 +163,7 @@ def subm_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), dil
     from . import tensorview as tv
     if coords.device < 0 or coords.dtype != tv.int32 or coords.ndim != 2 or coords.shape[1] != 4:
         raise ValueError("coords must be a device int32 tensor of shape [N, 4]")
+    _check_odd_ksize(ksize)
     n = int(coords.shape[0])
     kv = int(ksize[0]) * int(ksize[1]) * int(ksize[2])
     lib = _capi.lib()

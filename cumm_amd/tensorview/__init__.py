@@ -439,15 +439,26 @@ class Tensor:
             _capi.check(_capi.lib().cumm_hip_memset(ptr, 0, n, stream))
         return self
 
-    def fill_int_(self, val: int, ctx: Optional[Context] = None) -> "Tensor":
-        host = np.full(self._shape, val, dtype=_HOST_VIEW_DTYPE[self._dtype])
-        self.copy_(from_numpy(host), ctx)
+    def _fill_host_pattern(self, host: np.ndarray, ctx: Optional[Context]) -> "Tensor":
+        src = from_numpy(host)
+        if src.dtype != self._dtype:      # bf16 travels as uint16 bit patterns
+            src = src.type_view(self._dtype)
+        self.copy_(src, ctx)
         return self
 
+    def fill_int_(self, val: int, ctx: Optional[Context] = None) -> "Tensor":
+        if self._dtype == bfloat16:
+            return self.fill_float_(float(val), ctx)
+        return self._fill_host_pattern(np.full(self._shape, val, dtype=_HOST_VIEW_DTYPE[self._dtype]), ctx)
+
     def fill_float_(self, val: float, ctx: Optional[Context] = None) -> "Tensor":
-        host = np.full(self._shape, val, dtype=_HOST_VIEW_DTYPE[self._dtype])
-        self.copy_(from_numpy(host), ctx)
-        return self
+        if self._dtype == bfloat16:
+            # round to nearest even on bit 16 of the float32 pattern, NaN -> 0x7FFF
+            # (bfloat16_t(float), include/tensorview/gemm/dtypes/bfloat16.h:86-111 of the reference)
+            u = int(np.float32(val).view(np.uint32))
+            bits = 0x7FFF if val != val else ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF
+            return self._fill_host_pattern(np.full(self._shape, bits, dtype=np.uint16), ctx)
+        return self._fill_host_pattern(np.full(self._shape, val, dtype=_HOST_VIEW_DTYPE[self._dtype]), ctx)
 
     def __repr__(self):
         return "Tensor[%s|%s|%s]" % (self._shape, self._dtype, self.device)
@@ -467,7 +478,7 @@ def empty(shape, dtype=np.float32, device: int = -1, pinned: bool = False,
 def full(shape, val, dtype=np.float32, device: int = -1, pinned: bool = False,
          managed: bool = False) -> Tensor:
     t = Tensor(shape, _to_tv_dtype(dtype), device)
-    return t.fill_float_(val) if t.dtype in (float32, float16, float64) else t.fill_int_(val)
+    return t.fill_float_(val) if t.dtype in (float32, float16, float64, bfloat16, tf32) else t.fill_int_(val)
 
 
 def from_numpy(arr: np.ndarray) -> Tensor:

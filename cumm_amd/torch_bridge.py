@@ -166,7 +166,8 @@ class _SparseConvFunction(torch.autograd.Function):
         stream = current_stream()
         grad_in = grad_w = grad_b = None
         if ctx.needs_input_grad[0]:
-            grad_in = torch.empty_like(features)
+            # inputs that feed no output site sit in tiles the kernel skips (mask 0): zero them
+            grad_in = torch.empty_like(features) if g.subm else torch.zeros_like(features)
             p = ConvParams(3, ConvOpType.BackwardInput)
             p.conv_algo_desp = _desp_like(dtype, ConvOpType.BackwardInput)
             p.input, p.weight, p.output = torch2tensor(grad_in), torch2tensor(weight), torch2tensor(grad_out)

@@ -12,13 +12,14 @@ the timing done by events on the caller's stream.
 A candidate shares the kind of the descriptor already set in the parameter
 object (operation, element types, layouts, shuffle type, int8 epilogue) and
 differs in tile shape and split-k variant.  Results are cached per problem
-shape; the voxel count enters the key by its power-of-two bucket.
+shape; the voxel count enters the key by its power-of-two bucket, the pair density P/N
+(when the caller passes the pair count) by its half-octave bucket.
 """
 from typing import Callable, Dict, List, NamedTuple, Optional, Tuple
 
 from .conv.main import ConvMainUnitTest
 from .gemm.main import GemmMainUnitTest
-from .tensorview import CUDAEvent
+from .tensorview import Context, CUDAEvent, Tensor
 from .tensorview.gemm import (ConvAlgoDesp, ConvOpType, ConvParams, GemmAlgoDesp, GemmParams,
                               implicit_gemm_mnk)
 
@@ -31,6 +32,14 @@ class TuneResult(NamedTuple):
 
 def _bucket(n: int) -> int:
     return max(int(n) - 1, 0).bit_length()
+
+
+def _density_bucket(num_pairs: Optional[int], n: int) -> int:
+    """Half-octave bucket of P/N (pairs per position, 1 .. kernel volume); -1 when unknown."""
+    if num_pairs is None or n <= 0:
+        return -1
+    import math
+    return int(math.floor(2.0 * math.log2(max(float(num_pairs) / float(n), 1.0))))
 
 
 def conv_candidates(params: ConvParams, desps: Optional[List[ConvAlgoDesp]] = None) -> List[ConvAlgoDesp]:
@@ -77,6 +86,20 @@ def gemm_candidates(params: GemmParams, desps: Optional[List[GemmAlgoDesp]] = No
     return res
 
 
+def _stream_ctx(stream: int) -> Context:
+    ctx = Context()
+    ctx.set_cuda_stream(stream)
+    return ctx
+
+
+def _save(target: Tensor, ctx: Context) -> Tensor:
+    """Copy of ``target`` made on the stream the timed launches run on, so that neither the copy
+    nor the restore can overtake or trail a launch on a non-blocking stream."""
+    saved = Tensor(target.shape, target.dtype, target.device)
+    saved.copy_(target, ctx)
+    return saved
+
+
 def _time_calls(run: Callable[[], None], stream: int, steps: int, warmup: int) -> float:
     for _ in range(warmup):
         run()
@@ -97,16 +120,23 @@ class Tuner:
 
     # ---- sparse convolution
     @staticmethod
-    def conv_key(params: ConvParams) -> tuple:
+    def conv_key(params: ConvParams, num_pairs: Optional[int] = None) -> tuple:
+        """(operation, types, C, K, kernel volume, bucket of N, bucket of the pair density P/N, ...).
+        ``num_pairs`` is the number of active pairs P of the geometry when the caller knows it
+        (two clouds of one size and very different density want different tiles); without it
+        the density does not enter the key."""
         d = params.conv_algo_desp
+        n = params.indices.dim(1)
         return ("conv", ConvOpType(d.op_type).value, d.dtype_a, d.dtype_b, d.dtype_c, bool(d.is_int8_inference),
-                params.input.dim(1), params.weight.dim(0), params.weight.dim(1), _bucket(params.indices.dim(1)),
-                params.split_k_slices > 1, params.mask_width, bool(params.reverse_mask))
+                params.input.dim(1), params.weight.dim(0), params.weight.dim(1), _bucket(n),
+                _density_bucket(num_pairs, n), params.split_k_slices > 1, params.mask_width,
+                bool(params.reverse_mask))
 
-    def tune_conv(self, params: ConvParams, desps: Optional[List[ConvAlgoDesp]] = None) -> TuneResult:
+    def tune_conv(self, params: ConvParams, desps: Optional[List[ConvAlgoDesp]] = None,
+                  num_pairs: Optional[int] = None) -> TuneResult:
         """Times every candidate on ``params`` (its result tensor is saved and restored, the
         descriptor is left at the fastest) and remembers the winner."""
-        key = self.conv_key(params)
+        key = self.conv_key(params, num_pairs)
         hit = self.cache.get(key)
         if hit is not None:
             params.conv_algo_desp = hit.desp
@@ -117,7 +147,8 @@ class Tuner:
         op = ConvOpType(params.conv_algo_desp.op_type)
         target = {ConvOpType.Forward: params.output, ConvOpType.BackwardInput: params.input,
                   ConvOpType.BackwardWeight: params.weight}[op]
-        saved = target.clone()
+        ctx = _stream_ctx(params.stream)
+        saved = _save(target, ctx)
         tried = []
         for d in cands:
             params.conv_algo_desp = d
@@ -126,7 +157,7 @@ class Tuner:
             except (RuntimeError, ValueError):
                 continue     # e.g. a workspace this variant needs and the caller did not give
             tried.append((str(d), ms))
-            target.copy_(saved)
+            target.copy_(saved, ctx)
         if not tried:
             raise RuntimeError("can't find any suitable algo for your parameters.")
         names = [n for n, _ in tried]
@@ -156,7 +187,8 @@ class Tuner:
         cands = gemm_candidates(params, desps)
         if not cands:
             raise RuntimeError("can't find any suitable algo for your parameters.")
-        saved = params.c.clone()
+        ctx = _stream_ctx(params.stream)
+        saved = _save(params.c, ctx)
         tried = []
         for d in cands:
             params.algo_desp = d
@@ -165,7 +197,7 @@ class Tuner:
             except (RuntimeError, ValueError):
                 continue
             tried.append((str(d), ms))
-            params.c.copy_(saved)
+            params.c.copy_(saved, ctx)
         if not tried:
             raise RuntimeError("can't find any suitable algo for your parameters.")
         best = min(tried, key=lambda t: t[1])

@@ -186,7 +186,7 @@ int cumm_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* host out-p
  * linear-probing hash table include/tensorview/hash/linear.cu.h:111-840.
  *
  * cumm_hip_subm_pairs: pair tables of a submanifold convolution.
- *   coords [n, 4] int32 (batch, z, y, x), unique; spatial_shape, ksize (kernel volume <= 32),
+ *   coords [n, 4] int32 (batch, z, y, x), unique; spatial_shape, ksize (odd sizes, kernel volume <= 32),
  *   dilation: 3 ints each (host).  Outputs (device): indices_fwd [kv, n] int32 (-1 = none),
  *   mask_fwd [n] uint32; indices_bwd / mask_bwd may be NULL.  Kernel offset k = (kz*KY + ky)*KX + kx,
  *   output o gathers the input at coord[o] + (k_zyx - ksize/2) * dilation.

@@ -46,17 +46,30 @@ def test_views_share_memory_both_ways():
     assert tb.tensor2torch(u, cast_uint_to_int=True).dtype == torch.int32
 
 
-@pytest.mark.parametrize("strided", [False, True])
+@pytest.mark.parametrize("strided", [False, True, "pad0"])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_autograd_matches_torch_indexing(dtype, strided):
     from cumm_amd import torch_bridge as tb
     print("case torch bridge", dtype, strided, flush=True)
     tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
     coords, grid = H.small_cloud(21, 2500)
+    padding = (1, 1, 1)
+    if strided == "pad0":
+        # stride 2 without padding on even axes: the inputs on the last plane of an axis feed no
+        # output site.  A whole plane of them fills several 128-row tiles whose mask is zero, which
+        # the backward-input kernel skips: their gradient must still come back as zero.
+        padding = (0, 0, 0)
+        zz, yy = np.meshgrid(np.arange(grid[0]), np.arange(grid[1]), indexing="ij")
+        plane = np.stack([np.zeros(zz.size, np.int64), zz.ravel(), yy.ravel(),
+                          np.full(zz.size, grid[2] - 1)], axis=1).astype(np.int32)
+        coords = np.unique(np.concatenate([coords, plane]), axis=0).astype(np.int32)
     c_in, k_out = 64, 96
     torch.manual_seed(3)
-    geo = tb.SparseConvGeometry(torch.as_tensor(coords, device="cuda"), grid, stride=(2, 2, 2) if strided else None)
-    host = pairs.sparse_conv_pairs(coords, grid) if strided else pairs.subm_pairs(coords, grid)
+    geo = tb.SparseConvGeometry(torch.as_tensor(coords, device="cuda"), grid, stride=(2, 2, 2) if strided else None,
+                                padding=padding)
+    host = pairs.sparse_conv_pairs(coords, grid, padding=padding) if strided else pairs.subm_pairs(coords, grid)
+    if strided == "pad0":
+        assert int((host.mask_bwd == 0).sum()) >= 3 * 128
     np.testing.assert_array_equal(H.host(geo.indices_fwd), host.indices_fwd)
     feat = (torch.randn(coords.shape[0], c_in)).to(tdt)
     weight = (torch.randn(k_out, 27, c_in) * 0.05).to(tdt)

@@ -170,3 +170,58 @@ def test_validated_argument_cache_is_invalidated_by_any_assignment():
                          (1.0, 0x3FFF, 64), (1.0, 0x3FFF, 128)]
     finally:
         _capi._lib = real
+
+
+def test_conv_prelude_rejects_wrong_element_types():
+    """Every operand must have the descriptor's element type (the reference's data_ptr<T>()
+    check): the kernels size their buffer descriptors from the descriptor, so a narrower tensor
+    would be read past its end."""
+    cases = [("input", blob([1000, 64], tv.int8)), ("input", blob([1000, 64], tv.float32)),
+             ("weight", blob([64, 27, 64], tv.bfloat16)), ("output", blob([1000, 64], tv.int8)),
+             ("indices", blob([27, 1000], tv.int64)), ("mask_argsort", blob([1000], tv.int64)),
+             ("mask", blob([1000], tv.int32)), ("mask_output", blob([16], tv.int32)),
+             ("bias", blob([64], tv.float32))]
+    for name, bad in cases:
+        p = _fwd_params()
+        setattr(p, name, bad)
+        with pytest.raises(RuntimeError, match="dtype"):
+            ConvMainUnitTest.implicit_gemm2(p)
+    # int8 inference: scale and bias are float32
+    d = [x for x in ConvMainUnitTest.get_all_conv_algo_desp() if x.is_int8_inference][0]
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = d
+    p.input, p.weight, p.output = blob([1000, 64], tv.int8), blob([128, 27, 64], tv.int8), blob([1000, 128], tv.int8)
+    p.indices, p.mask, p.mask_argsort = blob([27, 1000], tv.int32), blob([1000], tv.uint32), blob([1000], tv.int32)
+    p.scale, p.bias = blob([128], tv.float16), blob([128], tv.float32)
+    with pytest.raises(RuntimeError, match="dtype"):
+        ConvMainUnitTest.implicit_gemm2(p)
+
+
+def test_gemm_prelude_rejects_wrong_index_types():
+    d = [x for x in GemmMainUnitTest.get_all_algo_desp()
+         if x.dtype_a == tv.float16 and x.shuffle_type == ShuffleStrideType.ShuffleAC and x.trans_b][0]
+    p = GemmParams()
+    p.algo_desp = d
+    p.a, p.b, p.c = blob([100, 64], tv.float16), blob([64, 64], tv.float16), blob([100, 64], tv.float16)
+    p.c_inds = blob([100], tv.int64)
+    with pytest.raises(RuntimeError, match="dtype"):
+        GemmMainUnitTest.matmul2(p)
+    p.c_inds = blob([100], tv.int32)
+    p.a_inds = blob([100], tv.int64)
+    with pytest.raises(RuntimeError, match="dtype"):
+        GemmMainUnitTest.matmul2(p)
+
+
+def test_full_and_fill_on_bfloat16():
+    """tv.full / fill_float_ on bf16 write bf16 bit patterns (round to nearest even), not the
+    value truncated to an integer."""
+    from cumm_amd import synth
+    for val in (1.0, -2.5, 0.1, 3.0e38, 1.00390625):   # the last one is a tie: rounds to even
+        t = tv.full([3, 4], val, tv.bfloat16)
+        assert t.dtype == tv.bfloat16
+        bits = t.numpy_view()
+        want = synth.f32_to_bf16_bits(np.full((3, 4), val, np.float32))
+        np.testing.assert_array_equal(bits, want)
+    t = tv.zeros([5], tv.bfloat16)
+    t.fill_int_(7)
+    np.testing.assert_array_equal(synth.bf16_bits_to_f32(t.numpy_view()), np.full(5, 7.0, np.float32))

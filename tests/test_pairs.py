@@ -56,3 +56,24 @@ def test_synthetic_cloud_is_unique_in_grid_and_seeded():
     assert len({tuple(r) for r in a.tolist()}) == a.shape[0]
     assert (a[:, 1:] >= 0).all() and (a[:, 1:] < np.array(grid)).all()
     assert abs(a.shape[0] - 5000) < 100
+
+
+def test_subm_backward_table_is_the_inverse_relation_and_even_sizes_are_rejected():
+    """indices_bwd must be the inverse relation of indices_fwd (input i feeds output o through
+    offset k iff o gathers i through k); for odd kernel sizes that is the forward table reversed.
+    Even sizes have asymmetric offsets, for which the reversal is wrong: rejected."""
+    rng = np.random.default_rng(5)
+    grid = (6, 12, 11)
+    coords = synth.clustered_voxels(rng, 250, grid, 3, sigma=2.0)
+    for ksize in ((3, 3, 3), (1, 3, 5), (3, 1, 1)):
+        pt = pairs.subm_pairs(coords, grid, ksize=ksize)
+        kv, n = pt.indices_fwd.shape
+        inv = np.full((kv, n), -1, np.int32)
+        for k in range(kv):
+            o = np.nonzero(pt.indices_fwd[k] >= 0)[0]
+            inv[k, pt.indices_fwd[k, o]] = o
+        np.testing.assert_array_equal(pt.indices_bwd, inv)
+        np.testing.assert_array_equal(pt.mask_bwd, pairs_ref.masks_ref(inv))
+    for ksize in ((1, 1, 2), (2, 2, 2), (3, 4, 3)):
+        with pytest.raises(ValueError, match="odd"):
+            pairs.subm_pairs(coords, grid, ksize=ksize)

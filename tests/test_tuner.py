@@ -46,6 +46,11 @@ def test_conv_candidates_share_the_kind_and_accept_the_problem():
     assert k1 == tuner.Tuner.conv_key(_host_conv_params(ConvOpType.Forward, "f16", 64, 64, n=400))   # same bucket
     assert k1 != tuner.Tuner.conv_key(_host_conv_params(ConvOpType.Forward, "f16", 64, 64, n=5000))
     assert k1 != tuner.Tuner.conv_key(_host_conv_params(ConvOpType.BackwardInput, "f16", 64, 64))
+    # two clouds of one size and a 10x different pair density do not share a cached tile
+    n = p.indices.dim(1)
+    assert tuner.Tuner.conv_key(p, num_pairs=2 * n) != tuner.Tuner.conv_key(p, num_pairs=20 * n)
+    assert tuner.Tuner.conv_key(p, num_pairs=2 * n) == tuner.Tuner.conv_key(p, num_pairs=int(2.2 * n))
+    assert tuner.Tuner.conv_key(p, num_pairs=2 * n) != k1      # unknown density is its own class
 
 
 def test_gemm_candidates():
