@@ -42,7 +42,7 @@ SEED = 20240607
 
 def find_desp(tv_dtype, op, tile_m, tile_n, int8=False, parallel=False):
     for d in ConvMainUnitTest.get_all_conv_algo_desp():
-        if (d.dtype_a == tv_dtype and ConvOpType(d.op_type) == op and d.tile_shape[0] == tile_m
+        if (d.dtype_a == tv_dtype and d.dtype_c == tv_dtype and ConvOpType(d.op_type) == op and d.tile_shape[0] == tile_m
                 and d.tile_shape[1] == tile_n and d.is_int8_inference == int8
                 and d.split_k_parallel == parallel):
             return d
@@ -116,7 +116,7 @@ def bench_wgrad(args, p, dout, n, C, K, tile_m, flops, parallel):
 
 def find_gemm_desp(shuffle, tile_m, tile_n, trans_b):
     for d in GemmMainUnitTest.get_all_algo_desp():
-        if (d.dtype_a == tv.float16 and d.shuffle_type == shuffle and d.tile_shape[0] == tile_m and
+        if (d.dtype_a == tv.float16 and d.dtype_c == tv.float16 and d.shuffle_type == shuffle and d.tile_shape[0] == tile_m and
                 d.tile_shape[1] == tile_n and not d.trans_a and d.trans_b == trans_b and not d.trans_c):
             return d
     raise KeyError((shuffle, tile_m, tile_n, trans_b))

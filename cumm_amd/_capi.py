@@ -82,6 +82,8 @@ SYMBOLS = {
     "cumm_hip_stream_destroy": (C.c_int, [_VP]),
     "cumm_hip_stream_synchronize": (C.c_int, [_VP]),
     "cumm_hip_device_synchronize": (C.c_int, []),
+    "cumm_hip_take_async_errors": (C.c_int, [C.POINTER(C.c_int32)]),
+    "cumm_hip_set_split_k_spin_limit": (C.c_int, [C.c_int]),
     "cumm_hip_event_create": (C.c_int, [_PVP]),
     "cumm_hip_event_destroy": (C.c_int, [_VP]),
     "cumm_hip_event_record": (C.c_int, [_VP, _VP]),

@@ -36,6 +36,9 @@ def _units():
         units.append(("rowgemm_" + name, os.path.join(CSRC, "rowgemm_inst.hip"), defs))
         extra = ["-DCUMM_NO_WGRAD_ATOMIC"] if tag == "S8" else []   # no s8 backward pass
         units.append(("tilegemm_" + name, os.path.join(CSRC, "tilegemm_inst.hip"), defs + extra))
+        # the same kernels with four-byte outputs (s8 -> s32, f16 / bf16 -> f32)
+        units.append(("rowgemm_wide_" + name, os.path.join(CSRC, "rowgemm_inst.hip"), defs + ["-DCUMM_WIDE=1"]))
+        units.append(("tilegemm_wide_" + name, os.path.join(CSRC, "tilegemm_inst.hip"), defs + ["-DCUMM_WIDE=1"]))
     return units
 
 

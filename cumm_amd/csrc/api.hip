@@ -1,6 +1,7 @@
 // C ABI of libcummhip.so: argument checks, kernel selection and launches.
 #include "../../include/cumm_hip.h"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -49,37 +50,49 @@ int pick_ks(int c_in, int dt) {
   return 4;
 }
 
-bool same_dtype3(const CummHipGemmDesc &d) {
-  return d.dtype_a == d.dtype_b && d.dtype_a == d.dtype_c &&
-         (is_float16_like(d.dtype_a) || d.dtype_a == CUMM_HIP_S8);
+// four-byte output of the accumulator type: s8 x s8 -> s32 ("s8,s8,s32,s32,s32",
+// cumm/gemm/main.py:350-364,500-523 of the reference), f16 / bf16 -> f32
+bool wide_out(const CummHipGemmDesc &d) {
+  return d.dtype_a == CUMM_HIP_S8 ? d.dtype_c == CUMM_HIP_S32 : d.dtype_c == CUMM_HIP_F32;
 }
 
+// operands of one element type; the output of the same type or of the accumulator's
+bool same_dtype3(const CummHipGemmDesc &d) {
+  return d.dtype_a == d.dtype_b && (is_float16_like(d.dtype_a) || d.dtype_a == CUMM_HIP_S8) &&
+         (d.dtype_a == d.dtype_c || wide_out(d));
+}
+
+// accumulator and arithmetic type of the linear combination: f32 / f32; s8 operands accumulate in
+// s32 and combine in f32 (s8 output, the requantising epilogues) or in s32 (s32 output)
 bool acc_ok(const CummHipGemmDesc &d) {
-  if (d.dtype_a == CUMM_HIP_S8) return d.dacc == CUMM_HIP_S32 && d.dcomp == CUMM_HIP_F32;
+  if (d.dtype_a == CUMM_HIP_S8)
+    return d.dacc == CUMM_HIP_S32 && d.dcomp == (d.dtype_c == CUMM_HIP_S32 ? CUMM_HIP_S32 : CUMM_HIP_F32);
   return d.dacc == CUMM_HIP_F32 && d.dcomp == CUMM_HIP_F32;
 }
 
-hipError_t launch_rowgemm(int dt, int tm, int tn, int ks, bool wt, const RowGemmParams &p,
+hipError_t launch_rowgemm(int dt, bool wide, int tm, int tn, int ks, bool wt, const RowGemmParams &p,
                           hipStream_t s) {
   switch (dt) {
-  case CUMM_HIP_F16: return launch_rowgemm_f16(tm, tn, ks, wt, p, s);
-  case CUMM_HIP_BF16: return launch_rowgemm_bf16(tm, tn, ks, wt, p, s);
-  case CUMM_HIP_S8: return launch_rowgemm_s8(tm, tn, ks, wt, p, s);
+  case CUMM_HIP_F16: return wide ? launch_rowgemm_wide_f16(tm, tn, ks, wt, p, s) : launch_rowgemm_f16(tm, tn, ks, wt, p, s);
+  case CUMM_HIP_BF16: return wide ? launch_rowgemm_wide_bf16(tm, tn, ks, wt, p, s) : launch_rowgemm_bf16(tm, tn, ks, wt, p, s);
+  case CUMM_HIP_S8: return wide ? launch_rowgemm_wide_s8(tm, tn, ks, wt, p, s) : launch_rowgemm_s8(tm, tn, ks, wt, p, s);
   }
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_tilegemm(int dt, int tm, int tn, bool xk, bool yk, const TileGemmParams &p,
+hipError_t launch_tilegemm(int dt, bool wide, int tm, int tn, bool xk, bool yk, const TileGemmParams &p,
                            dim3 grid, hipStream_t s) {
   switch (dt) {
-  case CUMM_HIP_F16: return launch_tilegemm_f16(tm, tn, xk, yk, p, grid, s);
-  case CUMM_HIP_BF16: return launch_tilegemm_bf16(tm, tn, xk, yk, p, grid, s);
-  case CUMM_HIP_S8: return launch_tilegemm_s8(tm, tn, xk, yk, p, grid, s);
+  case CUMM_HIP_F16: return wide ? launch_tilegemm_wide_f16(tm, tn, xk, yk, p, grid, s) : launch_tilegemm_f16(tm, tn, xk, yk, p, grid, s);
+  case CUMM_HIP_BF16: return wide ? launch_tilegemm_wide_bf16(tm, tn, xk, yk, p, grid, s) : launch_tilegemm_bf16(tm, tn, xk, yk, p, grid, s);
+  case CUMM_HIP_S8: return wide ? launch_tilegemm_wide_s8(tm, tn, xk, yk, p, grid, s) : launch_tilegemm_s8(tm, tn, xk, yk, p, grid, s);
   }
   return hipErrorInvalidValue;
 }
 
-constexpr int kSpinLimit = 1 << 24;
+// bound on the polls of a serial split-K semaphore (cumm_hip_set_split_k_spin_limit)
+constexpr int kDefaultSpinLimit = 1 << 24;
+std::atomic<int> g_spin_limit{kDefaultSpinLimit};
 
 // byte extent of a row-major 2-D operand for the buffer range checks; false if it does not fit
 // below 2 GiB (the kernels use 32-bit offsets and reserve the upper half for "absent")
@@ -118,11 +131,13 @@ int conv_family(const CummHipConvDesc &c) {
   if (tk != mk) return 0;
   if (d.split_k_parallel) {
     // only the balanced backward-weight kernel (fp32 atomic partial sums) splits "in parallel"
-    if (c.op_type != CUMM_HIP_OP_BACKWARD_WEIGHT || d.dtype_a == CUMM_HIP_S8 || d.split_k_serial) return 0;
+    if (c.op_type != CUMM_HIP_OP_BACKWARD_WEIGHT || d.dtype_a == CUMM_HIP_S8 || d.split_k_serial || wide_out(d)) return 0;
     if (!d.trans_a || d.trans_b || d.trans_c) return 0;
     return (tm == 64 && tn == 64) ? 3 : 0;
   }
-  if (c.is_int8_inference && (d.dtype_a != CUMM_HIP_S8 || c.op_type != CUMM_HIP_OP_FORWARD)) return 0;
+  if (c.is_int8_inference && (d.dtype_a != CUMM_HIP_S8 || c.op_type != CUMM_HIP_OP_FORWARD || wide_out(d))) return 0;
+  // (the weight gradient keeps the weight's type, as every kernel of the reference does)
+  if (wide_out(d) && c.op_type == CUMM_HIP_OP_BACKWARD_WEIGHT) return 0;
   if (c.op_type == CUMM_HIP_OP_FORWARD || c.op_type == CUMM_HIP_OP_BACKWARD_INPUT) {
     if (d.split_k_serial) return 0;
     return rowgemm_has_tile(tm, tn) ? 1 : 0;
@@ -135,11 +150,15 @@ int conv_family(const CummHipConvDesc &c) {
 }
 
 void fill_gemm_desc(CummHipGemmDesc &d, int dt, int ta, int tb, int tc, int tm, int tn, int shuffle,
-                    int splitk) {
+                    int splitk, bool wide = false) {
   std::memset(&d, 0, sizeof(d));
   d.dtype_a = d.dtype_b = d.dtype_c = dt;
   d.dacc = dt == CUMM_HIP_S8 ? CUMM_HIP_S32 : CUMM_HIP_F32;
   d.dcomp = CUMM_HIP_F32;
+  if (wide) {
+    d.dtype_c = d.dacc;
+    d.dcomp = d.dacc;
+  }
   d.trans_a = ta; d.trans_b = tb; d.trans_c = tc;
   const int tk = dt == CUMM_HIP_S8 ? 64 : 32;
   d.tile_shape[0] = tm; d.tile_shape[1] = tn; d.tile_shape[2] = tk;
@@ -196,6 +215,60 @@ int static_scratch(void **out) {
   return CUMM_HIP_OK;
 }
 
+// ---- failures that a kernel can only report after the fact.  Word 0 counts the serial split-K
+// slices whose bounded semaphore wait ran out (tilegemm.h); the synchronising entry points read
+// and clear it and turn a non-zero count into an error.  One array per GPU, like `scratch`.
+static __device__ int32_t async_status[4];
+int32_t *g_status_ptr[kMaxDevices] = {};
+
+int async_status_ptr(int32_t **out) {
+  int dev = -1;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(CUMM_HIP_ERUNTIME, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (g_status_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(async_status)));
+    if (ptr == nullptr) return fail(CUMM_HIP_ERUNTIME, "hipGetSymbolAddress returned no address for the status words");
+    g_status_ptr[dev] = reinterpret_cast<int32_t *>(ptr);
+  }
+  *out = g_status_ptr[dev];
+  return CUMM_HIP_OK;
+}
+
+// After a synchronisation: anything to report on this device?  (Nothing was ever launched that
+// could report: no device access at all.)
+int take_async_errors(int32_t *timeouts) {
+  *timeouts = 0;
+  int dev = -1;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return CUMM_HIP_OK;
+  int32_t *ptr;
+  {
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    ptr = g_status_ptr[dev];
+  }
+  if (ptr == nullptr) return CUMM_HIP_OK;
+  int32_t words[4] = {0, 0, 0, 0};
+  HIP_TRY(hipMemcpy(words, ptr, sizeof(words), hipMemcpyDeviceToHost));
+  if (words[0] != 0) {
+    const int32_t zero[4] = {0, 0, 0, 0};
+    HIP_TRY(hipMemcpy(ptr, zero, sizeof(zero), hipMemcpyHostToDevice));
+  }
+  *timeouts = words[0];
+  return CUMM_HIP_OK;
+}
+
+int report_async_errors() {
+  int32_t timeouts = 0;
+  if (int rc = take_async_errors(&timeouts)) return rc;
+  if (timeouts != 0)
+    return fail(CUMM_HIP_ERUNTIME,
+                "serial split-K: %d slice(s) gave up waiting for their turn at the semaphore; the results of "
+                "those launches are invalid", (int)timeouts);
+  return CUMM_HIP_OK;
+}
+
 int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a, void *stream_, void *workspace,
                      size_t workspace_bytes, size_t workspace_cap);
 
@@ -213,11 +286,13 @@ int cumm_hip_list_gemm_algos(CummHipGemmDesc *out, int cap) {
   const int dts[3] = {CUMM_HIP_F16, CUMM_HIP_BF16, CUMM_HIP_S8};
   const int row_tiles[4][2] = {{64, 64}, {128, 64}, {64, 128}, {128, 128}};
   const int sq_tiles[2][2] = {{64, 64}, {128, 128}};
+  // every kernel with the output in the operands' type and in the accumulator's (s32 / f32)
+  for (int wide = 0; wide < 2; ++wide)
   for (int dt : dts) {
     for (auto &t : row_tiles)
       for (int tb = 0; tb < 2; ++tb) {
         CummHipGemmDesc d;
-        fill_gemm_desc(d, dt, 0, tb, 0, t[0], t[1], CUMM_HIP_SHUFFLE_AC, 0);
+        fill_gemm_desc(d, dt, 0, tb, 0, t[0], t[1], CUMM_HIP_SHUFFLE_AC, 0, wide != 0);
         d.warp_tile_shape[0] = t[0] / 4; d.warp_tile_shape[1] = t[1]; d.warp_tile_shape[2] = d.tile_shape[2];
         v.push_back(d);
       }
@@ -226,12 +301,12 @@ int cumm_hip_list_gemm_algos(CummHipGemmDesc *out, int cap) {
         for (int tb = 0; tb < 2; ++tb)
           for (int tc = 0; tc < 2; ++tc) {
             CummHipGemmDesc d;
-            fill_gemm_desc(d, dt, ta, tb, tc, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 1);
+            fill_gemm_desc(d, dt, ta, tb, tc, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 1, wide != 0);
             d.warp_tile_shape[0] = t[0] / 2; d.warp_tile_shape[1] = t[1] / 2; d.warp_tile_shape[2] = d.tile_shape[2];
             v.push_back(d);
           }
       CummHipGemmDesc d;
-      fill_gemm_desc(d, dt, 1, 0, 0, t[0], t[1], CUMM_HIP_SHUFFLE_AB, 1);
+      fill_gemm_desc(d, dt, 1, 0, 0, t[0], t[1], CUMM_HIP_SHUFFLE_AB, 1, wide != 0);
       d.warp_tile_shape[0] = t[0] / 2; d.warp_tile_shape[1] = t[1] / 2; d.warp_tile_shape[2] = d.tile_shape[2];
       v.push_back(d);
     }
@@ -250,15 +325,16 @@ int cumm_hip_list_conv_algos(CummHipConvDesc *out, int cap) {
   };
   const int fdts[2] = {CUMM_HIP_F16, CUMM_HIP_BF16};
   for (int dt : fdts) {
+    for (int wide = 0; wide < 2; ++wide)   // output in the operands' type, then in f32
     for (auto &t : row_tiles) {
       // forward: A = input [N,C] row major, B = weight [K, kv*C] ("tn"), C = output
       CummHipConvDesc c;
-      fill_gemm_desc(c.gemm, dt, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      fill_gemm_desc(c.gemm, dt, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, wide != 0);
       c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
       base(c, CUMM_HIP_OP_FORWARD);
       v.push_back(c);
       // backward input: A = dOut [N,K], B = weight viewed [kv*K, C] ("tt")
-      fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, wide != 0);
       c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
       base(c, CUMM_HIP_OP_BACKWARD_INPUT);
       v.push_back(c);
@@ -282,12 +358,14 @@ int cumm_hip_list_conv_algos(CummHipConvDesc *out, int cap) {
     }
   }
   for (auto &t : row_tiles) {
-    for (int s8inf = 0; s8inf < 2; ++s8inf) {
+    // s8 forward: s8 output through alpha / beta, s8 output through the int8-inference epilogue,
+    // and the raw s32 accumulators
+    for (int kind = 0; kind < 3; ++kind) {
       CummHipConvDesc c;
-      fill_gemm_desc(c.gemm, CUMM_HIP_S8, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      fill_gemm_desc(c.gemm, CUMM_HIP_S8, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, kind == 2);
       c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 64;
       base(c, CUMM_HIP_OP_FORWARD);
-      c.is_int8_inference = s8inf;
+      c.is_int8_inference = kind == 1;
       v.push_back(c);
     }
   }
@@ -304,6 +382,11 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
   hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
   const int dt = d.dtype_a;
   const int pv = per_vec(dt);
+  const bool wide = wide_out(d);
+  const int pvc = wide ? 4 : pv;             // elements of C / D per 16-byte piece
+  const int ebc = wide ? 4 : elem_bytes(dt); // bytes of an element of C / D
+  if (wide && d.dtype_c == CUMM_HIP_S32 && a->act_type == CUMM_HIP_ACT_SIGMOID)
+    return fail(CUMM_HIP_EINVAL, "no sigmoid in integer arithmetic (s32 output)");
   if (a->m < 0 || a->n < 0 || a->k < 0) return fail(CUMM_HIP_EINVAL, "negative m, n or k");
   if (a->m == 0 || a->n == 0) return CUMM_HIP_OK;
   if (!a->ptr_A || !a->ptr_B || !a->ptr_C) return fail(CUMM_HIP_ERUNTIME, "a,b,c must not empty");
@@ -319,7 +402,7 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
   if (fam == 1) {
     // ShuffleAC: C[c_inds[i]] = act(alpha * A[a_inds[i]] @ op(B) + beta * D[c_inds[i]])
     if (!a->indiceBorC) return fail(CUMM_HIP_ERUNTIME, "a_inds,c_inds tensor must not empty");
-    if (a->k % pv || a->n % pv || a->stride_A % pv || a->stride_B % pv || a->stride_C % pv || ldd % pv)
+    if (a->k % pv || a->n % pv || a->stride_A % pv || a->stride_B % pv || a->stride_C % pvc || ldd % pvc)
       return fail(CUMM_HIP_EINVAL, "this m, n, k isn't supported due to misaligned contiguous dim.");
     RowGemmParams p;
     std::memset(&p, 0, sizeof(p));
@@ -346,11 +429,11 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
     const int64_t b_rows = d.trans_b ? a->n : a->k, b_cols = d.trans_b ? a->k : a->n;
     if (!extent32(a->rows_A, a->stride_A, a->k, eb, &p.a_bytes) ||
         !extent32(b_rows, a->stride_B, b_cols, eb, &p.w_bytes) ||
-        !extent32(a->rows_C, a->stride_C, a->n, eb, &p.c_bytes) ||
-        !extent32(ldd ? a->rows_C : 1, ldd, a->n, eb, &p.d_bytes))
+        !extent32(a->rows_C, a->stride_C, a->n, ebc, &p.c_bytes) ||
+        !extent32(ldd ? a->rows_C : 1, ldd, a->n, ebc, &p.d_bytes))
       return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
     p.gather_bytes = (uint32_t)a->m * 4u;
-    hipError_t e = launch_rowgemm(dt, d.tile_shape[0], d.tile_shape[1], pick_ks(a->k, dt), !d.trans_b, p, stream);
+    hipError_t e = launch_rowgemm(dt, wide, d.tile_shape[0], d.tile_shape[1], pick_ks(a->k, dt), !d.trans_b, p, stream);
     if (e != hipSuccess) return hip_fail(e, "gather-GEMM-scatter launch");
     return CUMM_HIP_OK;
   }
@@ -381,7 +464,7 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
   p.m = m; p.n = n; p.k = a->k; p.kv = 1; p.mask_filter = 0xffffffffu;
   p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act = a->act_type;
   p.split_k = a->split_k_slices;
-  p.spin_limit = kSpinLimit;
+  p.spin_limit = g_spin_limit.load();
   p.rows_x = 0x7fffffff; p.rows_y = 0x7fffffff;
   bool xk, yk;
   if (d.shuffle_type == CUMM_HIP_SHUFFLE_AB) {
@@ -402,8 +485,10 @@ int cumm_hip_gemm(const CummHipGemmDesc *desc, const CummHipGemmArgs *a, void *s
     if (reinterpret_cast<uintptr_t>(a->workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
     HIP_TRY(zero_device(a->workspace, need, stream));
     p.sem = reinterpret_cast<int32_t *>(a->workspace);
+    if (int rc = async_status_ptr(&p.timeouts)) return rc;
   }
-  hipError_t e = launch_tilegemm(dt, tm, tn, xk, yk, p, grid, stream);
+  p.split_contig = 1;
+  hipError_t e = launch_tilegemm(dt, wide, tm, tn, xk, yk, p, grid, stream);
   if (e != hipSuccess) return hip_fail(e, "GEMM launch");
   return CUMM_HIP_OK;
 }
@@ -435,6 +520,9 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
   hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
   const int dt = d.dtype_a;
   const int pv = per_vec(dt);
+  const bool wide = wide_out(d);
+  if (wide && d.dtype_c == CUMM_HIP_S32 && a->act_type == CUMM_HIP_ACT_SIGMOID)
+    return fail(CUMM_HIP_EINVAL, "no sigmoid in integer arithmetic (s32 output)");
   const int kv = a->kernel_volume;
   if (a->N < 0 || a->C <= 0 || a->K <= 0 || kv <= 0) return fail(CUMM_HIP_EINVAL, "bad N, C, K or kernel volume");
   if (kv > 32) return fail(CUMM_HIP_EINVAL, "kernel volume > 32 needs dynamic_mask, which this build has no kernel for");
@@ -485,15 +573,15 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
       p.bias = reinterpret_cast<const float *>(a->bias_pointer);
       p.ldd = p.ldc;  // the only source of the int8 epilogue is output_add (or the output itself)
     }
-    const int eb = elem_bytes(dt);
+    const int eb = elem_bytes(dt), ebc = wide ? 4 : eb;
     if (!extent32(p.rows_a, p.lda, p.c_in, eb, &p.a_bytes) ||
         !extent32((int64_t)a->K * kv, a->C, a->C, eb, &p.w_bytes) ||
-        !extent32(p.rows_c, p.ldc, p.k_out, eb, &p.c_bytes) ||
-        !extent32(p.ldd ? p.rows_c : 1, p.ldd, p.k_out, eb, &p.d_bytes) ||
+        !extent32(p.rows_c, p.ldc, p.k_out, ebc, &p.c_bytes) ||
+        !extent32(p.ldd ? p.rows_c : 1, p.ldd, p.k_out, ebc, &p.d_bytes) ||
         (int64_t)kv * a->N * 4 >= (int64_t)1 << 31)
       return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
     p.gather_bytes = (uint32_t)((int64_t)kv * a->N * 4);
-    hipError_t e = launch_rowgemm(dt, d.tile_shape[0], d.tile_shape[1], pick_ks(p.c_in, dt), !fwd, p, stream);
+    hipError_t e = launch_rowgemm(dt, wide, d.tile_shape[0], d.tile_shape[1], pick_ks(p.c_in, dt), !fwd, p, stream);
     if (e != hipSuccess) return hip_fail(e, "sparse conv launch");
     return CUMM_HIP_OK;
   }
@@ -578,7 +666,7 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
   p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act = a->act_type;
   p.split_k = a->split_k_slices < 1 ? 1 : a->split_k_slices;
   if (fam == 3) p.split_k = 1;   // a single slice needs no partial sums: plain tiled kernel
-  p.spin_limit = kSpinLimit;
+  p.spin_limit = g_spin_limit.load();
   const int n_tiles = (a->C + tn - 1) / tn;
   dim3 grid((a->K + tm - 1) / tm, n_tiles * kv, p.split_k);
   if (p.split_k > 1) {
@@ -590,8 +678,9 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
     HIP_TRY(zero_device(workspace, need, stream));
     p.sem = reinterpret_cast<int32_t *>(workspace);
+    if (int rc = async_status_ptr(&p.timeouts)) return rc;
   }
-  hipError_t e = launch_tilegemm(dt, tm, tn, false, false, p, grid, stream);
+  hipError_t e = launch_tilegemm(dt, false, tm, tn, false, false, p, grid, stream);
   if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
   return CUMM_HIP_OK;
 }
@@ -663,10 +752,19 @@ int cumm_hip_stream_destroy(void *stream) {
 }
 int cumm_hip_stream_synchronize(void *stream) {
   HIP_TRY(hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream)));
-  return CUMM_HIP_OK;
+  return report_async_errors();
 }
 int cumm_hip_device_synchronize(void) {
   HIP_TRY(hipDeviceSynchronize());
+  return report_async_errors();
+}
+int cumm_hip_take_async_errors(int32_t *split_k_timeouts) {
+  if (!split_k_timeouts) return fail(CUMM_HIP_EINVAL, "null out-param");
+  return take_async_errors(split_k_timeouts);
+}
+int cumm_hip_set_split_k_spin_limit(int polls) {
+  if (polls < 0) return fail(CUMM_HIP_EINVAL, "the number of polls must not be negative (0 = the default)");
+  g_spin_limit.store(polls == 0 ? kDefaultSpinLimit : polls);
   return CUMM_HIP_OK;
 }
 int cumm_hip_event_create(void **event) {

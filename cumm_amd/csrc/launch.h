@@ -12,12 +12,24 @@ hipError_t launch_rowgemm_f16(int tm, int tn, int ks, bool wt, const RowGemmPara
 hipError_t launch_rowgemm_bf16(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s);
 hipError_t launch_rowgemm_s8(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s);
 
+// the same tables with four-byte outputs (s32 for s8 operands, f32 for f16 / bf16)
+hipError_t launch_rowgemm_wide_f16(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s);
+hipError_t launch_rowgemm_wide_bf16(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s);
+hipError_t launch_rowgemm_wide_s8(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s);
+
 hipError_t launch_tilegemm_f16(int tm, int tn, bool xk, bool yk, const TileGemmParams &p, dim3 grid,
                                hipStream_t s);
 hipError_t launch_tilegemm_bf16(int tm, int tn, bool xk, bool yk, const TileGemmParams &p, dim3 grid,
                                 hipStream_t s);
 hipError_t launch_tilegemm_s8(int tm, int tn, bool xk, bool yk, const TileGemmParams &p, dim3 grid,
                               hipStream_t s);
+
+hipError_t launch_tilegemm_wide_f16(int tm, int tn, bool xk, bool yk, const TileGemmParams &p, dim3 grid,
+                                    hipStream_t s);
+hipError_t launch_tilegemm_wide_bf16(int tm, int tn, bool xk, bool yk, const TileGemmParams &p, dim3 grid,
+                                     hipStream_t s);
+hipError_t launch_tilegemm_wide_s8(int tm, int tn, bool xk, bool yk, const TileGemmParams &p, dim3 grid,
+                                   hipStream_t s);
 
 // balanced backward-weight with fp32 atomics: main kernel then finalize (f16 / bf16 only)
 hipError_t launch_wgrad_atomic_f16(const WgradParams &p, const WgradPrepareParams &pre, const WgradFinalizeParams &f, hipStream_t s);

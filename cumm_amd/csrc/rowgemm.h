@@ -28,6 +28,8 @@
 //   * tiles are handed out heaviest first; each wave owns RB blocks of 16 rows and skips a block
 //     none of whose rows has a pair at offset k (its contribution would be exactly zero).
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace cummhip {
@@ -67,11 +69,50 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint3
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
 }
 
+// Four-byte outputs (s32 for s8 operands, f32 for f16 / bf16 operands; "s8,s8,s32,s32,s32" in
+// cumm/gemm/main.py:350-364,500-523 of the reference): the accumulators themselves go through
+// the linear combination, whose arithmetic type (dcomp) is then the output type: for s32 alpha
+// and beta are converted to integers and alpha*acc + beta*src is integer arithmetic
+// (LinearCombination, cumm/gemm/output_op/linear.py:54-146; UnaryActivation on integers,
+// cumm/gemm/gemmmath/__init__.py:181-214).  One piece = four consecutive channels of one row.
+template <class AccV>
+__device__ __forceinline__ void store_wide_piece(const AccV &a, const RowGemmParams &p, __amdgpu_buffer_rsrc_t rs_c,
+                                                 __amdgpu_buffer_rsrc_t rs_d, bool ok, int o, int ch) {
+  const uint32_t coff = ok ? (uint32_t)((int64_t)o * p.ldc + ch) * 4u : kOob;
+  v4i src = {0, 0, 0, 0};
+  if (p.read_source) {
+    const uint32_t doff = ok ? (uint32_t)((int64_t)o * p.ldd + ch) * 4u : kOob;
+    src = __builtin_amdgcn_raw_buffer_load_b128(rs_d, doff, 0, 0);
+  }
+  v4i outv;
+  if constexpr (std::is_same<AccV, v4i>::value) {
+    // (unsigned arithmetic: wraps like the reference's int32 arithmetic, without undefined overflow)
+    const uint32_t ai = (uint32_t)(int)p.alpha, bi = (uint32_t)(int)p.beta, la = (uint32_t)(int)p.act_alpha;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      int t = (int)(ai * (uint32_t)a[x] + (p.read_source ? bi * (uint32_t)src[x] : 0u));
+      if (p.act == 1) t = t > 0 ? t : 0;
+      else if (p.act == 3) t = t >= 0 ? t : (int)((uint32_t)t * la);
+      outv[x] = t;
+    }
+  } else {
+    const v4f sf = __builtin_bit_cast(v4f, src);
+    v4f of;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const float t = p.read_source ? __builtin_fmaf(p.alpha, a[x], p.beta * sf[x]) : p.alpha * a[x];
+      of[x] = apply_act(t, p.act, p.act_alpha);
+    }
+    outv = __builtin_bit_cast(v4i, of);
+  }
+  __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
+}
+
 // T: element tag; NW: waves per workgroup; RB: 16-row blocks per wave; TN: output channels per
 // workgroup; KS: 16-byte fragments per lane per channel chunk; WT: weight is contiguous along the
 // output channel (needs a transposing stage) instead of along the contraction; B: kernel offsets
-// per batch.
-template <class T, int NW, int RB, int TN, int KS, bool WT, int B>
+// per batch; WIDE: four-byte outputs (see store_wide_piece).
+template <class T, int NW, int RB, int TN, int KS, bool WT, int B, bool WIDE = false>
 __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
@@ -349,6 +390,20 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
   const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.c_bytes);
   const __amdgpu_buffer_rsrc_t rs_d = make_rsrc(p.D, p.read_source ? p.d_bytes : 0u);
   const int ch0 = n0 + q * CPL;
+  if constexpr (WIDE) {
+    // lane (m, q): channels ch0 + 4*nb .. +3 of block nb, one 16-byte piece each
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int o = out_row[rb];
+      const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const int ch = ch0 + nb * 4;
+        store_wide_piece(acc[rb][nb], p, rs_c, rs_d, row_ok && ch < p.k_out, o, ch);
+      }
+    }
+    return;
+  }
   if constexpr (E::kBytes == 2) {
     constexpr int NG = CPL / 8;  // 16-byte groups of 8 channels
 #pragma unroll

@@ -12,6 +12,18 @@ namespace cummhip {
 #define CUMM_CAT_(a, b) a##b
 #define CUMM_CAT(a, b) CUMM_CAT_(a, b)
 
+// -DCUMM_WIDE=1 builds the same table with four-byte outputs (s32 / f32) under the name
+// launch_rowgemm_wide_<type>, in a translation unit of its own
+#ifndef CUMM_WIDE
+#define CUMM_WIDE 0
+#endif
+constexpr bool kWide = CUMM_WIDE != 0;
+#if CUMM_WIDE
+#define CUMM_LAUNCH_NAME CUMM_CAT(launch_rowgemm_wide_, CUMM_NAME)
+#else
+#define CUMM_LAUNCH_NAME CUMM_CAT(launch_rowgemm_, CUMM_NAME)
+#endif
+
 // kernel offsets per batch of the chunked kernel: bounded by the two LDS stages (TN * 64 * KS
 // bytes per offset and stage, at most 32 KB per workgroup) and by the registers that hold the
 // batch's gathered rows
@@ -57,7 +69,7 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
       if (shift <= 3 && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
         RowGemmParams q = p;
         q.chunk_shift = shift;
-        hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 2, NS2, WT>), grid, dim3(256), 0, s, q);
+        hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 2, NS2, WT, kWide>), grid, dim3(256), 0, s, q);
         return hipGetLastError();
       }
     }
@@ -66,18 +78,18 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   if constexpr (NS > 0 && (!WT || Elem<T>::kBytes == 2)) {
     // the LDS-streaming kernel: 2 x 2 waves, each TM/2 rows by TN/2 channels
     if (p.c_in <= chunk_e && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
-      hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS, WT>), grid, dim3(256), 0, s, p);
+      hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS, WT, kWide>), grid, dim3(256), 0, s, p);
       return hipGetLastError();
     }
   }
   if (p.c_in <= chunk_e) {
     constexpr int BW = step_width(TN, KS);
     constexpr int DA = rows_ahead(RB, KS, BW);
-    hipLaunchKernelGGL((rowgemm_pipe_kernel<T, NW, RB, TN, KS, WT, BW, DA, DA, CUMM_DW>), grid, dim3(NW * 64), 0, s, p);
+    hipLaunchKernelGGL((rowgemm_pipe_kernel<T, NW, RB, TN, KS, WT, BW, DA, DA, CUMM_DW, kWide>), grid, dim3(NW * 64), 0, s, p);
   } else {
     if constexpr (KS == 4) {
       constexpr int B = batch_size(RB, TN, KS);
-      hipLaunchKernelGGL((rowgemm_kernel<T, NW, RB, TN, KS, WT, B>), grid, dim3(NW * 64), 0, s, p);
+      hipLaunchKernelGGL((rowgemm_kernel<T, NW, RB, TN, KS, WT, B, kWide>), grid, dim3(NW * 64), 0, s, p);
     } else {
       return hipErrorInvalidValue;  // a contraction longer than one chunk always selects KS == 4
     }
@@ -103,8 +115,7 @@ static hipError_t launch_ks(int ks, bool wt, const RowGemmParams &p, hipStream_t
   return hipErrorInvalidValue;
 }
 
-hipError_t CUMM_CAT(launch_rowgemm_, CUMM_NAME)(int tm, int tn, int ks, bool wt,
-                                                const RowGemmParams &p, hipStream_t s) {
+hipError_t CUMM_LAUNCH_NAME(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s) {
   using T = CUMM_ELEM;
   if (tm == 64 && tn == 64) return launch_ks<T, 4, 1, 64>(ks, wt, p, s);
   if (tm == 128 && tn == 64) return launch_ks<T, 4, 2, 64>(ks, wt, p, s);

@@ -52,7 +52,9 @@ __device__ __forceinline__ bool run_steps(F &f, std::integer_sequence<int, Is...
 // that lane i/4 + 4j points to.  Lane s of a group points to row (first k) + s/4, channels
 // 4*(s%4) .. +3 of its 16-channel block, so lane i receives 4 consecutive k of channel i; two
 // reads make one operand.  A lane then owns channels nb*16 + 4q .. +3 of each block nb.
-template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT = false>
+// WIDE: four-byte outputs (s32 / f32: the accumulators through the linear combination, see
+// store_wide_piece in rowgemm.h).
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT = false, bool WIDE = false>
 __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmParams p) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
@@ -373,7 +375,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   };
   typedef int src_vec __attribute__((ext_vector_type(SRC_W)));
   src_vec src_pre[RBW][SRC_N] = {};
-  if (p.read_source) {
+  if (p.read_source && !WIDE) {   // (four-byte outputs read their source in the epilogue)
     const v4i rsw_d = rsrc_words(p.D, p.d_bytes);
 #pragma unroll
     for (int rb = 0; rb < RBW; ++rb) {
@@ -500,6 +502,20 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   // The activation and the blend mode are lifted out of the element loops (one straight-line
   // copy per combination): tested per element they cost more issue slots than the arithmetic.
   const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.c_bytes);
+  if constexpr (WIDE) {
+    const __amdgpu_buffer_rsrc_t rs_d = make_rsrc(p.D, p.read_source ? p.d_bytes : 0u);
+#pragma unroll
+    for (int rb = 0; rb < RBW; ++rb) {
+      const int o = out_row[rb];
+      const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+      for (int nb = 0; nb < NBW; ++nb) {
+        const int ch = ch0 + nb * 4;
+        store_wide_piece(acc[rb][nb], p, rs_c, rs_d, row_ok && ch < p.k_out, o, ch);
+      }
+    }
+    return;
+  }
   // MODE: 0 = alpha*acc, 1 = alpha*acc + beta*src, 2 = scale*acc + bias, 3 = ... + beta*src
   auto store_rows = [&](auto act_c, auto mode_c) {
     constexpr int ACT = decltype(act_c)::value;

@@ -39,7 +39,7 @@ __device__ __forceinline__ bool run_unrolled(F &f, std::integer_sequence<int, Is
   return (f(std::integral_constant<int, Is>{}) || ...);
 }
 
-template <class T, int NW, int RB, int TN, int KS, bool WT, int BW, int DA, int DI, int DW>
+template <class T, int NW, int RB, int TN, int KS, bool WT, int BW, int DA, int DI, int DW, bool WIDE = false>
 __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmParams p) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
@@ -388,6 +388,20 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
   const __amdgpu_buffer_rsrc_t rs_c = make_rsrc(p.C, p.c_bytes);
   const __amdgpu_buffer_rsrc_t rs_d = make_rsrc(p.D, p.read_source ? p.d_bytes : 0u);
   const int ch0 = n0 + q * CPL;
+  if constexpr (WIDE) {
+    // lane (m, q): channels ch0 + 4*nb .. +3 of block nb, one 16-byte piece each
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int o = out_row[rb];
+      const bool row_ok = o >= 0 && o < p.rows_c;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const int ch = ch0 + nb * 4;
+        store_wide_piece(acc[rb][nb], p, rs_c, rs_d, row_ok && ch < p.k_out, o, ch);
+      }
+    }
+    return;
+  }
   if constexpr (E::kBytes == 2) {
     constexpr int NG = CPL / 8;
 #pragma unroll

@@ -38,10 +38,19 @@ struct TileGemmParams {
   int32_t split_k;
   int32_t *sem;            // [grid.x * grid.y] zeroed before launch (serial split-K)
   int32_t spin_limit;      // bound on semaphore polls
+  int32_t *timeouts;       // counts the slices whose wait ran into the bound (the host reports them)
+  // plain GEMM: slice z owns the contiguous range of k-steps [z * per, (z + 1) * per), per =
+  // ceil(steps / split_k) (GemmUtils::get_gemm_k_size_per_split, include/tensorview/gemm/core/utils.h:30-37
+  // of the reference); backward-weight: slices interleave (z, z + split_k, ...)
+  int32_t split_contig;
 };
 
 // XK / YK: operand is contraction-contiguous in memory.  BM x BN 16x16 blocks per wave, 2x2 waves.
-template <class T, bool XK, bool YK, int BM, int BN, int KSTEPS>
+// WIDE: four-byte outputs (s32 for s8 operands, f32 for f16 / bf16 operands): the accumulators
+// through a linear combination in the output type, integer arithmetic for s32 ("s8,s8,s32,s32,s32",
+// cumm/gemm/main.py:350-364 of the reference; LinearCombination with dcomp = s32,
+// cumm/gemm/output_op/linear.py:54-146).
+template <class T, bool XK, bool YK, int BM, int BN, int KSTEPS, bool WIDE = false>
 __global__ __launch_bounds__(256) void tilegemm_kernel(const TileGemmParams p) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
@@ -83,9 +92,13 @@ __global__ __launch_bounds__(256) void tilegemm_kernel(const TileGemmParams p) {
     const uint32_t mw = mi < p.num_red_mask ? p.red_mask[mi] : 0u;
     return (mw >> r_off) & 1u;
   };
+  const int per_slice = (steps + p.split_k - 1) / p.split_k;
+  const int s_begin = p.split_contig ? z * per_slice : z;
+  const int s_end = p.split_contig ? (steps < (z + 1) * per_slice ? steps : (z + 1) * per_slice) : steps;
+  const int s_inc = p.split_contig ? 1 : p.split_k;
   auto next_live = [&](int s) -> int {
-    while (s < steps && !step_live(s)) s += p.split_k;
-    return s < steps ? s : -1;
+    while (s < s_end && !step_live(s)) s += s_inc;
+    return s < s_end ? s : -1;
   };
 
   // ---- per-thread staging assignment
@@ -235,12 +248,12 @@ __global__ __launch_bounds__(256) void tilegemm_kernel(const TileGemmParams p) {
 
   // ---- main loop: steps z, z + split, ... (slices interleave, cumm/gemm/blockmma/mma.py:634-655
   // of the reference); steps whose reduced mask lacks this offset's bit are skipped.
-  int s = next_live(z);
+  int s = next_live(s_begin);
   if (s >= 0) load_tiles(s);
   while (s >= 0) {
     store_tiles();
     __syncthreads();
-    const int s_next = next_live(s + p.split_k);
+    const int s_next = next_live(s + s_inc);
     if (s_next >= 0) load_tiles(s_next);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
@@ -271,11 +284,17 @@ __global__ __launch_bounds__(256) void tilegemm_kernel(const TileGemmParams p) {
     lock = p.sem + (blockIdx.x + blockIdx.y * gridDim.x);
     if (tid == 0) {
       int spins = 0;
-      while (__hip_atomic_load(lock, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != z &&
-             spins < p.spin_limit) {
+      bool mine = __hip_atomic_load(lock, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == z;
+      while (!mine && spins < p.spin_limit) {
         __builtin_amdgcn_s_sleep(8);
         ++spins;
+        mine = __hip_atomic_load(lock, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == z;
       }
+      // The wait is bounded so that no wave can spin for ever.  A slice that gives up goes on
+      // without its turn - the sum it writes is then not to be trusted - and says so: the host
+      // reports the count as an error at its next synchronisation.
+      if (!mine && p.timeouts != nullptr)
+        __hip_atomic_fetch_add(p.timeouts, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (z > 0) beta = 1.0f;
@@ -293,7 +312,32 @@ __global__ __launch_bounds__(256) void tilegemm_kernel(const TileGemmParams p) {
       if (nn >= p.n) continue;
       const int64_t coff = (int64_t)mm * p.ldc + (int64_t)r_off * p.c_off + nn;
       const int64_t doff = (int64_t)mm * p.ldd + (p.ldd ? (int64_t)r_off * p.c_off : 0) + nn;
-      if constexpr (E::kBytes == 2) {
+      if constexpr (WIDE) {
+        int32_t *cp = reinterpret_cast<int32_t *>(p.C) + coff;
+        v4i sv = {0, 0, 0, 0};
+        if (read_src) sv = *reinterpret_cast<const v4i *>((z > 0) ? cp : reinterpret_cast<const int32_t *>(p.D) + doff);
+        v4i ov;
+        if constexpr (E::kBytes == 1) {
+          const uint32_t ai = (uint32_t)(int)p.alpha, bi = (uint32_t)(int)beta, la = (uint32_t)(int)p.act_alpha;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            int t = (int)(ai * (uint32_t)acc[i][j][r] + (read_src ? bi * (uint32_t)sv[r] : 0u));
+            if (p.act == 1) t = t > 0 ? t : 0;
+            else if (p.act == 3) t = t >= 0 ? t : (int)((uint32_t)t * la);
+            ov[r] = t;
+          }
+        } else {
+          const v4f sf = __builtin_bit_cast(v4f, sv);
+          v4f of;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float t = read_src ? __builtin_fmaf(p.alpha, acc[i][j][r], beta * sf[r]) : p.alpha * acc[i][j][r];
+            of[r] = apply_act(t, p.act, p.act_alpha);
+          }
+          ov = __builtin_bit_cast(v4i, of);
+        }
+        *reinterpret_cast<v4i *>(cp) = ov;
+      } else if constexpr (E::kBytes == 2) {
         uint16_t *cp = reinterpret_cast<uint16_t *>(p.C) + coff;
         uint2 sv = {0, 0};
         if (read_src) {

@@ -7,13 +7,25 @@ namespace cummhip {
 #define CUMM_CAT_(a, b) a##b
 #define CUMM_CAT(a, b) CUMM_CAT_(a, b)
 
+// -DCUMM_WIDE=1 builds the tiled kernels with four-byte outputs (s32 / f32) under the name
+// launch_tilegemm_wide_<type>, in a translation unit of its own (and nothing else)
+#ifndef CUMM_WIDE
+#define CUMM_WIDE 0
+#endif
+constexpr bool kWide = CUMM_WIDE != 0;
+#if CUMM_WIDE
+#define CUMM_LAUNCH_NAME CUMM_CAT(launch_tilegemm_wide_, CUMM_NAME)
+#else
+#define CUMM_LAUNCH_NAME CUMM_CAT(launch_tilegemm_, CUMM_NAME)
+#endif
+
 template <class T, int BM, int BN>
 static hipError_t launch_xy(bool xk, bool yk, const TileGemmParams &p, dim3 grid, hipStream_t s) {
   if (grid.x == 0 || grid.y == 0 || grid.z == 0) return hipSuccess;
-  if (xk && yk) hipLaunchKernelGGL((tilegemm_kernel<T, true, true, BM, BN, 1>), grid, dim3(256), 0, s, p);
-  else if (xk && !yk) hipLaunchKernelGGL((tilegemm_kernel<T, true, false, BM, BN, 1>), grid, dim3(256), 0, s, p);
-  else if (!xk && yk) hipLaunchKernelGGL((tilegemm_kernel<T, false, true, BM, BN, 1>), grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((tilegemm_kernel<T, false, false, BM, BN, 1>), grid, dim3(256), 0, s, p);
+  if (xk && yk) hipLaunchKernelGGL((tilegemm_kernel<T, true, true, BM, BN, 1, kWide>), grid, dim3(256), 0, s, p);
+  else if (xk && !yk) hipLaunchKernelGGL((tilegemm_kernel<T, true, false, BM, BN, 1, kWide>), grid, dim3(256), 0, s, p);
+  else if (!xk && yk) hipLaunchKernelGGL((tilegemm_kernel<T, false, true, BM, BN, 1, kWide>), grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((tilegemm_kernel<T, false, false, BM, BN, 1, kWide>), grid, dim3(256), 0, s, p);
   return hipGetLastError();
 }
 
@@ -54,19 +66,20 @@ static bool launch_dense_ring(const TileGemmParams &p, hipStream_t s, hipError_t
   }
 }
 
-hipError_t CUMM_CAT(launch_tilegemm_, CUMM_NAME)(int tm, int tn, bool xk, bool yk,
-                                                 const TileGemmParams &p, dim3 grid, hipStream_t s) {
+hipError_t CUMM_LAUNCH_NAME(int tm, int tn, bool xk, bool yk, const TileGemmParams &p, dim3 grid, hipStream_t s) {
   using T = CUMM_ELEM;
-  if (xk && yk) {
-    hipError_t err = hipSuccess;
-    if (launch_dense_ring<T>(p, s, &err)) return err;
+  if constexpr (!kWide) {
+    if (xk && yk) {
+      hipError_t err = hipSuccess;
+      if (launch_dense_ring<T>(p, s, &err)) return err;
+    }
   }
   if (tm == 64 && tn == 64) return launch_xy<T, 2, 2>(xk, yk, p, grid, s);
   if (tm == 128 && tn == 128) return launch_xy<T, 4, 4>(xk, yk, p, grid, s);
   return hipErrorInvalidValue;
 }
 
-#ifndef CUMM_NO_WGRAD_ATOMIC
+#if !defined(CUMM_NO_WGRAD_ATOMIC) && !CUMM_WIDE
 hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const WgradPrepareParams &pre,
                                                      const WgradFinalizeParams &f, hipStream_t s) {
   using T = CUMM_ELEM;

@@ -53,7 +53,7 @@ def desp_from_c(d: _capi.GemmDesc, out: GemmAlgoDesp) -> GemmAlgoDesp:
     epa = _EPA[d.dtype_a]
     out.element_per_access_a = epa
     out.element_per_access_b = epa
-    out.element_per_access_c = epa
+    out.element_per_access_c = epa if d.dtype_c == d.dtype_a else 4   # 16-byte pieces of s32 / f32
     out.access_per_vector = 1
     out.min_arch = (9, 5)   # gfx950
     return out

@@ -80,7 +80,7 @@ _TUNER = tuner.Tuner(steps=3, warmup=1)
 
 def _desp_like(dtype, op, parallel=False):
     for d in ConvMainUnitTest.get_all_conv_algo_desp():
-        if (d.dtype_a == dtype and ConvOpType(d.op_type) == op and not d.is_int8_inference and
+        if (d.dtype_a == dtype and d.dtype_c == dtype and ConvOpType(d.op_type) == op and not d.is_int8_inference and
                 bool(d.split_k_parallel) == parallel and d.mask_sparse):
             return d
     raise RuntimeError("can't find any suitable algo for your parameters.")

@@ -168,9 +168,19 @@ int cumm_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 int cumm_hip_memset(void *ptr, int value, size_t bytes, void *stream);
 int cumm_hip_stream_create(void **stream);             /* host out-param; default priority */
 int cumm_hip_stream_destroy(void *stream);
-/* GemmMainUnitTest.stream_synchronize / device_synchronize (cumm/gemm/main.py:1028-1047) */
+/* GemmMainUnitTest.stream_synchronize / device_synchronize (cumm/gemm/main.py:1028-1047).
+ * Both also report what a kernel could only find out while running: a serial split-K slice whose
+ * bounded wait at the semaphore (tv::Semaphore, include/tensorview/gemm/arch/semaphore.h:37-100,
+ * waits without a bound) ran out went on without its turn and counted itself; a non-zero count
+ * comes back here as CUMM_HIP_ERUNTIME (once; the count is cleared). */
 int cumm_hip_stream_synchronize(void *stream);
 int cumm_hip_device_synchronize(void);
+/* The same count for callers that synchronise by other means (e.g. through torch): reads and
+ * clears the current device's count of timed-out split-K slices.  Call after a synchronisation. */
+int cumm_hip_take_async_errors(int32_t *split_k_timeouts);   /* host out-param */
+/* Polls a split-K slice makes before it gives up (0 = the default of 2^24, about a second).  For
+ * tests of the time-out path and for workloads with very long slices. */
+int cumm_hip_set_split_k_spin_limit(int polls);
 
 /* ---- events: tv::CUDAEvent / CUDAKernelTimer (include/tensorview/profile/cuda_profiler.h:97-406) */
 int cumm_hip_event_create(void **event);               /* host out-param */

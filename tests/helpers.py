@@ -9,7 +9,7 @@ from cumm_amd.gemm.main import GemmMainUnitTest
 from cumm_amd.tensorview.gemm import (Activation, ConvOpType, ConvParams, GemmParams,
                                       ShuffleStrideType)
 
-TV_DTYPE = {"f16": tv.float16, "bf16": tv.bfloat16, "s8": tv.int8, "f32": tv.float32}
+TV_DTYPE = {"f16": tv.float16, "bf16": tv.bfloat16, "s8": tv.int8, "f32": tv.float32, "s32": tv.int32}
 
 
 def to_storage(x_f32, dtype):
@@ -20,6 +20,8 @@ def to_storage(x_f32, dtype):
         return synth.f32_to_bf16_bits(x_f32)
     if dtype == "s8":
         return x_f32.astype(np.int8)
+    if dtype == "s32":
+        return x_f32.astype(np.int32)
     return x_f32.astype(np.float32)
 
 
@@ -48,18 +50,32 @@ def rel_err(got_f32, ref_f32):
     return float(np.max(np.abs(got_f32.astype(np.float64) - ref_f32.astype(np.float64)))) / denom
 
 
-def find_conv_desp(dtype, op, tile_m, tile_n, int8_inference=False, split_k_parallel=False):
+def rel_err_rows(got_f32, ref_f32, floor_frac=1e-2):
+    """The same, normalised per row: max over rows of max |got-ref| over the row / max |ref| over
+    the row, so that a wrong row of small magnitude cannot hide under the tensor's largest
+    value.  Rows whose own maximum is below ``floor_frac`` of the tensor's are measured against
+    that floor (rounding noise of a near-zero row is not a relative error)."""
+    g = got_f32.astype(np.float64).reshape(got_f32.shape[0], -1)
+    r = ref_f32.astype(np.float64).reshape(ref_f32.shape[0], -1)
+    floor = max(float(np.max(np.abs(r))) * floor_frac, 1e-6)
+    denom = np.maximum(np.max(np.abs(r), axis=1), floor)
+    return float(np.max(np.max(np.abs(g - r), axis=1) / denom))
+
+
+def find_conv_desp(dtype, op, tile_m, tile_n, int8_inference=False, split_k_parallel=False, dtype_out=None):
+    """``dtype_out``: element type of the result when it differs from the operands' ("s32", "f32")."""
     for d in ConvMainUnitTest.get_all_conv_algo_desp():
-        if (d.dtype_a == TV_DTYPE[dtype] and ConvOpType(d.op_type) == op and
+        if (d.dtype_a == TV_DTYPE[dtype] and d.dtype_output == TV_DTYPE[dtype_out or dtype] and
+                d.dtype_input == TV_DTYPE[dtype] and ConvOpType(d.op_type) == op and
                 d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and
                 d.is_int8_inference == int8_inference and d.split_k_parallel == split_k_parallel):
             return d
     raise KeyError((dtype, op, tile_m, tile_n, int8_inference, split_k_parallel))
 
 
-def find_gemm_desp(dtype, shuffle, tile_m, tile_n, trans_a, trans_b, trans_c=False):
+def find_gemm_desp(dtype, shuffle, tile_m, tile_n, trans_a, trans_b, trans_c=False, dtype_c=None):
     for d in GemmMainUnitTest.get_all_algo_desp():
-        if (d.dtype_a == TV_DTYPE[dtype] and d.shuffle_type == shuffle and
+        if (d.dtype_a == TV_DTYPE[dtype] and d.dtype_c == TV_DTYPE[dtype_c or dtype] and d.shuffle_type == shuffle and
                 d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and
                 d.trans_a == trans_a and d.trans_b == trans_b and d.trans_c == trans_c):
             return d

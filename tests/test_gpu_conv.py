@@ -407,3 +407,112 @@ def test_int8_inference_leaky_relu_bit_exact(act_alpha):
     got = H.host(p.output)
     np.testing.assert_array_equal(got, ref)
     assert (got < 0).any() and (got > 0).any()
+
+
+@pytest.mark.parametrize("tile", [(64, 64), (128, 64), (64, 128), (128, 128)])
+@pytest.mark.parametrize("strided", [False, True])
+def test_s8_forward_s32_accumulators_bit_exact(tile, strided):
+    """The "s8,s8,s32,s32,s32" kind: the raw s32 accumulators, and the integer linear combination
+    with a source and ReLU, bit for bit against the oracle's exact integer sums."""
+    print("case s8 -> s32", tile, strided, flush=True)
+    c_in, k_out = 64, 128
+    rng, coords, pt, feat, w, n_in, n_out = _case(25, 3000, c_in, k_out, "s8", strided=strided)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    src = rng.integers(-100000, 100000, size=(n_out, k_out)).astype(np.int32)
+    desp = H.find_conv_desp("s8", ConvOpType.Forward, *tile, dtype_out="s32")
+    _, mo, acc = conv_ref.implicit_gemm_fwd_ref(
+        feat, w, src, pt.indices_fwd, ms, order, tile_m=tile[0], dtype_in="s8", dtype_w="s8",
+        dtype_out="s32", return_acc=True)
+    for alpha, beta, act in ((1.0, 0.0, Activation.None_), (2.0, -1.0, Activation.ReLU)):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = desp
+        p.input, p.weight, p.output = H.dev(feat, "s8"), H.dev(w, "s8"), H.dev(src, "s32")
+        p.indices = H.dev(pt.indices_fwd, "i32")
+        p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+        p.mask_output = tv.zeros([(n_out + tile[0] - 1) // tile[0]], tv.uint32, 0)
+        p.alpha, p.beta, p.act_type = alpha, beta, act
+        ConvMainUnitTest.implicit_gemm2(p)
+        ref, _ = conv_ref.implicit_gemm_fwd_ref(
+            feat, w, src, pt.indices_fwd, ms, order, tile_m=tile[0], dtype_in="s8", dtype_w="s8",
+            dtype_out="s32", alpha=alpha, beta=beta, act=act.value)
+        got = H.host(p.output)
+        np.testing.assert_array_equal(got, ref)
+        np.testing.assert_array_equal(H.host(p.mask_output), mo)
+        if beta == 0.0:
+            np.testing.assert_array_equal(got, acc)     # alpha = 1: the accumulators themselves
+        else:                                           # the closed form on the exact sums
+            want = np.maximum(2 * acc.astype(np.int64) - src.astype(np.int64), 0)
+            np.testing.assert_array_equal(got.astype(np.int64), want)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("tile", [(64, 64), (128, 128)])
+def test_f32_output_forward_and_backward_input(dtype, tile):
+    """f16 / bf16 operands with the fp32 accumulators as the output (no rounding to 16 bits)."""
+    print("case f32 out", dtype, tile, flush=True)
+    c_in, k_out = 64, 96
+    rng, coords, pt, feat, w, n_in, n_out = _case(26, 2500, c_in, k_out, dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    out0 = rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32)
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, *tile, dtype_out="f32")
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, "f32")
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    p.alpha, p.beta = 0.5, 1.0
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref, _ = conv_ref.implicit_gemm_fwd_ref(
+        feat, w, out0, pt.indices_fwd, ms, order, tile_m=tile[0], dtype_in=dtype, dtype_w=dtype,
+        dtype_out="f32", alpha=0.5, beta=1.0)
+    assert H.rel_err(H.host(p.output), ref) < 2e-3
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    din0 = np.zeros((n_in, c_in), np.float32)
+    q = ConvParams(3, ConvOpType.BackwardInput)
+    # (the input gradient is the GEMM's C operand: dtype_c f32; dtype_output names the conv output, dOut)
+    q.conv_algo_desp = [d for d in ConvMainUnitTest.get_all_conv_algo_desp()
+                        if d.dtype_a == H.TV_DTYPE[dtype] and d.dtype_c == tv.float32 and
+                        ConvOpType(d.op_type) == ConvOpType.BackwardInput and list(d.tile_shape[:2]) == list(tile)][0]
+    q.input, q.weight, q.output = H.dev(din0, "f32"), H.dev(w, dtype), H.dev(dout, dtype)
+    q.indices = H.dev(pt.indices_bwd, "i32")
+    q.mask, q.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    q.reverse_mask = True
+    ConvMainUnitTest.implicit_gemm2(q)
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(
+        dout, w, din0, pt.indices_bwd, ms, order, tile_m=tile[0], dtype_in=dtype, dtype_w=dtype,
+        dtype_out="f32", reverse_mask=True)
+    assert H.rel_err(H.host(q.input), ref_d) < 2e-3
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_long_contraction_forward_and_backward_input(dtype):
+    """640 channels on the contraction side: more than eight stage rows, which the chunked
+    register-gather kernel serves (forward: C = 640; backward-input: K = 640)."""
+    print("case long contraction", dtype, flush=True)
+    c_in, k_out = 640, 64
+    rng, coords, pt, feat, w, n_in, n_out = _case(27, 600, c_in, k_out, dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    out0 = H.to_storage(np.zeros((n_out, k_out), np.float32), dtype)
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, 64, 64)
+    p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    ConvMainUnitTest.implicit_gemm2(p)
+    ref, _ = conv_ref.implicit_gemm_fwd_ref(
+        feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+    assert H.rel_err(H.as_f32(H.host(p.output), dtype), H.as_f32(ref, dtype)) < TOL
+    # backward-input with the roles swapped: K = 640 is the contraction
+    w2 = H.to_storage(rng.normal(0, 0.05, size=(640, 27, 64)).astype(np.float32), dtype)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, 640)).astype(np.float32), dtype)
+    din0 = H.to_storage(np.zeros((n_in, 64), np.float32), dtype)
+    q = ConvParams(3, ConvOpType.BackwardInput)
+    q.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, 64, 64)
+    q.input, q.weight, q.output = H.dev(din0, dtype), H.dev(w2, dtype), H.dev(dout, dtype)
+    q.indices = H.dev(pt.indices_bwd, "i32")
+    q.mask, q.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+    q.reverse_mask = True
+    ConvMainUnitTest.implicit_gemm2(q)
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(
+        dout, w2, din0, pt.indices_bwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype,
+        dtype_out=dtype, reverse_mask=True)
+    assert H.rel_err(H.as_f32(H.host(q.input), dtype), H.as_f32(ref_d, dtype)) < TOL

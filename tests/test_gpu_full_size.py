@@ -47,6 +47,7 @@ def test_subm_f16_c64_forward_dgrad_full_size(tile_m):
                                                    dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
     got = H.as_f32(H.host(p.output), dtype)
     assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+    assert H.rel_err_rows(got, H.as_f32(ref, dtype)) < TOL           # every row by its own scale
     np.testing.assert_array_equal(H.host(p.mask_output), mask_out)   # integer work: bit-exact
 
     # linearity: conv(2 x) == 2 conv(x); scaling by two is exact in f32 and in normal f16 (no
@@ -75,6 +76,7 @@ def test_subm_f16_c64_forward_dgrad_full_size(tile_m):
     ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, din0, pt.indices_bwd, ms, order, tile_m=tile_m,
                                              dtype_in=dtype, dtype_w=dtype, dtype_out=dtype, reverse_mask=True)
     assert H.rel_err(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_d, dtype)) < TOL
+    assert H.rel_err_rows(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_d, dtype)) < TOL
 
 
 def test_subm_f16_c64_wgrad_full_size():
@@ -100,6 +102,9 @@ def test_subm_f16_c64_wgrad_full_size():
         dout, feat, dw0, pt.indices_fwd, red, order, mask_width=tile_m, dtype_dout=dtype,
         dtype_in=dtype, dtype_w=dtype, split_k_slices=1)
     assert H.rel_err(H.as_f32(H.host(p.weight), dtype), H.as_f32(ref, dtype)) < TOL
+    # per (output channel, kernel offset) row of the gradient
+    assert H.rel_err_rows(H.as_f32(H.host(p.weight), dtype).reshape(64 * 27, 64),
+                          H.as_f32(ref, dtype).reshape(64 * 27, 64)) < TOL
 
 
 def test_s8_stride2_full_size_bit_exact():
@@ -121,10 +126,24 @@ def test_s8_stride2_full_size_bit_exact():
     p.indices = H.dev(pt.indices_fwd, "i32")
     p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
     ConvMainUnitTest.implicit_gemm2(p)
-    ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in="s8",
-                                            dtype_w="s8", dtype_out="s8", scale=scale, bias=bias,
-                                            int8_inference=True)
+    ref, _, acc = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in="s8",
+                                                 dtype_w="s8", dtype_out="s8", scale=scale, bias=bias,
+                                                 int8_inference=True, return_acc=True)
     np.testing.assert_array_equal(H.host(p.output), ref)
+
+    # the s32 accumulators themselves ("s8,s8,s32,s32,s32"): bit-exact against the oracle's
+    # exact integer sums, and through the integer linear combination with a source
+    src = rng.integers(-1000, 1000, size=(n_out, 128)).astype(np.int32)
+    q = ConvParams(3, ConvOpType.Forward)
+    q.conv_algo_desp = H.find_conv_desp("s8", ConvOpType.Forward, 64, 128, dtype_out="s32")
+    q.input, q.weight, q.output = p.input, p.weight, H.dev(src, "s32")
+    q.indices, q.mask, q.mask_argsort = p.indices, p.mask, p.mask_argsort
+    ConvMainUnitTest.implicit_gemm2(q)
+    np.testing.assert_array_equal(H.host(q.output), acc)
+    q.output = H.dev(src, "s32")
+    q.alpha, q.beta = 3.0, -2.0
+    ConvMainUnitTest.implicit_gemm2(q)
+    np.testing.assert_array_equal(H.host(q.output).astype(np.int64), 3 * acc.astype(np.int64) - 2 * src.astype(np.int64))
 
 
 def test_gather_gemm_scatter_full_size():
@@ -148,6 +167,7 @@ def test_gather_gemm_scatter_full_size():
                                shuffle=gemm_ref.SHUFFLE_AC, a_inds=a_inds, c_inds=c_inds, alpha=1.0, beta=1.0)
     got = H.as_f32(H.host(p.c), dtype)
     assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+    assert H.rel_err_rows(got, H.as_f32(ref, dtype)) < TOL
     untouched = np.setdiff1d(np.arange(rows), c_inds)
     np.testing.assert_array_equal(H.host(p.c)[untouched], c0[untouched])   # rows not in c_inds stay as they were
 

@@ -46,7 +46,8 @@ def _fwd_params():
     n = 1000
     p = ConvParams(3, ConvOpType.Forward)
     p.conv_algo_desp = [d for d in ConvMainUnitTest.get_all_conv_algo_desp()
-                        if d.dtype_a == tv.float16 and ConvOpType(d.op_type) == ConvOpType.Forward][0]
+                        if d.dtype_a == tv.float16 and d.dtype_c == tv.float16 and
+                        ConvOpType(d.op_type) == ConvOpType.Forward][0]
     p.input, p.weight, p.output = blob([n, 64], tv.float16), blob([64, 27, 64], tv.float16), blob([n, 64], tv.float16)
     p.indices, p.mask, p.mask_argsort = blob([27, n], tv.int32), blob([n], tv.uint32), blob([n], tv.int32)
     return p
@@ -91,7 +92,8 @@ def test_conv_prelude_errors():
 
 def test_gemm_prelude_errors():
     d = [x for x in GemmMainUnitTest.get_all_algo_desp()
-         if x.dtype_a == tv.float16 and x.shuffle_type == ShuffleStrideType.ShuffleAC and x.trans_b][0]
+         if x.dtype_a == tv.float16 and x.dtype_c == tv.float16 and
+         x.shuffle_type == ShuffleStrideType.ShuffleAC and x.trans_b][0]
     p = GemmParams()
     p.algo_desp = d
     with pytest.raises(RuntimeError, match="a,b,c must not empty"):
@@ -187,7 +189,7 @@ def test_conv_prelude_rejects_wrong_element_types():
         with pytest.raises(RuntimeError, match="dtype"):
             ConvMainUnitTest.implicit_gemm2(p)
     # int8 inference: scale and bias are float32
-    d = [x for x in ConvMainUnitTest.get_all_conv_algo_desp() if x.is_int8_inference][0]
+    d = [x for x in ConvMainUnitTest.get_all_conv_algo_desp() if x.is_int8_inference and x.dtype_c == tv.int8][0]
     p = ConvParams(3, ConvOpType.Forward)
     p.conv_algo_desp = d
     p.input, p.weight, p.output = blob([1000, 64], tv.int8), blob([128, 27, 64], tv.int8), blob([1000, 128], tv.int8)
@@ -199,7 +201,8 @@ def test_conv_prelude_rejects_wrong_element_types():
 
 def test_gemm_prelude_rejects_wrong_index_types():
     d = [x for x in GemmMainUnitTest.get_all_algo_desp()
-         if x.dtype_a == tv.float16 and x.shuffle_type == ShuffleStrideType.ShuffleAC and x.trans_b][0]
+         if x.dtype_a == tv.float16 and x.dtype_c == tv.float16 and
+         x.shuffle_type == ShuffleStrideType.ShuffleAC and x.trans_b][0]
     p = GemmParams()
     p.algo_desp = d
     p.a, p.b, p.c = blob([100, 64], tv.float16), blob([64, 64], tv.float16), blob([100, 64], tv.float16)

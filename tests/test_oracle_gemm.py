@@ -86,3 +86,62 @@ def test_int8_accumulator_is_exact_and_f16_rounds_once():
     want = (af.astype(np.float64) @ bf.astype(np.float64))
     np.testing.assert_allclose(got.astype(np.float64), want, rtol=2e-3, atol=2e-3)
     assert got.dtype == np.float16
+
+
+def test_s32_output_is_integer_arithmetic():
+    """Output type s32 of s8 operands: alpha and beta become integers (C conversion, toward zero)
+    and alpha*acc + beta*src is integer arithmetic.  Pinned by a brute-force product in Python
+    integers, by the conversion numpy's C cast makes, and by wrap-around at 2^31."""
+    rng = np.random.default_rng(11)
+    m, n, k = 5, 7, 9
+    a = rng.integers(-127, 128, size=(m, k)).astype(np.int8)
+    b = rng.integers(-127, 128, size=(k, n)).astype(np.int8)
+    c0 = rng.integers(-10 ** 6, 10 ** 6, size=(m, n)).astype(np.int32)
+    brute = [[sum(int(a[i, t]) * int(b[t, j]) for t in range(k)) for j in range(n)] for i in range(m)]
+    got = gr.matmul2_ref(a, b, c0, dtype_a="s8", dtype_b="s8", dtype_c="s32")
+    assert got.dtype == np.int32 and got.tolist() == brute
+    got = gr.matmul2_ref(a, b, c0, dtype_a="s8", dtype_b="s8", dtype_c="s32", alpha=3.0, beta=-2.0)
+    assert got.tolist() == [[3 * brute[i][j] - 2 * int(c0[i, j]) for j in range(n)] for i in range(m)]
+    # fractional parameters convert toward zero: 2.9 -> 2, -1.5 -> -1, 0.5 -> 0 (source not needed)
+    for alpha, beta in ((2.9, -1.5), (-2.9, 0.5)):
+        ai, bi = int(np.float32(alpha).astype(np.int32)), int(np.float32(beta).astype(np.int32))
+        got = gr.matmul2_ref(a, b, c0, dtype_a="s8", dtype_b="s8", dtype_c="s32", alpha=alpha, beta=beta)
+        assert got.tolist() == [[ai * brute[i][j] + bi * int(c0[i, j]) for j in range(n)] for i in range(m)]
+    # ReLU and LeakyReLU on integers
+    got = gr.matmul2_ref(a, b, c0, dtype_a="s8", dtype_b="s8", dtype_c="s32", act=nm.ACT_RELU)
+    assert got.tolist() == [[max(v, 0) for v in row] for row in brute]
+    got = gr.matmul2_ref(a, b, c0, dtype_a="s8", dtype_b="s8", dtype_c="s32", act=nm.ACT_LEAKY_RELU, act_alpha=3.7)
+    assert got.tolist() == [[v if v >= 0 else 3 * v for v in row] for row in brute]
+    # overflow wraps modulo 2^32
+    big = gr.linear_combination_s32(np.array([2 ** 30 + 5], np.int32), None, 4.0, 0.0, nm.ACT_NONE, 0.0)
+    assert int(big[0]) == ((4 * (2 ** 30 + 5) + 2 ** 31) % 2 ** 32) - 2 ** 31 == 20
+
+
+def test_serial_split_k_slices_round_between_slices():
+    """Slices are contiguous ranges of k of ceil(ceil(k / tile_k) / slices) * tile_k elements (the
+    size is pinned against the reference's header in test_desp.py); every slice after the first
+    adds onto the rounded result of the one before."""
+    assert gr.split_k_ranges(656, 4, 32) == [(0, 192), (192, 384), (384, 576), (576, 656)]
+    assert gr.split_k_ranges(64, 4, 32) == [(0, 32), (32, 64), (64, 64), (64, 64)]
+    assert gr.split_k_ranges(100, 3, 64) == [(0, 64), (64, 100), (100, 100)]
+    rng = np.random.default_rng(12)
+    m, n, k = 6, 10, 100
+    a = rng.normal(0, 1, size=(m, k)).astype(np.float16)
+    b = rng.normal(0, 1, size=(k, n)).astype(np.float16)
+    c0 = rng.normal(0, 1, size=(m, n)).astype(np.float16)
+    got = gr.matmul2_ref(a, b, c0, dtype_a="f16", dtype_b="f16", dtype_c="f16", alpha=0.5, beta=2.0,
+                         split_k_slices=3, tile_k=64)
+    af, bf = a.astype(np.float32), b.astype(np.float32)
+    step1 = (np.float32(0.5) * (af[:, :64] @ bf[:64]) + np.float32(2.0) * c0.astype(np.float32)).astype(np.float16)
+    step2 = (np.float32(0.5) * (af[:, 64:] @ bf[64:]) + step1.astype(np.float32)).astype(np.float16)
+    # (fused vs unfused multiply-add may differ in the last f16 digit)
+    assert np.max(np.abs(got.astype(np.float32) - step2.astype(np.float32))) <= 2 * np.max(np.abs(np.spacing(step2)))
+    one = gr.matmul2_ref(a, b, c0, dtype_a="f16", dtype_b="f16", dtype_c="f16", alpha=0.5, beta=2.0)
+    assert np.any(one != got)        # a single rounding is not the same thing
+    # integers: exact whatever the slicing
+    ai = rng.integers(-127, 128, size=(m, 300)).astype(np.int8)
+    bi = rng.integers(-127, 128, size=(300, n)).astype(np.int8)
+    ci = rng.integers(-1000, 1000, size=(m, n)).astype(np.int32)
+    s1 = gr.matmul2_ref(ai, bi, ci, dtype_a="s8", dtype_b="s8", dtype_c="s32", beta=1.0)
+    s4 = gr.matmul2_ref(ai, bi, ci, dtype_a="s8", dtype_b="s8", dtype_c="s32", beta=1.0, split_k_slices=4, tile_k=64)
+    np.testing.assert_array_equal(s1, s4)
