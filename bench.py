@@ -195,12 +195,18 @@ def bench_stack(args):
     prep_ms = (time.perf_counter() - t0) * 1e3          # first call, allocations included
     n_out2 = int(table2.indices_fwd.dim(1))
     prep = {}
-    for name, fn in (("subm_pairs", lambda: pairs.subm_pairs_device(d_coords, grid)),
-                     ("sort_by_mask", lambda: pairs.sort_by_mask_device(table.mask_fwd)),
+    # result tensors and workspaces of the first call are handed back in: nothing is allocated
+    from cumm_amd import _capi
+    lib = _capi.lib()
+    ws_p = tv.empty([int(lib.cumm_hip_subm_pairs_workspace(n))], tv.uint8, 0)
+    ws_s = tv.empty([int(lib.cumm_hip_sort_by_mask_workspace(max(n, n_out2)))], tv.uint8, 0)
+    sorted1, sorted2 = (ms_tv, order_tv), (ms2_tv, order2_tv)
+    for name, fn in (("subm_pairs", lambda: pairs.subm_pairs_device(d_coords, grid, workspace=ws_p, out=table)),
+                     ("sort_by_mask", lambda: pairs.sort_by_mask_device(table.mask_fwd, workspace=ws_s, out=sorted1)),
                      ("sparse_conv_pairs_stride2", lambda: pairs.sparse_conv_pairs_device(d_coords, grid, batch_size=1)),
-                     ("sort_by_mask_stride2", lambda: pairs.sort_by_mask_device(table2.mask_fwd))):
-        wms, _ = timed(fn, 5, 2)     # (wall clock: allocation of the result tensors included)
-        prep[name] = round(wms, 4)
+                     ("sort_by_mask_stride2", lambda: pairs.sort_by_mask_device(table2.mask_fwd, workspace=ws_s, out=sorted2))):
+        wms, ems = timed(fn, 5, 2)
+        prep[name] = {"wall_ms": round(wms, 4), "events_ms": round(ems, 4)}
     pairs1 = int((table.indices_fwd.cpu().numpy() >= 0).sum())
     pairs2 = int((table2.indices_fwd.cpu().numpy() >= 0).sum())
     x, w, b = bf16((n, c), 1 / 64), bf16((c, 27, c), 1 / 2048), bf16((c,), 1 / 512)
@@ -251,7 +257,97 @@ def bench_stack(args):
     p2.input, p2.weight, p2.bias, p2.output = x, w2, b2, tv.zeros([n_out2, 256], tv.bfloat16, 0)
     p2.indices, p2.mask, p2.mask_argsort = table2.indices_fwd, ms2_tv, order2_tv
     p2.beta, p2.act_type = 1.0, Activation.ReLU
+    red2 = tv.zeros([(n_out2 + 63) // 64], tv.uint32, 0)
     leg("stride2_c128_c256_forward", p2, 2.0 * pairs2 * c * 256)
+    # the stride-2 layer's backward passes: input gradient on the input-side masks, weight gradient
+    # on the reduced masks of a 64-row forward
+    dout2 = bf16((n_out2, 256), 1 / 64)
+    msb2_tv, orderb2_tv = pairs.sort_by_mask_device(table2.mask_bwd)
+    pd2 = ConvParams(3, ConvOpType.BackwardInput)
+    pd2.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.BackwardInput, 128, 128)
+    pd2.input, pd2.weight, pd2.output = tv.zeros([n, c], tv.bfloat16, 0), w2, dout2
+    pd2.indices, pd2.mask, pd2.mask_argsort = table2.indices_bwd, msb2_tv, orderb2_tv
+    leg("stride2_c128_c256_backward_input", pd2, 2.0 * pairs2 * c * 256)
+    pm2 = ConvParams(3, ConvOpType.Forward)
+    pm2.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 64, 128)
+    pm2.input, pm2.weight, pm2.output = x, w2, tv.zeros([n_out2, 256], tv.bfloat16, 0)
+    pm2.indices, pm2.mask, pm2.mask_argsort, pm2.mask_output = table2.indices_fwd, ms2_tv, order2_tv, red2
+    ConvMainUnitTest.implicit_gemm2(pm2)
+    pw2 = ConvParams(3, ConvOpType.BackwardWeight)
+    pw2.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.BackwardWeight, 64, 64, parallel=True)
+    pw2.input, pw2.weight, pw2.output = x, tv.zeros([256, 27, c], tv.bfloat16, 0), dout2
+    pw2.indices, pw2.mask, pw2.mask_argsort = table2.indices_fwd, red2, order2_tv
+    pw2.mask_width, pw2.split_k_slices = 64, 32
+    wms, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw2), steps, warm)
+    res["stride2_c128_c256_backward_weight_balanced"] = {
+        "ms_per_step": round(wms, 5), "tflops": round(2.0 * pairs2 * c * 256 / (wms * 1e-3) / 1e12, 2)}
+
+    # ---- the whole stack: 4 SubM C = 128 layers (bias + ReLU) + the stride-2 128 -> 256 layer,
+    # forward then full backward (input and weight gradients of every layer), every launch through
+    # the operator; activations chained layer to layer, gradients likewise
+    acts = [x] + [tv.zeros([n, c], tv.bfloat16, 0) for _ in range(4)]
+    grads = [tv.zeros([n, c], tv.bfloat16, 0) for _ in range(5)]
+    fwd, bwd_in, bwd_w = [], [], []
+    for i in range(4):
+        q = ConvParams(3, ConvOpType.Forward)
+        q.conv_algo_desp = pf.conv_algo_desp
+        q.input, q.weight, q.bias, q.output = acts[i], w, b, acts[i + 1]
+        q.indices, q.mask, q.mask_argsort = table.indices_fwd, ms_tv, order_tv
+        q.beta, q.act_type = 1.0, Activation.ReLU
+        fwd.append(q)
+        g = ConvParams(3, ConvOpType.BackwardInput)
+        g.conv_algo_desp = pd.conv_algo_desp
+        g.input, g.weight, g.output = grads[i], w, grads[i + 1]
+        g.indices, g.mask, g.mask_argsort = table.indices_bwd, ms_tv, order_tv
+        g.reverse_mask = True
+        bwd_in.append(g)
+        u = ConvParams(3, ConvOpType.BackwardWeight)
+        u.conv_algo_desp = pw.conv_algo_desp
+        u.input, u.weight, u.output = acts[i], tv.zeros([c, 27, c], tv.bfloat16, 0), grads[i + 1]
+        u.indices, u.mask, u.mask_argsort = table.indices_fwd, red, order_tv
+        u.mask_width, u.split_k_slices, u.workspace = 64, 32, pw.workspace
+        bwd_w.append(u)
+    q5 = ConvParams(3, ConvOpType.Forward)
+    q5.conv_algo_desp = p2.conv_algo_desp
+    q5.input, q5.weight, q5.bias, q5.output = acts[4], w2, b2, p2.output
+    q5.indices, q5.mask, q5.mask_argsort = table2.indices_fwd, ms2_tv, order2_tv
+    q5.beta, q5.act_type = 1.0, Activation.ReLU
+    g5 = ConvParams(3, ConvOpType.BackwardInput)
+    g5.conv_algo_desp = pd2.conv_algo_desp
+    g5.input, g5.weight, g5.output = grads[4], w2, dout2
+    g5.indices, g5.mask, g5.mask_argsort = table2.indices_bwd, msb2_tv, orderb2_tv
+    u5 = ConvParams(3, ConvOpType.BackwardWeight)
+    u5.conv_algo_desp = pw2.conv_algo_desp
+    u5.input, u5.weight, u5.output = acts[4], pw2.weight, dout2
+    u5.indices, u5.mask, u5.mask_argsort = table2.indices_fwd, red2, order2_tv
+    u5.mask_width, u5.split_k_slices, u5.workspace = 64, 32, pw2.workspace
+
+    def stack_forward():
+        for q in fwd:
+            ConvMainUnitTest.implicit_gemm2(q)
+        ConvMainUnitTest.implicit_gemm2(q5)
+
+    def stack_backward():
+        ConvMainUnitTest.implicit_gemm2(u5)
+        ConvMainUnitTest.implicit_gemm2(g5)
+        for i in (3, 2, 1, 0):
+            ConvMainUnitTest.implicit_gemm2(bwd_w[i])
+            ConvMainUnitTest.implicit_gemm2(bwd_in[i])
+
+    def stack_both():
+        stack_forward()
+        stack_backward()
+
+    wf, ef = timed(stack_forward, steps, warm)
+    wb, eb = timed(stack_backward, steps, warm)
+    wa, ea = timed(stack_both, steps, warm)
+    flops_f = 4 * 2.0 * pairs1 * c * c + 2.0 * pairs2 * c * 256
+    res["stack_4_subm_plus_stride2"] = {
+        "launches_forward": 5, "launches_backward": 10,
+        "forward_ms": {"wall": round(wf, 4), "events": round(ef, 4)},
+        "backward_ms": {"wall": round(wb, 4), "events": round(eb, 4)},
+        "forward_backward_ms": {"wall": round(wa, 4), "events": round(ea, 4)},
+        "tflops_forward_backward": round(3.0 * flops_f / (wa * 1e-3) / 1e12, 2)}
     return res
 
 

@@ -53,7 +53,8 @@ class SparseConvArgs(C.Structure):
                 ("mask_filter", C.c_uint32), ("reverse_mask", C.c_int32),
                 ("mask_width", C.c_int32),
                 ("ndim", C.c_int32), ("N", C.c_int32), ("C", C.c_int32), ("K", C.c_int32),
-                ("kernel_volume", C.c_int32), ("d_is_bias", C.c_int32),
+                ("kernel_volume", C.c_int32), ("mode", C.c_int32), ("groups", C.c_int32),
+                ("d_is_bias", C.c_int32),
                 ("bias_pointer", C.c_void_p), ("scale_pointer", C.c_void_p),
                 ("rows_in", C.c_int32), ("rows_out", C.c_int32)]
 
@@ -64,6 +65,8 @@ SYMBOLS = {
     "cumm_hip_gemm": (C.c_int, [C.POINTER(GemmDesc), C.POINTER(GemmArgs), _VP]),
     "cumm_hip_sparse_conv": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(SparseConvArgs), _VP]),
     "cumm_hip_sparse_conv_static_ws": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(SparseConvArgs), _VP]),
+    "cumm_hip_query_gemm_workspace": (C.c_int64, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.c_int]),
+    "cumm_hip_query_conv_workspace": (C.c_int64, [C.POINTER(ConvDesc), C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "cumm_hip_list_gemm_algos": (C.c_int, [C.POINTER(GemmDesc), C.c_int]),
     "cumm_hip_list_conv_algos": (C.c_int, [C.POINTER(ConvDesc), C.c_int]),
     "cumm_hip_gemm_supported": (C.c_int, [C.POINTER(GemmDesc)]),
@@ -100,6 +103,13 @@ SYMBOLS = {
                                   [C.POINTER(C.c_int32), C.POINTER(C.c_int32), _VP, C.c_size_t, _VP]),
     "cumm_hip_conv_pairs_fill": (C.c_int, [_VP, C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5 +
                                  [C.c_int, _VP, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_pair_lists_workspace": (C.c_size_t, [C.c_int, C.c_int]),
+    "cumm_hip_pair_lists": (C.c_int, [_VP, C.c_int, C.c_int, _VP, _VP, _VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_finish_rows": (C.c_int, [_VP, C.c_int, _VP, _VP, C.c_int64, C.c_int, C.c_float, C.c_float, C.c_int,
+                                       C.c_float, _VP]),
+    "cumm_hip_relu_backward": (C.c_int, [_VP, _VP, _VP, C.c_size_t, C.c_int, _VP]),
+    "cumm_hip_column_sum_workspace": (C.c_size_t, [C.c_int64, C.c_int]),
+    "cumm_hip_column_sum": (C.c_int, [_VP, _VP, C.c_int64, C.c_int, C.c_int, _VP, C.c_size_t, _VP]),
     "cumm_hip_gather_rows": (C.c_int, [_VP, _VP, _VP, C.c_int, C.c_int, C.c_size_t, _VP]),
     "cumm_hip_scatter_add_rows": (C.c_int, [_VP, _VP, _VP, C.c_int, C.c_int, C.c_int, C.c_int, _VP]),
 }

@@ -30,7 +30,9 @@ ELEMS = [("F16", "f16"), ("BF16", "bf16"), ("S8", "s8")]
 def _units():
     units = [("api", os.path.join(CSRC, "api.hip"), []),
              ("pairs", os.path.join(CSRC, "pairs_inst.hip"), []),
-             ("gather", os.path.join(CSRC, "gather_inst.hip"), [])]
+             ("gather", os.path.join(CSRC, "gather_inst.hip"), []),
+             ("elementwise", os.path.join(CSRC, "elementwise_inst.hip"), []),
+             ("sort", os.path.join(CSRC, "sort_inst.hip"), [])]
     for tag, name in ELEMS:
         defs = ["-DCUMM_ELEM=%s" % tag, "-DCUMM_NAME=%s" % name]
         units.append(("rowgemm_" + name, os.path.join(CSRC, "rowgemm_inst.hip"), defs))

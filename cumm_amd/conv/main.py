@@ -215,6 +215,7 @@ class ConvMainUnitTest:
         args.mask_width = mask_width
         args.ndim, args.N, args.C, args.K = desp.ndim, N, C, K
         args.kernel_volume = kernel_volume
+        args.mode, args.groups = 1, 1      # ConvMode.CrossCorrelation, ungrouped: all the reference's mask kernels do
         args.d_is_bias = int(not bias.empty())
         args.bias_pointer = _ptr(bias)
         args.scale_pointer = _ptr(scale)

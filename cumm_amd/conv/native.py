@@ -1,0 +1,151 @@
+"""Per-offset ("native") sparse convolution: one gather-GEMM-scatter per kernel offset.
+
+``SparseConvAlgo.Native`` of the reference (include/tensorview/gemm/core/constants.h:34-38): what
+its callers fall back to when the mask-based kernels do not apply, and the only path for kernel
+volumes above 32, which 32-bit masks cannot describe (the reference's ``dynamic_mask`` loader,
+cumm/gemm/blockmma/mma.py:78-269, is not built here).  The pattern is the reference's own check
+of its kernels, cumm/conv/main_real_spconv.py:309-403:
+
+    forward          out[pair_out[k]]  += inp[pair_in[k]]   @ W[:, k, :].T     (matmul2, ShuffleAC)
+    backward-input   dinp[pair_in[k]]  += dout[pair_out[k]] @ W[:, k, :]       (matmul2, ShuffleAC)
+    backward-weight  dW[:, k, :]        = dout[pair_out[k]].T @ inp[pair_in[k]] (matmul2, ShuffleAB)
+
+Forward and backward-input accumulate all offsets in an fp32 image (the f16 / bf16 -> f32 kernels)
+and round once at the end (``cumm_hip_finish_rows``, with bias and activation): one rounding, as
+the mask-based kernels make, instead of one per offset.
+"""
+import ctypes
+from typing import Optional
+
+import numpy as np
+
+from .. import _capi
+from .. import tensorview as tv
+from ..gemm.main import GemmMainUnitTest
+from ..tensorview.gemm import Activation, GemmParams, ShuffleStrideType
+
+
+def _find(dtype: int, dtype_c: int, shuffle: ShuffleStrideType, tile_m: int, tile_n: int, trans_a: bool,
+          trans_b: bool):
+    for d in _descs():
+        if (d.dtype_a == dtype and d.dtype_c == dtype_c and d.shuffle_type == shuffle and
+                d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and d.trans_a == trans_a and
+                d.trans_b == trans_b and not d.trans_c):
+            return d
+    raise RuntimeError("can't find any suitable algo for your parameters.")
+
+
+_DESCS = None
+
+
+def _descs():
+    global _DESCS
+    if _DESCS is None:
+        _DESCS = GemmMainUnitTest.get_all_algo_desp()
+    return _DESCS
+
+
+def _check(inp, weight, lists, n_rows_out):
+    if inp.ndim != 2 or weight.ndim != 3:
+        raise RuntimeError("error")
+    if inp.dtype != weight.dtype or inp.dtype not in (tv.float16, tv.bfloat16):
+        raise RuntimeError("the native path takes f16 or bf16 features and weights of one type")
+    kv = weight.dim(1)
+    if lists.pair_in.dim(0) != kv or lists.pair_out.dim(0) != kv or len(lists.counts) != kv:
+        raise RuntimeError("pair lists and weight disagree on the kernel volume")
+    if inp.dim(1) % 8 or weight.dim(0) % 8 or weight.dim(2) % 8:
+        raise RuntimeError("channel counts must be multiples of 8")
+    return kv
+
+
+def _accumulate(a, a_inds_all, c_inds_all, counts, weight, acc, trans_b, stream):
+    """acc[c_inds[k]] += a[a_inds[k]] @ op(W[:, k, :]) for every offset with pairs."""
+    kv = weight.dim(1)
+    n_ch = acc.dim(1)
+    for k in range(kv):
+        cnt = int(counts[k])
+        if cnt == 0:
+            continue
+        p = GemmParams()
+        tile_m = 128 if cnt >= 16384 else 64
+        tile_n = 128 if n_ch >= 128 else 64
+        p.algo_desp = _find(a.dtype, tv.float32, ShuffleStrideType.ShuffleAC, tile_m, tile_n, False, trans_b).copy()
+        p.a, p.b, p.c = a, weight.select(1, k), acc
+        p.a_inds = a_inds_all.select(0, k).slice_first_axis(0, cnt)
+        p.c_inds = c_inds_all.select(0, k).slice_first_axis(0, cnt)
+        p.alpha, p.beta = 1.0, 1.0
+        p.stream = stream
+        GemmMainUnitTest.matmul2(p)
+
+
+def _finish(out, acc, bias, act_type, act_alpha, stream):
+    _capi.check(_capi.lib().cumm_hip_finish_rows(
+        out.byte_pointer(), out.dtype, acc.byte_pointer(), None if bias is None or bias.empty() else bias.byte_pointer(),
+        out.dim(0), out.dim(1), 1.0, 1.0, act_type.value if hasattr(act_type, "value") else int(act_type),
+        float(act_alpha), stream))
+
+
+def _fp32_image(rows, channels, acc, stream):
+    if acc is None or acc.empty():
+        acc = tv.empty([rows, channels], tv.float32, 0)
+    elif acc.dtype != tv.float32 or acc.shape != [rows, channels] or acc.device < 0:
+        raise RuntimeError("acc must be a device float32 tensor [%d, %d]" % (rows, channels))
+    ctx = tv.Context()
+    ctx.set_cuda_stream(stream)
+    acc.zero_(ctx)
+    return acc
+
+
+def forward(inp: tv.Tensor, weight: tv.Tensor, output: tv.Tensor, lists, *, bias: Optional[tv.Tensor] = None,
+            act_type=Activation.None_, act_alpha: float = 0.0, stream: int = 0, acc: Optional[tv.Tensor] = None) -> None:
+    """output [N_out, K] = act(sum over offsets + bias); ``lists`` from ``pairs.pair_lists_device``
+    on the forward table; ``acc``: an fp32 [N_out, K] device tensor to reuse as the image."""
+    _check(inp, weight, lists, output.dim(0))
+    if output.ndim != 2 or output.dim(1) != weight.dim(0) or output.dtype != inp.dtype or weight.dim(2) != inp.dim(1):
+        raise RuntimeError("error")
+    acc = _fp32_image(output.dim(0), output.dim(1), acc, stream)
+    # W[:, k, :] is [K, C]: B stored [n, k]
+    _accumulate(inp, lists.pair_in, lists.pair_out, lists.counts, weight, acc, True, stream)
+    _finish(output, acc, bias, act_type, act_alpha, stream)
+
+
+def backward_input(dout: tv.Tensor, weight: tv.Tensor, dinp: tv.Tensor, lists, *, stream: int = 0,
+                   acc: Optional[tv.Tensor] = None) -> None:
+    """dinp [N_in, C] = sum over offsets of dout[pair_out[k]] @ W[:, k, :] scattered to pair_in[k]."""
+    _check(dout, weight, lists, dinp.dim(0))
+    if dinp.ndim != 2 or dinp.dim(1) != weight.dim(2) or dout.dim(1) != weight.dim(0) or dinp.dtype != dout.dtype:
+        raise RuntimeError("error")
+    acc = _fp32_image(dinp.dim(0), dinp.dim(1), acc, stream)
+    # W[:, k, :] is [K, C] with K the contraction: B stored [k, n]
+    _accumulate(dout, lists.pair_out, lists.pair_in, lists.counts, weight, acc, False, stream)
+    _finish(dinp, acc, None, Activation.None_, 0.0, stream)
+
+
+_NO_PAIR = {}
+
+
+def backward_weight(dout: tv.Tensor, inp: tv.Tensor, dweight: tv.Tensor, lists, *, split_k_slices: int = 1,
+                    stream: int = 0, workspace: Optional[tv.Tensor] = None) -> None:
+    """dweight[:, k, :] = dout[pair_out[k]].T @ inp[pair_in[k]] for every offset (zero without pairs)."""
+    kv = _check(inp, dweight, lists, dout.dim(0))
+    if dout.dim(1) != dweight.dim(0) or dout.dtype != inp.dtype:
+        raise RuntimeError("error")
+    for k in range(kv):
+        cnt = int(lists.counts[k])
+        p = GemmParams()
+        p.algo_desp = _find(inp.dtype, inp.dtype, ShuffleStrideType.ShuffleAB, 64, 64, True, False).copy()
+        p.a, p.b, p.c = dout, inp, dweight.select(1, k)
+        if cnt > 0:
+            p.a_inds = lists.pair_out.select(0, k).slice_first_axis(0, cnt)
+            p.b_inds = lists.pair_in.select(0, k).slice_first_axis(0, cnt)
+        else:
+            # an offset without pairs: one step of absent rows (index -1) writes the zeros
+            dev = inp.device
+            if dev not in _NO_PAIR:
+                _NO_PAIR[dev] = tv.from_numpy(np.full(32, -1, np.int32)).cuda()
+            p.a_inds = p.b_inds = _NO_PAIR[dev]
+        p.split_k_slices = split_k_slices if cnt >= 4096 * split_k_slices else 1
+        if workspace is not None:
+            p.workspace = workspace
+        p.stream = stream
+        GemmMainUnitTest.matmul2(p)

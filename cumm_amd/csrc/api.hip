@@ -216,8 +216,9 @@ int static_scratch(void **out) {
 }
 
 // ---- failures that a kernel can only report after the fact.  Word 0 counts the serial split-K
-// slices whose bounded semaphore wait ran out (tilegemm.h); the synchronising entry points read
-// and clear it and turn a non-zero count into an error.  One array per GPU, like `scratch`.
+// slices whose bounded semaphore wait ran out (tilegemm.h), word 1 the look-backs of the mask sort
+// that ran into their bound (sort_inst.hip); the synchronising entry points read and clear them and
+// turn a non-zero count into an error.  One array per GPU, like `scratch`.
 static __device__ int32_t async_status[4];
 int32_t *g_status_ptr[kMaxDevices] = {};
 
@@ -238,8 +239,9 @@ int async_status_ptr(int32_t **out) {
 
 // After a synchronisation: anything to report on this device?  (Nothing was ever launched that
 // could report: no device access at all.)
-int take_async_errors(int32_t *timeouts) {
+int take_async_errors(int32_t *timeouts, int32_t *sort_give_ups = nullptr) {
   *timeouts = 0;
+  if (sort_give_ups) *sort_give_ups = 0;
   int dev = -1;
   HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return CUMM_HIP_OK;
@@ -251,17 +253,21 @@ int take_async_errors(int32_t *timeouts) {
   if (ptr == nullptr) return CUMM_HIP_OK;
   int32_t words[4] = {0, 0, 0, 0};
   HIP_TRY(hipMemcpy(words, ptr, sizeof(words), hipMemcpyDeviceToHost));
-  if (words[0] != 0) {
+  if (words[0] != 0 || words[1] != 0) {
     const int32_t zero[4] = {0, 0, 0, 0};
     HIP_TRY(hipMemcpy(ptr, zero, sizeof(zero), hipMemcpyHostToDevice));
   }
   *timeouts = words[0];
+  if (sort_give_ups) *sort_give_ups = words[1];
   return CUMM_HIP_OK;
 }
 
 int report_async_errors() {
-  int32_t timeouts = 0;
-  if (int rc = take_async_errors(&timeouts)) return rc;
+  int32_t timeouts = 0, sort_give_ups = 0;
+  if (int rc = take_async_errors(&timeouts, &sort_give_ups)) return rc;
+  if (sort_give_ups != 0)
+    return fail(CUMM_HIP_ERUNTIME, "mask sort: %d look-back(s) gave up waiting for an earlier chunk; the result of that "
+                "sort is invalid", (int)sort_give_ups);
   if (timeouts != 0)
     return fail(CUMM_HIP_ERUNTIME,
                 "serial split-K: %d slice(s) gave up waiting for their turn at the semaphore; the results of "
@@ -280,6 +286,34 @@ const char *cumm_hip_last_error(void) { return g_err.c_str(); }
 
 int cumm_hip_gemm_supported(const CummHipGemmDesc *desc) { return desc && gemm_family(*desc) != 0; }
 int cumm_hip_conv_supported(const CummHipConvDesc *desc) { return desc && conv_family(*desc) != 0; }
+
+int64_t cumm_hip_query_gemm_workspace(const CummHipGemmDesc *desc, int m, int n, int k, int split_k_slices) {
+  (void)k;
+  if (!desc || m < 0 || n < 0 || split_k_slices < 1) return -1;
+  if (split_k_slices == 1) return 0;
+  const int64_t tiles_m = (m + desc->tile_shape[0] - 1) / desc->tile_shape[0];
+  const int64_t tiles_n = (n + desc->tile_shape[1] - 1) / desc->tile_shape[1];
+  if (desc->split_k_serial) return (int64_t)sizeof(int32_t) * tiles_m * tiles_n;
+  if (desc->split_k_parallel) return (int64_t)4 * m * n * split_k_slices;   // (accumulators are 4 bytes: f32 or s32)
+  return -1;
+}
+
+int64_t cumm_hip_query_conv_workspace(const CummHipConvDesc *desc, int m, int n, int k, int split_k_slices,
+                                      int kernel_volume) {
+  if (!desc || kernel_volume < 1) return -1;
+  if (!desc->mask_sparse) return cumm_hip_query_gemm_workspace(&desc->gemm, m, n, k, split_k_slices);
+  if (m < 0 || n < 0 || split_k_slices < 1) return -1;
+  if (split_k_slices == 1) return 0;
+  const CummHipGemmDesc &d = desc->gemm;
+  const int64_t tiles_m = (m + d.tile_shape[0] - 1) / d.tile_shape[0];
+  // backward weight: every kernel offset has its own column blocks (get_spconv_logical_tile_count, utils.h:39-60)
+  const int64_t tiles_n = desc->op_type == CUMM_HIP_OP_BACKWARD_WEIGHT
+                              ? (int64_t)((n / kernel_volume + d.tile_shape[1] - 1) / d.tile_shape[1]) * kernel_volume
+                              : (n + d.tile_shape[1] - 1) / d.tile_shape[1];
+  if (d.split_k_serial) return (int64_t)sizeof(int32_t) * tiles_m * tiles_n;
+  if (d.split_k_parallel) return (int64_t)4 * m * n * split_k_slices;
+  return -1;
+}
 
 int cumm_hip_list_gemm_algos(CummHipGemmDesc *out, int cap) {
   std::vector<CummHipGemmDesc> v;
@@ -525,6 +559,9 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     return fail(CUMM_HIP_EINVAL, "no sigmoid in integer arithmetic (s32 output)");
   const int kv = a->kernel_volume;
   if (a->N < 0 || a->C <= 0 || a->K <= 0 || kv <= 0) return fail(CUMM_HIP_EINVAL, "bad N, C, K or kernel volume");
+  if (a->mode != CUMM_HIP_CONV_CROSS_CORRELATION)
+    return fail(CUMM_HIP_EINVAL, "mode must be cross-correlation (1): the mask-based kernels implement nothing else");
+  if (a->groups != 1) return fail(CUMM_HIP_EINVAL, "grouped convolution has no kernel (groups must be 1)");
   if (kv > 32) return fail(CUMM_HIP_EINVAL, "kernel volume > 32 needs dynamic_mask, which this build has no kernel for");
   if (!a->ptr_A || !a->ptr_B || !a->ptr_C) return fail(CUMM_HIP_ERUNTIME, "input, weight and output must not be empty");
   if (!a->indice_ptr || !a->mask_ptr || !a->mask_argsort_ptr)
@@ -814,10 +851,13 @@ int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_sha
   if (n < 0 || !spatial_shape || !ksize || !dilation) return fail(CUMM_HIP_EINVAL, "bad arguments");
   if (n == 0) return CUMM_HIP_OK;
   if (n > (1 << 30)) return fail(CUMM_HIP_EINVAL, "too many voxels");
-  if (!coords || !indices_fwd || !mask_fwd) return fail(CUMM_HIP_EINVAL, "coords, indices_fwd and mask_fwd must not be empty");
+  if (!coords || !indices_fwd) return fail(CUMM_HIP_EINVAL, "coords and indices_fwd must not be empty");
   if (!aligned16(coords) || !aligned16(workspace)) return fail(CUMM_HIP_EINVAL, "coords and workspace must be 16-byte aligned");
   const int64_t kv = (int64_t)ksize[0] * ksize[1] * ksize[2];
-  if (ksize[0] < 1 || ksize[1] < 1 || ksize[2] < 1 || kv > 32) return fail(CUMM_HIP_EINVAL, "kernel volume must be 1..32");
+  if (ksize[0] < 1 || ksize[1] < 1 || ksize[2] < 1 || kv > kMaxKernelVolume)
+    return fail(CUMM_HIP_EINVAL, "kernel volume must be 1..%d", kMaxKernelVolume);
+  if (kv > 32 && (mask_fwd || mask_bwd))
+    return fail(CUMM_HIP_EINVAL, "kernel volumes above 32 have no 32-bit masks: pass NULL for mask_fwd and mask_bwd");
   // indices_bwd[k] = indices_fwd[kv-1-k] and the bit-reversed masks hold only when offset kv-1-k is
   // the negative of offset k, i.e. for odd kernel sizes
   if (!(ksize[0] & 1) || !(ksize[1] & 1) || !(ksize[2] & 1))
@@ -851,23 +891,22 @@ int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_sha
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-size_t cumm_hip_sort_by_mask_workspace(int n) {
-  const size_t words = align256(sizeof(uint32_t) * (size_t)(n > 0 ? n : 1));
-  return 2 * words + align256(sort_by_mask_temp_bytes(n));
-}
+size_t cumm_hip_sort_by_mask_workspace(int n) { return sort_by_mask_workspace_bytes(n); }
 
 int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
                           int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream) {
   if (n < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
   if (n == 0) return CUMM_HIP_OK;
+  if (n >= (1 << 30)) return fail(CUMM_HIP_EINVAL, "too many positions");
   if (!mask || !sorted_mask || !argsort) return fail(CUMM_HIP_EINVAL, "mask, sorted_mask and argsort must not be empty");
+  if (mask == sorted_mask) return fail(CUMM_HIP_EINVAL, "the sort is not in place: mask and sorted_mask must differ");
   if (!workspace || workspace_bytes < cumm_hip_sort_by_mask_workspace(n))
     return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", cumm_hip_sort_by_mask_workspace(n));
   if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(CUMM_HIP_EINVAL, "workspace must be 256-byte aligned");
-  const size_t words = align256(sizeof(uint32_t) * (size_t)n);
-  char *base = reinterpret_cast<char *>(workspace);
-  hipError_t e = launch_sort_by_mask(mask, n, mask_filter, sorted_mask, argsort, base, base + words, base + 2 * words,
-                                     workspace_bytes - 2 * words, reinterpret_cast<hipStream_t>(stream));
+  int32_t *status = nullptr;
+  if (int rc = async_status_ptr(&status)) return rc;
+  hipError_t e = launch_sort_by_mask(mask, n, mask_filter, sorted_mask, argsort, workspace, status + 1,
+                                     reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "mask sort launch");
   return CUMM_HIP_OK;
 }
@@ -889,7 +928,7 @@ const char *conv_pairs_check(int batch_size, const int32_t *spatial_shape, const
   if (!spatial_shape || !ksize || !stride || !padding || !dilation) return "geometry arrays must not be empty";
   if (batch_size < 1) return "batch_size must be positive";
   const int64_t kv = (int64_t)ksize[0] * ksize[1] * ksize[2];
-  if (ksize[0] < 1 || ksize[1] < 1 || ksize[2] < 1 || kv > 32) return "kernel volume must be 1..32";
+  if (ksize[0] < 1 || ksize[1] < 1 || ksize[2] < 1 || kv > kMaxKernelVolume) return "kernel volume must be 1..128";
   unsigned long long total = (unsigned long long)batch_size;
   for (int d = 0; d < 3; ++d) {
     if (spatial_shape[d] < 1 || dilation[d] < 1 || stride[d] < 1 || padding[d] < 0)
@@ -1029,8 +1068,10 @@ int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, co
   if (!conv_pairs_layout(n_in, sites, ksize, stride, dilation, &l)) return fail(CUMM_HIP_EINVAL, "too many voxels");
   if (!l.bitmap && (size_t)n_out > l.bound) return fail(CUMM_HIP_EINVAL, "n_out is not what cumm_hip_conv_pairs_sites returned");
   if (!coords || !aligned16(coords)) return fail(CUMM_HIP_EINVAL, "coords must be 16-byte aligned and not empty");
-  if (n_out > 0 && (!out_coords || !indices_fwd || !mask_fwd || !aligned16(out_coords) || !aligned16(indices_fwd)))
-    return fail(CUMM_HIP_EINVAL, "out_coords, indices_fwd (both 16-byte aligned) and mask_fwd must not be empty");
+  if (n_out > 0 && (!out_coords || !indices_fwd || !aligned16(out_coords) || !aligned16(indices_fwd)))
+    return fail(CUMM_HIP_EINVAL, "out_coords and indices_fwd (both 16-byte aligned) must not be empty");
+  if ((int64_t)ksize[0] * ksize[1] * ksize[2] > 32 && (mask_fwd || mask_bwd))
+    return fail(CUMM_HIP_EINVAL, "kernel volumes above 32 have no 32-bit masks: pass NULL for mask_fwd and mask_bwd");
   if (!workspace || workspace_bytes < l.total) return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", l.total);
   if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(CUMM_HIP_EINVAL, "workspace must be 256-byte aligned");
   ConvPairsParams p;
@@ -1039,6 +1080,32 @@ int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, co
   p.out_coords = out_coords; p.ind_f = indices_fwd; p.ind_b = indices_bwd; p.mask_f = mask_fwd; p.mask_b = mask_bwd;
   hipError_t e = launch_conv_pairs_fill(p, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "pair table launch");
+  return CUMM_HIP_OK;
+}
+
+// ---- per-offset pair lists for the native (per-offset) convolution
+size_t cumm_hip_pair_lists_workspace(int kv, int n) {
+  if (kv <= 0 || n <= 0) return 0;
+  const size_t chunks = ((size_t)n + kPairListChunk - 1) / kPairListChunk;
+  return sizeof(int32_t) * (size_t)kv * chunks;
+}
+
+int cumm_hip_pair_lists(const int32_t *indices, int kv, int n, int32_t *pair_in, int32_t *pair_out, int32_t *counts,
+                        void *workspace, size_t workspace_bytes, void *stream) {
+  if (kv < 0 || n < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (kv == 0) return CUMM_HIP_OK;
+  if (!counts) return fail(CUMM_HIP_EINVAL, "counts must not be empty");
+  if (n > 0 && (!indices || !pair_in || !pair_out)) return fail(CUMM_HIP_EINVAL, "indices, pair_in and pair_out must not be empty");
+  const size_t need = cumm_hip_pair_lists_workspace(kv, n);
+  if (need > 0 && (!workspace || workspace_bytes < need)) return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
+  if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
+  PairListsParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.indices = indices; p.pair_in = pair_in; p.pair_out = pair_out; p.counts = counts;
+  p.chunk_counts = reinterpret_cast<int32_t *>(workspace);
+  p.kv = kv; p.n = n; p.chunks = (n + kPairListChunk - 1) / kPairListChunk;
+  hipError_t e = launch_pair_lists(p, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "pair list launch");
   return CUMM_HIP_OK;
 }
 
@@ -1092,6 +1159,58 @@ int cumm_hip_scatter_add_rows(void *output, const void *input, const int32_t *in
   if (!row_move_params(&p, output, input, indices, m, rows_out, row_bytes, &wide)) return fail(CUMM_HIP_EINVAL, "rows too long");
   hipError_t e = launch_scatter_add_rows(p, dtype, wide, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "scatter launch");
+  return CUMM_HIP_OK;
+}
+
+// ---- row-wise helpers
+int cumm_hip_finish_rows(void *out, int dtype, const float *acc, const void *bias, int64_t rows, int channels,
+                         float alpha, float beta, int act_type, float act_alpha, void *stream) {
+  if (rows < 0 || channels < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (!is_float16_like(dtype)) return fail(CUMM_HIP_EINVAL, "the output must be f16 or bf16");
+  if (channels % 8) return fail(CUMM_HIP_EINVAL, "channels must be a multiple of 8");
+  if (rows == 0 || channels == 0) return CUMM_HIP_OK;
+  if (!out || !acc || !aligned16(out) || !aligned16(acc) || (bias && !aligned16(bias)))
+    return fail(CUMM_HIP_EINVAL, "out, acc (and bias) must be 16-byte aligned and not empty");
+  FinishRowsParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.out = out; p.acc = acc; p.bias = bias; p.rows = rows; p.channels = channels;
+  p.alpha = alpha; p.beta = beta; p.act = act_type; p.act_alpha = act_alpha;
+  hipError_t e = launch_finish_rows(p, dtype == CUMM_HIP_BF16, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "finish_rows launch");
+  return CUMM_HIP_OK;
+}
+
+int cumm_hip_relu_backward(void *dst, const void *grad, const void *out, size_t elems, int dtype, void *stream) {
+  if (!is_float16_like(dtype)) return fail(CUMM_HIP_EINVAL, "dtype must be f16 or bf16");
+  if (elems % 8) return fail(CUMM_HIP_EINVAL, "the element count must be a multiple of 8");
+  if (elems == 0) return CUMM_HIP_OK;
+  if (!dst || !grad || !out || !aligned16(dst) || !aligned16(grad) || !aligned16(out))
+    return fail(CUMM_HIP_EINVAL, "dst, grad and out must be 16-byte aligned and not empty");
+  hipError_t e = launch_relu_backward(dst, grad, out, elems / 8, dtype == CUMM_HIP_BF16, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "relu_backward launch");
+  return CUMM_HIP_OK;
+}
+
+size_t cumm_hip_column_sum_workspace(int64_t rows, int channels) {
+  if (rows <= 0 || channels <= 0) return 0;
+  return sizeof(float) * (size_t)column_sum_blocks(rows, channels) * (size_t)channels;
+}
+
+int cumm_hip_column_sum(void *dst, const void *src, int64_t rows, int channels, int dtype, void *workspace,
+                        size_t workspace_bytes, void *stream) {
+  if (rows < 0 || channels < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (!is_float16_like(dtype)) return fail(CUMM_HIP_EINVAL, "dtype must be f16 or bf16");
+  if (channels % 8 || channels > 2048) return fail(CUMM_HIP_EINVAL, "channels must be a multiple of 8, at most 2048");
+  if (channels == 0) return CUMM_HIP_OK;
+  if (!dst || (!src && rows > 0) || !aligned16(src)) return fail(CUMM_HIP_EINVAL, "dst and src (16-byte aligned) must not be empty");
+  const size_t need = sizeof(float) * (size_t)column_sum_blocks(rows, channels) * (size_t)channels;
+  if (!workspace || workspace_bytes < need) return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", need);
+  if (reinterpret_cast<uintptr_t>(workspace) & 3u) return fail(CUMM_HIP_EINVAL, "workspace must be 4-byte aligned");
+  ColumnSumParams p;
+  std::memset(&p, 0, sizeof(p));
+  p.dst = dst; p.src = src; p.partial = reinterpret_cast<float *>(workspace); p.rows = rows; p.channels = channels;
+  hipError_t e = launch_column_sum(p, dtype == CUMM_HIP_BF16, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "column_sum launch");
   return CUMM_HIP_OK;
 }
 

@@ -43,14 +43,18 @@ inline bool tilegemm_has_tile(int tm, int tn) {
   return (tm == 64 && tn == 64) || (tm == 128 && tn == 128);
 }
 
+// Largest kernel volume the pair builders take (5 x 5 x 5).  Volumes above 32 have no 32-bit
+// masks: their tables feed the per-offset ("native") convolution, not the mask-based kernels.
+constexpr int kMaxKernelVolume = 128;
+
 // ---- pair tables of a submanifold convolution and the mask sort (pairs_inst.hip)
 struct SubmPairsParams {
   const int32_t *coords;   // [n, 4] (batch, z, y, x)
   int32_t n, kv;
   int32_t shape[3];
-  int32_t off[32][3];      // (k_zyx - center) * dilation per kernel offset
+  int32_t off[kMaxKernelVolume][3];   // (k_zyx - center) * dilation per kernel offset
   int32_t *ind_f, *ind_b;  // [kv, n]; ind_b may be NULL
-  uint32_t *mask_f, *mask_b;
+  uint32_t *mask_f, *mask_b;   // may be NULL (must be for kernel volumes above 32)
   void *table;             // (slot_mask + 1) slots of 16 bytes
   uint32_t slot_mask;
   uint32_t *filter;        // (filter_mask + 1) presence words
@@ -65,7 +69,7 @@ struct ConvPairsParams {
   const int32_t *coords;        // [n_in, 4] (batch, z, y, x)
   int32_t n_in, n_out, kv, batch;
   int32_t out_shape[3], stride[3], pad[3];
-  int32_t koff[32][3];          // k_zyx * dilation per kernel offset
+  int32_t koff[kMaxKernelVolume][3];   // k_zyx * dilation per kernel offset
   void *table;                  // (slot_mask + 1) slots of 16 bytes: {output site key, output row}
   uint32_t slot_mask;
   unsigned long long *uniq;     // output site keys in order of discovery
@@ -76,7 +80,7 @@ struct ConvPairsParams {
   unsigned long long n_words;   // (0 = hash set and sort)
   int32_t *out_coords;          // [n_out, 4]
   int32_t *ind_f, *ind_b;       // [kv, n_out], [kv, n_in] (may be NULL)
-  uint32_t *mask_f, *mask_b;    // [n_out], [n_in] (may be NULL)
+  uint32_t *mask_f, *mask_b;    // [n_out], [n_in] (may be NULL; must be for kernel volumes above 32)
 };
 hipError_t launch_conv_pairs_sites(const ConvPairsParams &p, hipStream_t s);
 size_t conv_pairs_sort_temp_bytes(size_t max_sites);
@@ -85,9 +89,21 @@ hipError_t launch_conv_pairs_sort(const ConvPairsParams &p, unsigned long long m
 hipError_t launch_conv_pairs_fill(const ConvPairsParams &p, hipStream_t s);
 size_t conv_pairs_scan_temp_bytes(size_t n_words);
 hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t temp_bytes, hipStream_t s);
-size_t sort_by_mask_temp_bytes(int n);
+// stable radix sort of mask & filter with its permutation (sort_inst.hip)
+size_t sort_by_mask_workspace_bytes(int n);
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
-                               void *keys_ws, void *iota_ws, void *temp, size_t temp_bytes, hipStream_t s);
+                               void *workspace, int32_t *give_ups, hipStream_t s);
+
+// per-offset lists of (input row, output row) out of a pair table [kv, n] (pairs_inst.hip)
+struct PairListsParams {
+  const int32_t *indices;   // [kv, n]: input row of output o at offset k, -1 = none
+  int32_t *pair_in, *pair_out;   // [kv, n] each: the pairs of offset k, ascending output row, packed to the front
+  int32_t *counts;          // [kv]
+  int32_t *chunk_counts;    // [kv, chunks] scratch
+  int32_t kv, n, chunks;
+};
+constexpr int kPairListChunk = 2048;   // table entries per workgroup
+hipError_t launch_pair_lists(const PairListsParams &p, hipStream_t s);
 
 // ---- stand-alone row gather / scatter-add (gather_inst.hip)
 struct RowMoveParams {
@@ -101,5 +117,27 @@ struct RowMoveParams {
 };
 hipError_t launch_gather_rows(const RowMoveParams &p, bool wide, hipStream_t s);
 hipError_t launch_scatter_add_rows(const RowMoveParams &p, int dtype, bool wide, hipStream_t s);
+
+// ---- row-wise helpers (elementwise_inst.hip)
+struct FinishRowsParams {
+  void *out;            // [rows, channels] f16 / bf16
+  const float *acc;     // [rows, channels] fp32
+  const void *bias;     // [channels] in the output's type, or NULL
+  int64_t rows;
+  int32_t channels;     // a multiple of 8
+  float alpha, beta, act_alpha;
+  int32_t act;
+};
+hipError_t launch_finish_rows(const FinishRowsParams &p, bool bf16, hipStream_t s);
+hipError_t launch_relu_backward(void *dst, const void *grad, const void *out, size_t vecs, bool bf16, hipStream_t s);
+struct ColumnSumParams {
+  void *dst;            // [channels]
+  const void *src;      // [rows, channels]
+  float *partial;       // [blocks, channels] fp32
+  int64_t rows, rows_per_block;
+  int32_t channels, blocks;
+};
+int column_sum_blocks(int64_t rows, int channels);
+hipError_t launch_column_sum(ColumnSumParams p, bool bf16, hipStream_t s);
 
 }  // namespace cummhip

@@ -1,4 +1,4 @@
-// Pair tables of a submanifold convolution and the mask sort, on the GPU: the step right before
+// Pair tables of a submanifold convolution, on the GPU: the step right before
 // the mask-based kernels (the reference's callers get it from spconv's generate_subm_conv_inds and
 // sort_1d_by_key, cumm/conv/main_real_spconv.py:91-145; the reference's own building block is the
 // linear-probing LinearHashTable of include/tensorview/hash/linear.cu.h:111-840).
@@ -18,7 +18,6 @@
 //   * the lookup kernel is one lane per (voxel, (kz, ky)): for a fixed offset consecutive lanes
 //     write consecutive table entries (coalesced).  Measured at 120 k voxels: one lane per voxel
 //     walking its 27 offsets 127 us, one lane per (voxel, offset) without the bitmap 66 us;
-//   * the mask sort is rocPRIM's radix sort by key (stable, like the host's argsort).
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -57,7 +56,7 @@ __global__ __launch_bounds__(256) void pairs_clear_kernel(const SubmPairsParams 
   if (i < (uint32_t)p.n) {
     // every voxel pairs with itself through the centre offset: that bit is set here, and the
     // look-up kernel neither probes the table nor touches the masks for it
-    p.mask_f[i] = p.center_k >= 0 ? 1u << p.center_k : 0u;
+    if (p.mask_f) p.mask_f[i] = p.center_k >= 0 ? 1u << p.center_k : 0u;
     if (p.mask_b) p.mask_b[i] = p.center_k >= 0 ? 1u << (p.kv - 1 - p.center_k) : 0u;
   }
 }
@@ -134,18 +133,10 @@ __global__ __launch_bounds__(256) void pairs_lookup_kernel(const SubmPairsParams
     p.ind_f[(int64_t)k * p.n + i] = row;
     if (p.ind_b) p.ind_b[(int64_t)(p.kv - 1 - k) * p.n + i] = row;
     if (row >= 0) {
-      atomicOr(&p.mask_f[i], 1u << k);
+      if (p.mask_f) atomicOr(&p.mask_f[i], 1u << k);
       if (p.mask_b) atomicOr(&p.mask_b[i], 1u << (p.kv - 1 - k));
     }
   }
-}
-
-__global__ __launch_bounds__(256) void sort_keys_kernel(const uint32_t *mask, uint32_t filter, uint32_t *keys,
-                                                        int32_t *iota, int n) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= n) return;
-  keys[i] = mask[i] & filter;
-  iota[i] = i;
 }
 
 // ---- regular (strided) sparse convolution: an output site is active iff an input falls into
@@ -284,7 +275,7 @@ __global__ __launch_bounds__(256) void conv_pairs_rows_kernel(const ConvPairsPar
   c.y = (int)(key % (unsigned long long)p.out_shape[0]); key /= (unsigned long long)p.out_shape[0];
   c.x = (int)key;
   reinterpret_cast<int4 *>(p.out_coords)[j] = c;
-  p.mask_f[j] = 0u;
+  if (p.mask_f) p.mask_f[j] = 0u;
 }
 
 template <bool BITS>
@@ -312,7 +303,7 @@ __global__ __launch_bounds__(256) void conv_pairs_fill_kernel(const ConvPairsPar
   if (p.ind_b) p.ind_b[(int64_t)k * p.n_in + i] = row;
   if (row >= 0 && row < p.n_out) {
     p.ind_f[(int64_t)k * p.n_out + row] = i;
-    atomicOr(&p.mask_f[row], 1u << k);
+    if (p.mask_f) atomicOr(&p.mask_f[row], 1u << k);
     if (p.mask_b) atomicOr(&p.mask_b[i], 1u << k);
   }
 }
@@ -358,7 +349,8 @@ __global__ __launch_bounds__(256) void conv_bits_rows_kernel(const ConvPairsPara
   }
   if (p.mask_b)
     for (unsigned long long i = j; i < (unsigned long long)p.n_in; i += step) p.mask_b[i] = 0u;
-  for (unsigned long long o = j; o < (unsigned long long)p.n_out; o += step) p.mask_f[o] = 0u;
+  if (p.mask_f)
+    for (unsigned long long o = j; o < (unsigned long long)p.n_out; o += step) p.mask_f[o] = 0u;
   for (unsigned long long w = j; w < p.n_words; w += step) {
     uint32_t word = p.bits[w];
     uint32_t row = p.prefix[w];
@@ -377,7 +369,104 @@ __global__ __launch_bounds__(256) void conv_bits_rows_kernel(const ConvPairsPara
   }
 }
 
+// ---- per-offset pair lists out of a pair table: what the per-offset ("native") convolution walks
+// (spconv's indice_pairs [2, kv, N] and indice_num_per_loc, which the reference's check script
+// rebuilds from the mask tables, cumm/conv/main_real_spconv.py:300-326).  Three small kernels:
+// pairs per chunk of 2048 entries, an exclusive scan over the chunks of an offset, and the write.
+// Within a chunk a thread takes entries t, t + 256, ...: ranks by ballot keep the output rows in
+// ascending order.
+constexpr int kChunkIters = kPairListChunk / 256;
+
+__global__ __launch_bounds__(256) void pair_lists_count_kernel(const PairListsParams p) {
+  __shared__ int wave_cnt[4];
+  const int k = blockIdx.y, t = threadIdx.x;
+  const int base = blockIdx.x * kPairListChunk;
+  int mine = 0;
+#pragma unroll
+  for (int u = 0; u < kChunkIters; ++u) {
+    const int o = base + u * 256 + t;
+    const bool have = o < p.n && p.indices[(int64_t)k * p.n + o] >= 0;
+    mine += __popcll(__ballot(have));
+  }
+  if ((t & 63) == 0) wave_cnt[t >> 6] = mine;
+  __syncthreads();
+  if (t == 0) p.chunk_counts[(int64_t)k * p.chunks + blockIdx.x] = wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
+}
+
+// one workgroup per offset: chunk counts -> exclusive prefix sums (in place), total -> counts[k]
+__global__ __launch_bounds__(256) void pair_lists_scan_kernel(const PairListsParams p) {
+  __shared__ int lds[256];
+  __shared__ int carry;
+  const int k = blockIdx.x, t = threadIdx.x;
+  int32_t *cc = p.chunk_counts + (int64_t)k * p.chunks;
+  if (t == 0) carry = 0;
+  __syncthreads();
+  for (int c0 = 0; c0 < p.chunks; c0 += 256) {
+    const int c = c0 + t;
+    const int v = c < p.chunks ? cc[c] : 0;
+    lds[t] = v;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+      const int add = t >= off ? lds[t - off] : 0;
+      __syncthreads();
+      lds[t] += add;
+      __syncthreads();
+    }
+    const int base = carry;
+    if (c < p.chunks) cc[c] = base + lds[t] - v;
+    __syncthreads();
+    if (t == 255) carry = base + lds[255];
+    __syncthreads();
+  }
+  if (t == 0) p.counts[k] = carry;
+}
+
+__global__ __launch_bounds__(256) void pair_lists_write_kernel(const PairListsParams p) {
+  __shared__ int wave_cnt[kChunkIters][4];
+  const int k = blockIdx.y, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int base = blockIdx.x * kPairListChunk;
+  int in_row[kChunkIters];
+  unsigned long long bal[kChunkIters];
+#pragma unroll
+  for (int u = 0; u < kChunkIters; ++u) {
+    const int o = base + u * 256 + t;
+    in_row[u] = o < p.n ? p.indices[(int64_t)k * p.n + o] : -1;
+    bal[u] = __ballot(in_row[u] >= 0);
+    if (lane == 0) wave_cnt[u][wave] = __popcll(bal[u]);
+  }
+  __syncthreads();
+  int at = p.chunk_counts[(int64_t)k * p.chunks + blockIdx.x];
+#pragma unroll
+  for (int u = 0; u < kChunkIters; ++u) {
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int c = wave_cnt[u][w];
+      before += w < wave ? c : 0;
+      total += c;
+    }
+    if (in_row[u] >= 0) {
+      const int64_t dst = (int64_t)k * p.n + at + before + __popcll(bal[u] & ((1ull << lane) - 1ull));
+      p.pair_in[dst] = in_row[u];
+      p.pair_out[dst] = base + u * 256 + t;
+    }
+    at += total;
+  }
+}
+
 }  // namespace
+
+hipError_t launch_pair_lists(const PairListsParams &p, hipStream_t s) {
+  if (p.kv <= 0) return hipSuccess;
+  if (p.n <= 0 || p.chunks <= 0) {
+    hipLaunchKernelGGL(pair_lists_scan_kernel, dim3(p.kv), dim3(256), 0, s, p);   // (counts = 0)
+    return hipGetLastError();
+  }
+  hipLaunchKernelGGL(pair_lists_count_kernel, dim3(p.chunks, p.kv), dim3(256), 0, s, p);
+  hipLaunchKernelGGL(pair_lists_scan_kernel, dim3(p.kv), dim3(256), 0, s, p);
+  hipLaunchKernelGGL(pair_lists_write_kernel, dim3(p.chunks, p.kv), dim3(256), 0, s, p);
+  return hipGetLastError();
+}
 
 hipError_t launch_conv_pairs_sites(const ConvPairsParams &p, hipStream_t s) {
   hipLaunchKernelGGL(conv_pairs_clear_kernel, dim3((p.slot_mask + 256u) / 256u), dim3(256), 0, s, p);
@@ -456,27 +545,6 @@ hipError_t launch_subm_pairs(const SubmPairsParams &p, hipStream_t s) {
   hipLaunchKernelGGL(pairs_insert_kernel, dim3((p.n + 255) / 256), dim3(256), 0, s, p);
   hipLaunchKernelGGL(pairs_lookup_kernel, dim3((p.n + 255) / 256, p.kv / p.kx), dim3(256), 0, s, p);
   return hipGetLastError();
-}
-
-size_t sort_by_mask_temp_bytes(int n) {
-  size_t bytes = 0;
-  (void)rocprim::radix_sort_pairs(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr, (const int32_t *)nullptr,
-                            (int32_t *)nullptr, (size_t)(n > 0 ? n : 1), 0, 32);
-  return bytes;
-}
-
-hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
-                               void *keys_ws, void *iota_ws, void *temp, size_t temp_bytes, hipStream_t s) {
-  // only the bits the filter lets through can differ: fewer radix passes
-  int end_bit = 32;
-  while (end_bit > 1 && !((filter >> (end_bit - 1)) & 1u)) --end_bit;
-  if (n <= 0) return hipSuccess;
-  hipLaunchKernelGGL(sort_keys_kernel, dim3((n + 255) / 256), dim3(256), 0, s, mask, filter,
-                     reinterpret_cast<uint32_t *>(keys_ws), reinterpret_cast<int32_t *>(iota_ws), n);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  return rocprim::radix_sort_pairs(temp, temp_bytes, reinterpret_cast<const uint32_t *>(keys_ws), sorted,
-                                   reinterpret_cast<const int32_t *>(iota_ws), argsort, (size_t)n, 0, end_bit, s);
 }
 
 }  // namespace cummhip

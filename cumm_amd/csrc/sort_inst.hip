@@ -1,0 +1,240 @@
+// Stable ascending sort of (mask & filter) with the permutation that does it: the step between
+// the pair tables and the mask-based kernels (the reference's callers take it from spconv's
+// sort_1d_by_key[_split], cumm/conv/main_real_spconv.py:118-145).
+//
+// Least-significant-digit radix sort, 9 bits per pass (three passes for the 27 offsets of a
+// 3 x 3 x 3 kernel), one kernel per pass plus one kernel in front:
+//   * sort_setup_kernel reads the keys once and makes the histograms of ALL passes (the digits of
+//     a key do not depend on the order the keys are in), clears the look-back state and the block
+//     tickets;
+//   * a pass kernel is a single sweep: a workgroup takes the next chunk of 4096 keys (by ticket,
+//     so that a chunk's predecessors have always started), ranks its keys per digit - per wave
+//     by ballot matching, in position order, which is what makes the pass stable -, publishes its
+//     per-digit counts, finds the counts of all chunks before it by looking back over what they
+//     have published (a chunk publishes its own counts at once and the running total when it
+//     knows it; a look-back stops at the first running total), and scatters.
+// Every spin on another workgroup's state is bounded: a wave that gives up counts itself and goes
+// on (the result is then wrong, and the host says so at its next synchronisation), so the grid
+// always drains.
+// Integer work, bound by launch latency at 10^5 keys and by HBM / L2 traffic at 10^6 and more.
+#include "launch.h"
+
+namespace cummhip {
+
+namespace {
+
+constexpr int kRadixBits = 9;
+constexpr int kBins = 1 << kRadixBits;            // 512
+constexpr int kSortThreads = 512;                 // one bin per thread
+constexpr int kSortWaves = kSortThreads / 64;     // 8
+constexpr int kItems = 8;                         // keys per lane
+constexpr int kChunk = kSortThreads * kItems;     // 4096 keys per workgroup
+constexpr uint32_t kFlagAggregate = 1u << 30, kFlagInclusive = 2u << 30, kValueMask = (1u << 30) - 1u;
+constexpr int kLookbackSpins = 1 << 22;
+
+struct SortParams {
+  const uint32_t *mask;      // [n] the caller's masks
+  uint32_t filter;
+  int32_t n, chunks, passes;
+  uint32_t *hist;            // [passes][kBins] keys per digit value
+  uint32_t *state;           // [passes][chunks][kBins] look-back words
+  uint32_t *tickets;         // [passes] next chunk to hand out
+  int32_t *give_ups;         // counts the look-backs that ran into their bound (the host reports them)
+  // pass p reads keys/vals from src and writes dst (pass 0 reads the masks and an implicit iota)
+  const uint32_t *src_keys;
+  const int32_t *src_vals;
+  uint32_t *dst_keys;
+  int32_t *dst_vals;
+  int32_t pass;
+};
+
+__global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortParams p) {
+  __shared__ uint32_t lds_hist[4][kBins];
+  const int t = threadIdx.x;
+  for (int q = 0; q < p.passes; ++q) lds_hist[q][t] = 0u;
+  // look-back state and tickets start at zero (the workspace holds whatever was there)
+  const size_t words = (size_t)p.passes * p.chunks * kBins;
+  for (size_t i = (size_t)blockIdx.x * kSortThreads + t; i < words; i += (size_t)gridDim.x * kSortThreads) p.state[i] = 0u;
+  if (blockIdx.x == 0 && t < p.passes) p.tickets[t] = 0u;
+  __syncthreads();
+  for (int64_t i = (int64_t)blockIdx.x * kSortThreads + t; i < p.n; i += (int64_t)gridDim.x * kSortThreads) {
+    const uint32_t key = p.mask[i] & p.filter;
+    for (int q = 0; q < p.passes; ++q) atomicAdd(&lds_hist[q][(key >> (q * kRadixBits)) & (kBins - 1)], 1u);
+  }
+  __syncthreads();
+  for (int q = 0; q < p.passes; ++q) {
+    const uint32_t c = lds_hist[q][t];
+    if (c) atomicAdd(&p.hist[q * kBins + t], c);
+  }
+}
+
+// (the histograms are accumulated with atomics: they start from zero in a kernel of their own
+// stream order before the setup kernel - see launch_sort_by_mask)
+__global__ __launch_bounds__(256) void sort_clear_hist_kernel(uint32_t *hist, int words) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < words) hist[i] = 0u;
+}
+
+__global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParams p) {
+  __shared__ uint32_t wave_hist[kSortWaves][kBins];   // per wave: keys per digit, then the prefix over waves
+  __shared__ uint32_t bin_base[kBins];                // where this chunk's keys of a digit go
+  __shared__ uint32_t scan_tmp[kBins];
+  __shared__ int chunk_of_block;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int shift = p.pass * kRadixBits;
+
+  if (t == 0) chunk_of_block = (int)atomicAdd(&p.tickets[p.pass], 1u);
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) wave_hist[w][t] = 0u;
+  // exclusive prefix over the digit values of the whole input: thread = bin, Hillis-Steele
+  const uint32_t total_of_bin = p.hist[p.pass * kBins + t];
+  scan_tmp[t] = total_of_bin;
+  __syncthreads();
+  for (int off = 1; off < kBins; off <<= 1) {
+    const uint32_t add = t >= off ? scan_tmp[t - off] : 0u;
+    __syncthreads();
+    scan_tmp[t] += add;
+    __syncthreads();
+  }
+  const uint32_t global_excl = scan_tmp[t] - total_of_bin;
+  const int chunk = chunk_of_block;
+  if (chunk >= p.chunks) return;   // (never: the grid has one workgroup per chunk)
+
+  // ---- keys of this chunk, wave-striped: wave w owns positions [base_w, base_w + 64 * kItems),
+  // item u of lane l is position base_w + u * 64 + l, i.e. position order = (u, l)
+  const int64_t base_w = (int64_t)chunk * kChunk + (int64_t)wave * (64 * kItems);
+  uint32_t key[kItems];
+  int32_t val[kItems];
+  uint32_t rank[kItems];   // offset among this wave's keys of the same digit
+#pragma unroll
+  for (int u = 0; u < kItems; ++u) {
+    const int64_t pos = base_w + u * 64 + lane;
+    const bool valid = pos < p.n;
+    if (p.pass == 0) {
+      key[u] = valid ? (p.mask[pos] & p.filter) : 0u;
+      val[u] = (int32_t)pos;
+    } else {
+      key[u] = valid ? p.src_keys[pos] : 0u;
+      val[u] = valid ? p.src_vals[pos] : 0;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kItems; ++u) {
+    const int64_t pos = base_w + u * 64 + lane;
+    const bool valid = pos < p.n;
+    const uint32_t d = (key[u] >> shift) & (kBins - 1);
+    // lanes with the same digit (positions past the end match nobody)
+    unsigned long long peers = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < kRadixBits; ++b) {
+      const unsigned long long has = __ballot((d >> b) & 1u);
+      peers &= ((d >> b) & 1u) ? has : ~has;
+    }
+    const uint32_t before = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
+    uint32_t prev = 0;
+    if (valid) prev = wave_hist[wave][d];
+    __builtin_amdgcn_wave_barrier();
+    if (valid && before == 0) wave_hist[wave][d] = prev + (uint32_t)__popcll(peers);
+    __builtin_amdgcn_wave_barrier();
+    rank[u] = prev + before;
+  }
+  __syncthreads();
+
+  // ---- thread = bin: prefix over the waves, this chunk's count, look-back over the chunks before
+  uint32_t count = 0;
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) {
+    const uint32_t c = wave_hist[w][t];
+    wave_hist[w][t] = count;
+    count += c;
+  }
+  uint32_t *my_state = p.state + ((size_t)p.pass * p.chunks + chunk) * kBins;
+  __hip_atomic_store(&my_state[t], (chunk == 0 ? kFlagInclusive : kFlagAggregate) | count, __ATOMIC_RELEASE,
+                     __HIP_MEMORY_SCOPE_AGENT);
+  uint32_t before_chunks = 0;
+  if (chunk > 0) {
+    bool gave_up = false;
+    for (int j = chunk - 1; j >= 0; --j) {
+      const uint32_t *st = p.state + ((size_t)p.pass * p.chunks + j) * kBins + t;
+      uint32_t s = __hip_atomic_load(st, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+      for (int spins = 0; (s >> 30) == 0u && spins < kLookbackSpins; ++spins) {
+        __builtin_amdgcn_s_sleep(2);
+        s = __hip_atomic_load(st, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      if ((s >> 30) == 0u) {
+        gave_up = true;
+        break;
+      }
+      before_chunks += s & kValueMask;
+      if ((s >> 30) == 2u) break;
+    }
+    if (gave_up && p.give_ups != nullptr) atomicAdd(p.give_ups, 1);
+    __hip_atomic_store(&my_state[t], kFlagInclusive | (before_chunks + count), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  bin_base[t] = global_excl + before_chunks;
+  __syncthreads();
+
+  // ---- scatter
+#pragma unroll
+  for (int u = 0; u < kItems; ++u) {
+    const int64_t pos = base_w + u * 64 + lane;
+    if (pos < p.n) {
+      const uint32_t d = (key[u] >> shift) & (kBins - 1);
+      const uint32_t dst = bin_base[d] + wave_hist[wave][d] + rank[u];
+      p.dst_keys[dst] = key[u];
+      p.dst_vals[dst] = val[u];
+    }
+  }
+}
+
+size_t align256s(size_t x) { return (x + 255) & ~(size_t)255; }
+
+int sort_passes(uint32_t filter) {
+  int end_bit = 32;
+  while (end_bit > 1 && !((filter >> (end_bit - 1)) & 1u)) --end_bit;
+  return (end_bit + kRadixBits - 1) / kRadixBits;   // 1 .. 4
+}
+
+}  // namespace
+
+// keys + values of the intermediate order, histograms, tickets, look-back state
+size_t sort_by_mask_workspace_bytes(int n) {
+  const size_t nn = (size_t)(n > 0 ? n : 1);
+  const size_t chunks = (nn + kChunk - 1) / kChunk;
+  return 2 * align256s(4 * nn) + align256s(4 * 4 * kBins) + 256 + align256s(4 * 4 * chunks * kBins);
+}
+
+hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
+                               void *workspace, int32_t *give_ups, hipStream_t s) {
+  if (n <= 0) return hipSuccess;
+  char *base = reinterpret_cast<char *>(workspace);
+  const size_t words = align256s(4 * (size_t)n);
+  SortParams p;
+  p.mask = mask; p.filter = filter; p.n = n;
+  p.chunks = (n + kChunk - 1) / kChunk;
+  p.passes = sort_passes(filter);
+  uint32_t *tmp_keys = reinterpret_cast<uint32_t *>(base);
+  int32_t *tmp_vals = reinterpret_cast<int32_t *>(base + words);
+  p.hist = reinterpret_cast<uint32_t *>(base + 2 * words);
+  p.tickets = reinterpret_cast<uint32_t *>(base + 2 * words + align256s(4 * 4 * kBins));
+  p.state = reinterpret_cast<uint32_t *>(base + 2 * words + align256s(4 * 4 * kBins) + 256);
+  p.give_ups = give_ups;
+  p.src_keys = nullptr; p.src_vals = nullptr; p.dst_keys = nullptr; p.dst_vals = nullptr; p.pass = 0;
+  hipLaunchKernelGGL(sort_clear_hist_kernel, dim3((4 * kBins + 255) / 256), dim3(256), 0, s, p.hist, 4 * kBins);
+  int setup_blocks = p.chunks < 512 ? p.chunks : 512;
+  hipLaunchKernelGGL(sort_setup_kernel, dim3(setup_blocks), dim3(kSortThreads), 0, s, p);
+  // the last pass writes the caller's arrays; the passes before it alternate
+  for (int q = 0; q < p.passes; ++q) {
+    const bool to_out = ((p.passes - 1 - q) & 1) == 0;
+    SortParams r = p;
+    r.pass = q;
+    r.dst_keys = to_out ? sorted : tmp_keys;
+    r.dst_vals = to_out ? argsort : tmp_vals;
+    r.src_keys = to_out ? tmp_keys : sorted;
+    r.src_vals = to_out ? tmp_vals : argsort;
+    hipLaunchKernelGGL(sort_pass_kernel, dim3(p.chunks), dim3(kSortThreads), 0, s, r);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace cummhip

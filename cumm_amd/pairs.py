@@ -20,8 +20,8 @@ import numpy as np
 class PairTable(NamedTuple):
     indices_fwd: np.ndarray   # [kv, N_out] int32: output row -> input row, -1 = none
     indices_bwd: np.ndarray   # [kv, N_in]  int32: input row -> output row, -1 = none
-    mask_fwd: np.ndarray      # [N_out] uint32, bit k set iff indices_fwd[k][o] >= 0
-    mask_bwd: np.ndarray      # [N_in]  uint32, bit k set iff indices_bwd[k][i] >= 0
+    mask_fwd: np.ndarray      # [N_out] uint32, bit k set iff indices_fwd[k][o] >= 0 (None if kv > 32)
+    mask_bwd: np.ndarray      # [N_in]  uint32, bit k set iff indices_bwd[k][i] >= 0 (None if kv > 32)
     out_coords: np.ndarray    # [N_out, 4] int32 (batch, z, y, x)
     out_shape: Tuple[int, int, int]
 
@@ -37,9 +37,12 @@ def _offsets(ksize: Sequence[int]) -> np.ndarray:
     return np.stack([kz.ravel(), ky.ravel(), kx.ravel()], axis=1).astype(np.int64)
 
 
-def _masks(indices: np.ndarray) -> np.ndarray:
+def _masks(indices: np.ndarray):
+    """One bit per kernel offset; kernel volumes above 32 have no 32-bit masks (None): their
+    tables feed the per-offset convolution (:func:`pair_lists`), not the mask-based kernels."""
     kv = indices.shape[0]
-    assert kv <= 32
+    if kv > 32:
+        return None
     bits = (np.uint32(1) << np.arange(kv, dtype=np.uint32))[:, None]
     return np.bitwise_or.reduce(np.where(indices >= 0, bits, np.uint32(0)), axis=0).astype(np.uint32)
 
@@ -143,6 +146,28 @@ def sort_by_mask(mask: np.ndarray, mask_filter: int = 0xFFFFFFFF):
     return np.ascontiguousarray(key[order]), order
 
 
+class PairLists(NamedTuple):
+    pair_in: np.ndarray    # [kv, N] int32: input rows of offset k's pairs, packed to the front
+    pair_out: np.ndarray   # [kv, N] int32: their output rows (ascending)
+    counts: np.ndarray     # [kv] int32: pairs per offset
+
+
+def pair_lists(indices_fwd: np.ndarray) -> PairLists:
+    """Per-offset (input row, output row) lists of a forward pair table, ascending output row:
+    what the per-offset ("native") convolution walks (spconv's indice_pairs / indice_num_per_loc,
+    rebuilt the same way in cumm/conv/main_real_spconv.py:300-326 of the reference)."""
+    kv, n = indices_fwd.shape
+    pin = np.full((kv, n), -1, np.int32)
+    pout = np.full((kv, n), -1, np.int32)
+    counts = np.zeros(kv, np.int32)
+    for k in range(kv):
+        o = np.nonzero(indices_fwd[k] >= 0)[0]
+        counts[k] = o.size
+        pin[k, :o.size] = indices_fwd[k, o]
+        pout[k, :o.size] = o
+    return PairLists(pin, pout, counts)
+
+
 # ---- the same tables built on the GPU (cumm_hip_subm_pairs / cumm_hip_sort_by_mask) ----------
 
 class DevicePairTable(NamedTuple):
@@ -153,10 +178,13 @@ class DevicePairTable(NamedTuple):
 
 
 def subm_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), dilation=(1, 1, 1),
-                      workspace=None, stream: int = 0) -> DevicePairTable:
+                      workspace=None, stream: int = 0, out: "DevicePairTable" = None) -> DevicePairTable:
     """GPU counterpart of :func:`subm_pairs`: ``coords`` is a device ``tv.Tensor`` [N, 4] int32 of
     unique (batch, z, y, x); the tables stay on the device.  What the reference's callers take from
-    ``SpconvOps.generate_subm_conv_inds`` (cumm/conv/main_real_spconv.py:91-105 of the reference)."""
+    ``SpconvOps.generate_subm_conv_inds`` (cumm/conv/main_real_spconv.py:91-105 of the reference).
+    With ``workspace`` (``cumm_hip_subm_pairs_workspace(n)`` bytes) and ``out`` (a DevicePairTable
+    of the right shapes, e.g. the previous call's result) the call allocates nothing.  Kernel
+    volumes above 32 (up to 128) come without masks."""
     import ctypes as C
 
     from . import _capi
@@ -170,15 +198,21 @@ def subm_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), dil
     need = int(lib.cumm_hip_subm_pairs_workspace(n))
     if workspace is None or workspace.empty():
         workspace = tv.empty([max(need, 16)], tv.uint8, 0)
-    ind_f = tv.empty([kv, n], tv.int32, 0)
-    ind_b = tv.empty([kv, n], tv.int32, 0)
-    mask_f = tv.empty([n], tv.uint32, 0)
-    mask_b = tv.empty([n], tv.uint32, 0)
+    if out is not None:     # the caller's tensors, reused from call to call: nothing is allocated
+        ind_f, ind_b, mask_f, mask_b = out
+        if (ind_f.shape != [kv, n] or ind_b.shape != [kv, n] or ind_f.dtype != tv.int32 or ind_b.dtype != tv.int32):
+            raise ValueError("out must hold int32 tables of shape [kv, N]")
+    else:
+        ind_f = tv.empty([kv, n], tv.int32, 0)
+        ind_b = tv.empty([kv, n], tv.int32, 0)
+        mask_f = tv.empty([n], tv.uint32, 0) if kv <= 32 else None
+        mask_b = tv.empty([n], tv.uint32, 0) if kv <= 32 else None
     arr3 = C.c_int32 * 3
     _capi.check(lib.cumm_hip_subm_pairs(
         coords.byte_pointer(), n, arr3(*[int(v) for v in spatial_shape]), arr3(*[int(v) for v in ksize]),
-        arr3(*[int(v) for v in dilation]), ind_f.byte_pointer(), ind_b.byte_pointer(), mask_f.byte_pointer(),
-        mask_b.byte_pointer(), workspace.byte_pointer(), workspace.nbytes, stream))
+        arr3(*[int(v) for v in dilation]), ind_f.byte_pointer(), ind_b.byte_pointer(),
+        mask_f.byte_pointer() if mask_f is not None else None,
+        mask_b.byte_pointer() if mask_b is not None else None, workspace.byte_pointer(), workspace.nbytes, stream))
     return DevicePairTable(ind_f, ind_b, mask_f, mask_b)
 
 
@@ -211,7 +245,7 @@ def sparse_conv_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 
     geo = [arr3(*[int(v) for v in a]) for a in (spatial_shape, ksize, stride, padding, dilation)]
     need = int(lib.cumm_hip_conv_pairs_workspace(n_in, int(batch_size), *geo))
     if need == 0:
-        raise ValueError("bad geometry (kernel volume 1..32, non-empty output grid) or too many voxels")
+        raise ValueError("bad geometry (kernel volume 1..128, non-empty output grid) or too many voxels")
     if workspace is None or workspace.empty():
         workspace = tv.empty([max(need, 256)], tv.uint8, 0)
     out_shape = arr3()
@@ -222,19 +256,21 @@ def sparse_conv_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 
     out_coords = tv.empty([n, 4], tv.int32, 0)
     ind_f = tv.empty([kv, n], tv.int32, 0)
     ind_b = tv.empty([kv, n_in], tv.int32, 0)
-    mask_f = tv.empty([n], tv.uint32, 0)
-    mask_b = tv.empty([n_in], tv.uint32, 0)
+    mask_f = tv.empty([n], tv.uint32, 0) if kv <= 32 else None
+    mask_b = tv.empty([n_in], tv.uint32, 0) if kv <= 32 else None
     _capi.check(lib.cumm_hip_conv_pairs_fill(
         coords.byte_pointer(), n_in, int(batch_size), *geo, n, out_coords.byte_pointer(), ind_f.byte_pointer(),
-        ind_b.byte_pointer(), mask_f.byte_pointer(), mask_b.byte_pointer(), workspace.byte_pointer(),
+        ind_b.byte_pointer(), mask_f.byte_pointer() if mask_f is not None else None,
+        mask_b.byte_pointer() if mask_b is not None else None, workspace.byte_pointer(),
         workspace.nbytes, stream))
     return DeviceConvPairTable(ind_f, ind_b, mask_f, mask_b, out_coords, tuple(int(v) for v in out_shape))
 
 
-def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, stream: int = 0):
+def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, stream: int = 0, out=None):
     """GPU counterpart of :func:`sort_by_mask` on a device ``tv.Tensor`` [N] uint32: returns
     (sorted mask, argsort) device tensors (spconv's sort_1d_by_key[_split], call site
-    cumm/conv/main_real_spconv.py:118-145 of the reference)."""
+    cumm/conv/main_real_spconv.py:118-145 of the reference).  With ``workspace`` and ``out`` =
+    (sorted mask, argsort) tensors of a previous call the call allocates nothing."""
     from . import _capi
     from . import tensorview as tv
     if mask.device < 0 or mask.dtype != tv.uint32 or mask.ndim != 1:
@@ -244,9 +280,42 @@ def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, str
     need = int(lib.cumm_hip_sort_by_mask_workspace(n))
     if workspace is None or workspace.empty():
         workspace = tv.empty([max(need, 256)], tv.uint8, 0)
-    out_mask = tv.empty([n], tv.uint32, 0)
-    order = tv.empty([n], tv.int32, 0)
+    if out is not None:
+        out_mask, order = out
+        if out_mask.shape != [n] or order.shape != [n] or out_mask.dtype != tv.uint32 or order.dtype != tv.int32:
+            raise ValueError("out must be (uint32 [N], int32 [N]) device tensors")
+    else:
+        out_mask = tv.empty([n], tv.uint32, 0)
+        order = tv.empty([n], tv.int32, 0)
     _capi.check(lib.cumm_hip_sort_by_mask(mask.byte_pointer(), n, int(mask_filter) & 0xFFFFFFFF,
                                           out_mask.byte_pointer(), order.byte_pointer(),
                                           workspace.byte_pointer(), workspace.nbytes, stream))
     return out_mask, order
+
+
+class DevicePairLists(NamedTuple):
+    pair_in: "object"    # tv.Tensor [kv, N] int32 on the device
+    pair_out: "object"   # tv.Tensor [kv, N] int32
+    counts: np.ndarray   # [kv] int32 on the host (the launches of the per-offset convolution are sized by them)
+
+
+def pair_lists_device(indices_fwd, workspace=None, stream: int = 0) -> DevicePairLists:
+    """GPU counterpart of :func:`pair_lists` on a device table [kv, N]; the counts come back to
+    the host (one stream synchronisation): the per-offset launches are sized by them."""
+    from . import _capi
+    from . import tensorview as tv
+    if indices_fwd.device < 0 or indices_fwd.dtype != tv.int32 or indices_fwd.ndim != 2:
+        raise ValueError("indices_fwd must be a device int32 tensor [kv, N]")
+    kv, n = int(indices_fwd.shape[0]), int(indices_fwd.shape[1])
+    lib = _capi.lib()
+    need = int(lib.cumm_hip_pair_lists_workspace(kv, n))
+    if workspace is None or workspace.empty():
+        workspace = tv.empty([max(need, 4)], tv.uint8, 0)
+    pin = tv.empty([kv, n], tv.int32, 0)
+    pout = tv.empty([kv, n], tv.int32, 0)
+    counts = tv.empty([kv], tv.int32, 0)
+    _capi.check(lib.cumm_hip_pair_lists(indices_fwd.byte_pointer(), kv, n, pin.byte_pointer(), pout.byte_pointer(),
+                                        counts.byte_pointer(), workspace.byte_pointer(), workspace.nbytes, stream))
+    ctx = tv.Context()
+    ctx.set_cuda_stream(stream)
+    return DevicePairLists(pin, pout, counts.cpu(ctx).numpy())

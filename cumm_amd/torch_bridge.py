@@ -3,14 +3,16 @@ convolution (forward = implicit_gemm2 Forward, backward = BackwardInput + Backwa
 
 ``torch2tensor`` / ``tensor2torch`` stand where the reference's ``PyTorchTools.torch2tensor`` /
 ``tensor2torch`` do (cumm/bindings.py:53-86 over include/tensorview/torch_utils.h).  torch is
-plumbing here: it owns activations, parameters and the stream; every kernel that runs is this
-library's.  Imported on demand: nothing else in the package needs torch.
+plumbing here: it owns activations, parameters and the stream (allocation, zero fill, making a
+tensor contiguous); every computing kernel that runs is this library's, including the ReLU gate
+and the bias gradient of the backward pass.  Imported on demand: nothing else in the package
+needs torch.
 """
 from typing import Optional, Sequence, Tuple
 
 import torch
 
-from . import pairs, tuner
+from . import _capi, pairs, tuner
 from . import tensorview as tv
 from .conv.main import ConvMainUnitTest
 from .tensorview.gemm import Activation, ConvOpType, ConvParams
@@ -116,20 +118,13 @@ class SparseConvGeometry:
             self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, stream=stream)
         self._reduced = {}
 
-    def reduced_mask(self, width: int) -> tv.Tensor:
-        """OR of the sorted forward masks over runs of ``width`` positions (backward-weight)."""
+    def reduced_mask_buffer(self, width: int) -> tv.Tensor:
+        """One word per run of ``width`` sorted output positions: the forward launch writes the
+        OR of the run's masks here (its ``mask_output``), and backward-weight reads it."""
         if width not in self._reduced:
-            m = tensor2torch(self.mask_fwd, clone=False, cast_uint_to_int=True)
             tiles = (self.n_out + width - 1) // width
-            padded = torch.zeros(tiles * width, dtype=torch.int32, device=m.device)
-            padded[: self.n_out] = m
-            red = padded.view(tiles, width)
-            while red.shape[1] > 1:
-                half = red.shape[1] // 2
-                red = torch.bitwise_or(red[:, :half], red[:, half:2 * half]) if red.shape[1] % 2 == 0 else \
-                    torch.cat([torch.bitwise_or(red[:, :half], red[:, half:2 * half]), red[:, 2 * half:]], dim=1)
-            red = red.reshape(tiles).contiguous()
-            self._reduced[width] = (torch2tensor(red).type_view(tv.uint32), red)
+            buf = torch.zeros(max(tiles, 1), dtype=torch.int32, device=self.out_coords.device)
+            self._reduced[width] = (torch2tensor(buf).type_view(tv.uint32), buf)
         return self._reduced[width][0]
 
 
@@ -150,8 +145,11 @@ class _SparseConvFunction(torch.autograd.Function):
             p.act_type = Activation.ReLU
         p.stream = current_stream()
         _TUNER.tune_conv(p)
+        # the tile masks the forward launch computes anyway are what backward-weight needs
+        tile_m = int(p.conv_algo_desp.tile_shape[0])
+        p.mask_output = geometry.reduced_mask_buffer(tile_m)
         ConvMainUnitTest.implicit_gemm2(p)
-        ctx.geometry, ctx.relu, ctx.has_bias = geometry, relu, bias is not None
+        ctx.geometry, ctx.relu, ctx.has_bias, ctx.tile_m = geometry, relu, bias is not None, tile_m
         ctx.save_for_backward(features, weight, out if relu else None)
         return out
 
@@ -160,10 +158,14 @@ class _SparseConvFunction(torch.autograd.Function):
         features, weight, out = ctx.saved_tensors
         g: SparseConvGeometry = ctx.geometry
         grad_out = grad_out.contiguous()
-        if ctx.relu:
-            grad_out = grad_out * (out > 0).to(grad_out.dtype)
         dtype = _TORCH_TO_TV[features.dtype]
         stream = current_stream()
+        lib = _capi.lib()
+        if ctx.relu:       # the gradient passes where the fused ReLU let the output through
+            gated = torch.empty_like(grad_out)
+            _capi.check(lib.cumm_hip_relu_backward(gated.data_ptr(), grad_out.data_ptr(), out.data_ptr(),
+                                                   grad_out.numel(), dtype, stream))
+            grad_out = gated
         grad_in = grad_w = grad_b = None
         if ctx.needs_input_grad[0]:
             # inputs that feed no output site sit in tiles the kernel skips (mask 0): zero them
@@ -181,12 +183,17 @@ class _SparseConvFunction(torch.autograd.Function):
             p = ConvParams(3, ConvOpType.BackwardWeight)
             p.conv_algo_desp = _desp_like(dtype, ConvOpType.BackwardWeight, parallel=True)
             p.input, p.weight, p.output = torch2tensor(features), torch2tensor(grad_w), torch2tensor(grad_out)
-            p.indices, p.mask, p.mask_argsort = g.indices_fwd, g.reduced_mask(64), g.order_fwd
-            p.mask_width, p.split_k_slices = 64, 32
+            p.indices, p.mask, p.mask_argsort = g.indices_fwd, g.reduced_mask_buffer(ctx.tile_m), g.order_fwd
+            p.mask_width, p.split_k_slices = ctx.tile_m, 32
             p.stream = stream
             ConvMainUnitTest.implicit_gemm2(p)
         if ctx.has_bias and ctx.needs_input_grad[2]:
-            grad_b = grad_out.float().sum(0).to(grad_out.dtype)
+            rows, k_out = int(grad_out.shape[0]), int(grad_out.shape[1])
+            grad_b = torch.empty(k_out, dtype=grad_out.dtype, device=grad_out.device)
+            need = int(lib.cumm_hip_column_sum_workspace(rows, k_out))
+            ws = torch.empty(max(need, 4), dtype=torch.uint8, device=grad_out.device)
+            _capi.check(lib.cumm_hip_column_sum(grad_b.data_ptr(), grad_out.data_ptr(), rows, k_out, dtype,
+                                                ws.data_ptr(), need, stream))
         return grad_in, grad_w, grad_b, None, None
 
 

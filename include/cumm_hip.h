@@ -43,6 +43,8 @@ extern "C" {
 #define CUMM_HIP_NO_SHUFFLE 0
 #define CUMM_HIP_SHUFFLE_AC 1
 #define CUMM_HIP_SHUFFLE_AB 2
+#define CUMM_HIP_CONV_CONVOLUTION 0
+#define CUMM_HIP_CONV_CROSS_CORRELATION 1
 #define CUMM_HIP_ACT_NONE 0
 #define CUMM_HIP_ACT_RELU 1
 #define CUMM_HIP_ACT_SIGMOID 2
@@ -112,6 +114,9 @@ typedef struct CummHipSparseConvArgs {
   int32_t mask_width;               /* wgrad: positions covered by one mask word */
   int32_t ndim, N, C, K;
   int32_t kernel_volume;
+  int32_t mode;                     /* tv::gemm::ConvMode: must be CUMM_HIP_CONV_CROSS_CORRELATION, the only one
+                                       the reference's mask-based kernels implement */
+  int32_t groups;                   /* must be 1 */
   int32_t d_is_bias;
   const void *bias_pointer;         /* int8 inference: f32 [K] */
   const void *scale_pointer;        /* int8 inference: f32 [K] */
@@ -140,6 +145,14 @@ int cumm_hip_sparse_conv(const CummHipConvDesc *desc, const CummHipSparseConvArg
 #define CUMM_HIP_STATIC_WORKSPACE_BYTES (8u << 20)
 int cumm_hip_sparse_conv_static_ws(const CummHipConvDesc *desc, const CummHipSparseConvArgs *args,
                                    void *stream);
+
+/* GemmAlgoDesp::query_workspace_size / ConvAlgoDesp::query_conv_workspace_size
+ * (include/tensorview/gemm/core/params.h:115-132, 286-307): bytes of workspace a launch with these
+ * m, n, k (GemmUtils::implicit_gemm_mnk for a convolution, utils.h:62-92) and split_k_slices needs;
+ * 0 when it needs none; -1 for a descriptor without a split-K variant and split_k_slices > 1. */
+int64_t cumm_hip_query_gemm_workspace(const CummHipGemmDesc *desc, int m, int n, int k, int split_k_slices);
+int64_t cumm_hip_query_conv_workspace(const CummHipConvDesc *desc, int m, int n, int k, int split_k_slices,
+                                      int kernel_volume);
 
 /* GemmMainUnitTest.get_all_algo_desp / ConvMainUnitTest.get_all_conv_algo_desp
  * (cumm/gemm/main.py:914-965, cumm/conv/main.py:467-481): the descriptors this
@@ -196,9 +209,10 @@ int cumm_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* host out-p
  * linear-probing hash table include/tensorview/hash/linear.cu.h:111-840.
  *
  * cumm_hip_subm_pairs: pair tables of a submanifold convolution.
- *   coords [n, 4] int32 (batch, z, y, x), unique; spatial_shape, ksize (odd sizes, kernel volume <= 32),
+ *   coords [n, 4] int32 (batch, z, y, x), unique; spatial_shape, ksize (odd sizes, kernel volume <= 128),
  *   dilation: 3 ints each (host).  Outputs (device): indices_fwd [kv, n] int32 (-1 = none),
- *   mask_fwd [n] uint32; indices_bwd / mask_bwd may be NULL.  Kernel offset k = (kz*KY + ky)*KX + kx,
+ *   mask_fwd [n] uint32; indices_bwd / mask_fwd / mask_bwd may be NULL.  A kernel volume above 32
+ *   has no 32-bit masks (pass NULL for both): its tables feed the per-offset convolution.  Kernel offset k = (kz*KY + ky)*KX + kx,
  *   output o gathers the input at coord[o] + (k_zyx - ksize/2) * dilation.
  *   workspace: at least cumm_hip_subm_pairs_workspace(n) bytes, 16-byte aligned.
  * cumm_hip_sort_by_mask: sorted = stable ascending sort of (mask & mask_filter), argsort = the
@@ -228,7 +242,8 @@ int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uin
  * batch_size: the batch indices of coords are 0 .. batch_size-1 (others are ignored).  Output
  *   grids of up to 2^33 sites (batch included) are handled with a bitmap of the grid (an eighth
  *   of a byte per site, twice), larger ones with a hash set and a sort: same results.
- * workspace: at least cumm_hip_conv_pairs_workspace(...) bytes (0 = bad geometry), 256-byte aligned. */
+ * workspace: at least cumm_hip_conv_pairs_workspace(...) bytes (0 = bad geometry), 256-byte aligned.
+ * Kernel volumes up to 128; above 32 there are no 32-bit masks: pass NULL for mask_fwd and mask_bwd. */
 size_t cumm_hip_conv_pairs_workspace(int n_in, int batch_size, const int32_t *spatial_shape, const int32_t *ksize,
                                      const int32_t *stride, const int32_t *padding, const int32_t *dilation);
 int cumm_hip_conv_pairs_sites(const int32_t *coords, int n_in, int batch_size, const int32_t *spatial_shape,
@@ -240,6 +255,18 @@ int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, co
                              const int32_t *dilation, int n_out, int32_t *out_coords, int32_t *indices_fwd,
                              int32_t *indices_bwd, uint32_t *mask_fwd, uint32_t *mask_bwd, void *workspace,
                              size_t workspace_bytes, void *stream);
+
+/* Per-offset pair lists out of a pair table indices [kv, n] (either direction): for every offset k
+ * the pairs (indices[k][o], o) with indices[k][o] >= 0, ascending o, packed to the front of
+ * pair_in[k, :] / pair_out[k, :] ([kv, n] each), their number in counts[k] (device).  This is the
+ * form the per-offset ("native") convolution walks - SparseConvAlgo::kNative,
+ * include/tensorview/gemm/core/constants.h:34-38; spconv's indice_pairs [2, kv, N] and
+ * indice_num_per_loc, as rebuilt in cumm/conv/main_real_spconv.py:300-326 - and the only one for
+ * kernel volumes above 32, which the 32-bit masks cannot describe.
+ * workspace: cumm_hip_pair_lists_workspace(kv, n) bytes. */
+size_t cumm_hip_pair_lists_workspace(int kv, int n);
+int cumm_hip_pair_lists(const int32_t *indices, int kv, int n, int32_t *pair_in, int32_t *pair_out, int32_t *counts,
+                        void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- stand-alone row gather / scatter-add (the "native" per-offset path around a plain GEMM)
  * cumm_hip_gather_rows: output[i, :] = input[indices[i], :] for i < m; rows of row_bytes bytes
@@ -254,6 +281,21 @@ int cumm_hip_gather_rows(void *output, const void *input, const int32_t *indices
                          size_t row_bytes, void *stream);
 int cumm_hip_scatter_add_rows(void *output, const void *input, const int32_t *indices, int m, int rows_out,
                               int channels, int dtype, void *stream);
+
+/* ---- row-wise helpers between launches.  The reference has no counterpart: its callers (spconv's
+ * autograd functions and its native convolution) take these steps from torch.
+ * cumm_hip_finish_rows: out[r, c] = cvt(act(alpha * acc[r, c] + beta * bias[c])) for an fp32 image
+ *   acc [rows, channels] of a result (the per-offset native convolution accumulates in fp32 and
+ *   rounds once); out f16 / bf16 (dtype), bias [channels] in that type or NULL, channels % 8 == 0.
+ * cumm_hip_relu_backward: dst[i] = out[i] > 0 ? grad[i] : 0 (the gradient through a fused ReLU).
+ * cumm_hip_column_sum: dst[c] = cvt(sum over rows of src[r, c]) in fp32, same result from run to
+ *   run (the gradient of a bias); workspace of cumm_hip_column_sum_workspace(rows, channels) bytes. */
+int cumm_hip_finish_rows(void *out, int dtype, const float *acc, const void *bias, int64_t rows, int channels,
+                         float alpha, float beta, int act_type, float act_alpha, void *stream);
+int cumm_hip_relu_backward(void *dst, const void *grad, const void *out, size_t elems, int dtype, void *stream);
+size_t cumm_hip_column_sum_workspace(int64_t rows, int channels);
+int cumm_hip_column_sum(void *dst, const void *src, int64_t rows, int channels, int dtype, void *workspace,
+                        size_t workspace_bytes, void *stream);
 
 /* Plain device-to-device copy kernel of `bytes` bytes (16-byte aligned); used to
  * calibrate the HBM traffic counters against a transfer of known size. */

@@ -31,7 +31,7 @@ def test_struct_layouts_match_the_header():
     """sizeof() of the ctypes mirrors against the C compiler's view of include/cumm_hip.h
     (a silent drift would corrupt arguments); the literal sizes guard machines without gcc."""
     sizes = [ctypes.sizeof(c) for c in (_capi.GemmDesc, _capi.ConvDesc, _capi.GemmArgs, _capi.SparseConvArgs)]
-    assert sizes == [72, 96, 160, 168]
+    assert sizes == [72, 96, 160, 176]
     import shutil
     import subprocess
     import tempfile
@@ -94,5 +94,37 @@ def test_argument_errors_without_a_gpu():
     lib.cumm_hip_list_conv_algos(carr, m)
     sargs = _capi.SparseConvArgs()
     sargs.N, sargs.C, sargs.K, sargs.kernel_volume = 10, 64, 64, 125
+    sargs.mode, sargs.groups = 1, 1
     assert lib.cumm_hip_sparse_conv(ctypes.byref(carr[0]), ctypes.byref(sargs), None) == _capi.EINVAL
+    assert b"kernel volume" in lib.cumm_hip_last_error()
+    # true convolution (flipped kernel) and grouped convolution have no kernel
+    sargs.kernel_volume, sargs.mode = 27, 0
+    assert lib.cumm_hip_sparse_conv(ctypes.byref(carr[0]), ctypes.byref(sargs), None) == _capi.EINVAL
+    assert b"cross-correlation" in lib.cumm_hip_last_error()
+    sargs.mode, sargs.groups = 1, 2
+    assert lib.cumm_hip_sparse_conv(ctypes.byref(carr[0]), ctypes.byref(sargs), None) == _capi.EINVAL
+    assert b"groups" in lib.cumm_hip_last_error()
     assert lib.cumm_hip_copy_kernel(8, 16, 32, None) == _capi.EINVAL
+
+
+def test_workspace_queries_follow_the_descriptors():
+    """cumm_hip_query_*_workspace against the Python mirrors of GemmAlgoDesp.query_workspace_size /
+    ConvAlgoDesp.query_conv_workspace_size (which the golden cases pin against the reference's headers)."""
+    from cumm_amd.conv.main import ConvMainUnitTest, conv_desp_to_c
+    from cumm_amd.gemm.main import GemmMainUnitTest, desp_to_c
+    lib = _capi.lib()
+    for d in GemmMainUnitTest.get_all_algo_desp():
+        cd = desp_to_c(d)
+        for m, n, k, s in ((1000, 136, 64, 1), (1000, 136, 640, 4), (64, 64, 64, 2)):
+            if s > 1 and not (d.split_k_serial or d.split_k_parallel):
+                assert lib.cumm_hip_query_gemm_workspace(ctypes.byref(cd), m, n, k, s) == -1
+            else:
+                assert lib.cumm_hip_query_gemm_workspace(ctypes.byref(cd), m, n, k, s) == d.query_workspace_size(m, n, k, s)
+    for d in ConvMainUnitTest.get_all_conv_algo_desp():
+        cd = conv_desp_to_c(d)
+        for m, n, k, s, kv in ((64, 27 * 64, 120000, 1, 27), (128, 27 * 128, 5000, 32, 27), (64, 8 * 72, 999, 2, 8)):
+            if s > 1 and not (d.split_k_serial or d.split_k_parallel):
+                assert lib.cumm_hip_query_conv_workspace(ctypes.byref(cd), m, n, k, s, kv) == -1
+            else:
+                assert lib.cumm_hip_query_conv_workspace(ctypes.byref(cd), m, n, k, s, kv) == \
+                    d.query_conv_workspace_size(m, n, k, s, kv)

@@ -61,7 +61,19 @@ def test_pairs_argument_errors():
     assert lib.cumm_hip_subm_pairs_workspace(1000) >= 2 * 1000 * 16
     c = tv.zeros([8, 4], tv.int32, 0)
     with pytest.raises(ValueError):
-        pairs.subm_pairs_device(c, (4, 4, 4), ksize=(3, 3, 5))        # kernel volume 45 > 32
+        pairs.subm_pairs_device(c, (4, 4, 4), ksize=(5, 5, 7))        # kernel volume 175 > 128
+    with pytest.raises(ValueError):
+        pairs.subm_pairs_device(c, (4, 4, 4), ksize=(3, 2, 3))        # even kernel size
+    # kernel volume 45: tables without masks; asking for masks is an error
+    big = pairs.subm_pairs_device(c, (4, 4, 4), ksize=(3, 3, 5))
+    assert big.mask_fwd is None and big.indices_fwd.shape == [45, 8]
+    import ctypes as C
+    arr3 = C.c_int32 * 3
+    ws = tv.zeros([int(lib.cumm_hip_subm_pairs_workspace(8))], tv.uint8, 0)
+    m = tv.zeros([8], tv.uint32, 0)
+    assert lib.cumm_hip_subm_pairs(c.byte_pointer(), 8, arr3(4, 4, 4), arr3(3, 3, 5), arr3(1, 1, 1),
+                                   big.indices_fwd.byte_pointer(), None, m.byte_pointer(), None,
+                                   ws.byte_pointer(), ws.nbytes, 0) == _capi.EINVAL
     with pytest.raises(RuntimeError):
         pairs.subm_pairs_device(c, (4, 4, 4), workspace=tv.zeros([64], tv.uint8, 0))   # too small
 
@@ -151,8 +163,41 @@ def test_sparse_conv_pairs_empty_and_errors():
     assert got.out_coords.shape[0] == 0 and tuple(got.out_shape) == (4, 4, 4)
     c = tv.zeros([8, 4], tv.int32, 0)
     with pytest.raises(ValueError):
-        pairs.sparse_conv_pairs_device(c, (4, 4, 4), ksize=(3, 3, 5))        # kernel volume 45 > 32
+        pairs.sparse_conv_pairs_device(c, (8, 8, 8), ksize=(5, 5, 7))        # kernel volume 175 > 128
     with pytest.raises(ValueError):
         pairs.sparse_conv_pairs_device(c, (2, 2, 2), ksize=(3, 3, 3), padding=(0, 0, 0))   # no output
     with pytest.raises(RuntimeError):
         pairs.sparse_conv_pairs_device(c, (4, 4, 4), workspace=tv.zeros([256], tv.uint8, 0))   # too small
+
+
+@pytest.mark.parametrize("n", [1, 63, 4096, 4097, 50000, 300001])
+@pytest.mark.parametrize("kind", ["random27", "few", "all_equal", "random32", "sorted", "reverse"])
+def test_sort_by_mask_against_stable_argsort(n, kind):
+    """The hand-written radix sort against numpy's stable argsort: random 27- and 32-bit keys, a
+    handful of distinct keys (long runs of ties across chunk borders), one key only, keys already
+    in order and in reverse; with a filter that drops bits; outputs and workspace reused."""
+    print("case sort", n, kind, flush=True)
+    rng = np.random.default_rng(n + len(kind))
+    if kind == "random27":
+        mask = rng.integers(0, 1 << 27, size=n, dtype=np.uint32)
+    elif kind == "random32":
+        mask = rng.integers(0, 1 << 32, size=n, dtype=np.uint64).astype(np.uint32)
+    elif kind == "few":
+        mask = rng.choice(np.array([0x2000, 0x6000, 0x7FFFFFF, 0x2001, 0x4002000], np.uint32), size=n)
+    elif kind == "all_equal":
+        mask = np.full(n, 0x2000, np.uint32)
+    elif kind == "sorted":
+        mask = np.sort(rng.integers(0, 1 << 27, size=n, dtype=np.uint32))
+    else:
+        mask = np.sort(rng.integers(0, 1 << 27, size=n, dtype=np.uint32))[::-1].copy()
+    d_mask = H.dev(mask, "u32")
+    lib = _capi.lib()
+    ws = tv.empty([int(lib.cumm_hip_sort_by_mask_workspace(n))], tv.uint8, 0)
+    out = (tv.empty([n], tv.uint32, 0), tv.empty([n], tv.int32, 0))
+    for filt in (0xFFFFFFFF, 0x07FFFFFF, 0x3FFF, 0x1FFF << 14, 0x1):
+        ms_ref, order_ref = pairs.sort_by_mask(mask, filt)
+        ms, order = pairs.sort_by_mask_device(d_mask, filt, workspace=ws, out=out)
+        np.testing.assert_array_equal(H.host(ms), ms_ref)
+        np.testing.assert_array_equal(H.host(order), order_ref)
+    from cumm_amd.gemm.main import GemmMainUnitTest
+    GemmMainUnitTest.device_synchronize()      # (would raise if a look-back had given up)
