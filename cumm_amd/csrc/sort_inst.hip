@@ -30,7 +30,7 @@ constexpr int kSortWaves = kSortThreads / 64;     // 8
 constexpr int kItems = 8;                         // keys per lane
 constexpr int kChunk = kSortThreads * kItems;     // 4096 keys per workgroup
 constexpr uint32_t kFlagAggregate = 1u << 30, kFlagInclusive = 2u << 30, kValueMask = (1u << 30) - 1u;
-constexpr int kLookbackSpins = 1 << 22;
+constexpr int kLookbackSpins = 1 << 20;   // (about a second)
 
 struct SortParams {
   const uint32_t *mask;      // [n] the caller's masks
@@ -57,9 +57,34 @@ __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortPara
   for (size_t i = (size_t)blockIdx.x * kSortThreads + t; i < words; i += (size_t)gridDim.x * kSortThreads) p.state[i] = 0u;
   if (blockIdx.x == 0 && t < p.passes) p.tickets[t] = 0u;
   __syncthreads();
-  for (int64_t i = (int64_t)blockIdx.x * kSortThreads + t; i < p.n; i += (int64_t)gridDim.x * kSortThreads) {
-    const uint32_t key = p.mask[i] & p.filter;
-    for (int q = 0; q < p.passes; ++q) atomicAdd(&lds_hist[q][(key >> (q * kRadixBits)) & (kBins - 1)], 1u);
+  // lanes of a wave with the same digit add once (most masks of a sparse cloud are the same word:
+  // one add per lane would queue 64 deep on one LDS address)
+  const int lane = t & 63;
+  const int64_t span = (int64_t)gridDim.x * kSortThreads;
+  const int64_t rounds = (p.n + span - 1) / span;
+  for (int64_t r0 = 0; r0 < rounds; r0 += kItems) {
+    // kItems keys per lane are requested together (one memory round trip, not one per key)
+    uint32_t keys[kItems];
+    bool valids[kItems];
+#pragma unroll
+    for (int u = 0; u < kItems; ++u) {
+      const int64_t i = (r0 + u) * span + (int64_t)blockIdx.x * kSortThreads + t;
+      valids[u] = r0 + u < rounds && i < p.n;
+      keys[u] = valids[u] ? (p.mask[i] & p.filter) : 0u;
+    }
+#pragma unroll
+    for (int u = 0; u < kItems; ++u) {
+      for (int q = 0; q < p.passes; ++q) {
+        const uint32_t d = (keys[u] >> (q * kRadixBits)) & (kBins - 1);
+        unsigned long long peers = __ballot(valids[u]);
+#pragma unroll
+        for (int b = 0; b < kRadixBits; ++b) {
+          const unsigned long long has = __ballot((d >> b) & 1u);
+          peers &= ((d >> b) & 1u) ? has : ~has;
+        }
+        if (valids[u] && (peers & ((1ull << lane) - 1ull)) == 0ull) atomicAdd(&lds_hist[q][d], (uint32_t)__popcll(peers));
+      }
+    }
   }
   __syncthreads();
   for (int q = 0; q < p.passes; ++q) {
@@ -86,17 +111,21 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   if (t == 0) chunk_of_block = (int)atomicAdd(&p.tickets[p.pass], 1u);
 #pragma unroll
   for (int w = 0; w < kSortWaves; ++w) wave_hist[w][t] = 0u;
-  // exclusive prefix over the digit values of the whole input: thread = bin, Hillis-Steele
+  // exclusive prefix over the digit values of the whole input: thread = bin; a scan inside each
+  // wave by lane shuffles, then the totals of the waves before
   const uint32_t total_of_bin = p.hist[p.pass * kBins + t];
-  scan_tmp[t] = total_of_bin;
-  __syncthreads();
-  for (int off = 1; off < kBins; off <<= 1) {
-    const uint32_t add = t >= off ? scan_tmp[t - off] : 0u;
-    __syncthreads();
-    scan_tmp[t] += add;
-    __syncthreads();
+  uint32_t incl = total_of_bin;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+    if (lane >= off) incl += up;
   }
-  const uint32_t global_excl = scan_tmp[t] - total_of_bin;
+  if (lane == 63) scan_tmp[wave] = incl;
+  __syncthreads();
+  uint32_t waves_before = 0;
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) waves_before += w < wave ? scan_tmp[w] : 0u;
+  const uint32_t global_excl = waves_before + incl - total_of_bin;
   const int chunk = chunk_of_block;
   if (chunk >= p.chunks) return;   // (never: the grid has one workgroup per chunk)
 
@@ -149,27 +178,49 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
     count += c;
   }
   uint32_t *my_state = p.state + ((size_t)p.pass * p.chunks + chunk) * kBins;
-  __hip_atomic_store(&my_state[t], (chunk == 0 ? kFlagInclusive : kFlagAggregate) | count, __ATOMIC_RELEASE,
+  // (relaxed device-scope stores: the word itself carries flag and value, nothing else is published
+  // through it; a release here writes back the whole L2 of the XCD, once per wave)
+  __hip_atomic_store(&my_state[t], (chunk == 0 ? kFlagInclusive : kFlagAggregate) | count, __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
   uint32_t before_chunks = 0;
   if (chunk > 0) {
-    bool gave_up = false;
-    for (int j = chunk - 1; j >= 0; --j) {
-      const uint32_t *st = p.state + ((size_t)p.pass * p.chunks + j) * kBins + t;
-      uint32_t s = __hip_atomic_load(st, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
-      for (int spins = 0; (s >> 30) == 0u && spins < kLookbackSpins; ++spins) {
+    // Look back over the chunks before this one, kLook of them per round trip: the words of a
+    // batch are requested together (the word carries flag and value, so relaxed loads do), then
+    // taken in order until a running total ends the walk; a word that is not there yet is asked
+    // for again, from there.  One thread walking one predecessor per round trip made a pass of
+    // 30 chunks take 45 us.
+    constexpr int kLook = 16;
+    bool gave_up = false, done = false;
+    int j = chunk - 1, spins = 0;
+    while (!done && !gave_up) {
+      uint32_t sw[kLook];
+#pragma unroll
+      for (int i = 0; i < kLook; ++i) {
+        const int c = j - i;
+        sw[i] = c >= 0 ? __hip_atomic_load(p.state + ((size_t)p.pass * p.chunks + c) * kBins + t, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT)
+                       : kFlagInclusive;
+      }
+      int taken = 0;
+#pragma unroll
+      for (int i = 0; i < kLook; ++i) {
+        if (!done && taken == i) {
+          const uint32_t flag = sw[i] >> 30;
+          if (flag != 0u) {
+            before_chunks += sw[i] & kValueMask;
+            ++taken;
+            if (flag == 2u) done = true;
+          }
+        }
+      }
+      j -= taken;
+      if (!done && taken == 0) {
+        if (++spins > kLookbackSpins) gave_up = true;
         __builtin_amdgcn_s_sleep(2);
-        s = __hip_atomic_load(st, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
       }
-      if ((s >> 30) == 0u) {
-        gave_up = true;
-        break;
-      }
-      before_chunks += s & kValueMask;
-      if ((s >> 30) == 2u) break;
     }
     if (gave_up && p.give_ups != nullptr) atomicAdd(p.give_ups, 1);
-    __hip_atomic_store(&my_state[t], kFlagInclusive | (before_chunks + count), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&my_state[t], kFlagInclusive | (before_chunks + count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   bin_base[t] = global_excl + before_chunks;
   __syncthreads();
