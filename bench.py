@@ -30,10 +30,40 @@ from cumm_amd.tensorview.gemm import (ConvOpType, ConvParams, GemmParams,  # noq
                                       ShuffleStrideType)
 
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per forward launch of the default workload (tile_m = 64), from two rocprofv3 --pmc runs
-# (FETCH_SIZE scaled by the factor 2.000 a copy kernel of known size gives on this part, plus
-# WRITE_SIZE): 2.000 * 16854.4 KiB + 15057.1 KiB.  The counter runs are offline; this is their result.
-MEASURED_TRAFFIC_BYTES = 49936282
+# The HBM traffic counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) are taken in runs of their own;
+# their result lives in this summary, on a line that also carries a hash of the kernel's sources.
+TRAFFIC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                               "rowgemm_lds_f16_subm_c64_fwd.md")
+KERNEL_SOURCES = ("rowgemm_lds.h", "rowgemm.h", "lds_dma.h", "common.h", "rowgemm_inst.hip")
+
+
+def kernel_source_hash():
+    """sha256 (16 hex digits) over the sources of the forward kernel."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "cumm_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(tile_m):
+    """(bytes per launch, note) from the line ``TRAFFIC tile_m=64 fetch_kib=.. write_kib=.. fetch_factor=..
+    write_factor=.. sources=<hash>`` of the counter summary; None when the kernel's sources have
+    changed since the counters were taken (the figure would describe another kernel)."""
+    try:
+        text = open(TRAFFIC_SUMMARY).read()
+    except OSError:
+        return None, "no counter summary"
+    for m in re.finditer(r"^TRAFFIC (.*)$", text, flags=re.M):
+        kv = dict(item.split("=", 1) for item in m.group(1).split())
+        if int(kv.get("tile_m", -1)) != tile_m:
+            continue
+        if kv.get("sources") != kernel_source_hash():
+            return None, "counters were taken on other kernel sources (%s, now %s)" % (kv.get("sources"), kernel_source_hash())
+        kib = float(kv["fetch_factor"]) * float(kv["fetch_kib"]) + float(kv["write_factor"]) * float(kv["write_kib"])
+        return int(round(kib * 1024)), "profiles/" + os.path.basename(TRAFFIC_SUMMARY)
+    return None, "no counters for this tile"
 PEAK_MFMA_F16_TFLOPS = 2516.6
 PEAK_MFMA_I8_TOPS = 5033.2
 GRID = (41, 1600, 1408)
@@ -351,6 +381,33 @@ def bench_stack(args):
     return res
 
 
+def bench_native(args, coords):
+    """Kernel volume 125 (5 x 5 x 5 submanifold, no 32-bit masks) through the per-offset path on the
+    headline voxel set: pair tables and per-offset lists on the GPU, then forward = 125 gather-GEMM-
+    scatter launches into an fp32 image + one finishing pass."""
+    from cumm_amd.conv import native
+    n, c = int(coords.shape[0]), 64
+    rngn = np.random.default_rng(SEED + 9)
+    d_coords = dev(np.ascontiguousarray(coords, np.int32))
+    t0 = time.perf_counter()
+    table = pairs.subm_pairs_device(d_coords, GRID, ksize=(5, 5, 5))
+    lists = pairs.pair_lists_device(table.indices_fwd)
+    prep_ms = (time.perf_counter() - t0) * 1e3
+    P = int(lists.counts.sum())
+    x = dev(rngn.normal(0, 1, size=(n, c)).astype(np.float16))
+    w = dev(rngn.normal(0, 0.03, size=(c, 125, c)).astype(np.float16))
+    out, acc = tv.zeros([n, c], tv.float16, 0), tv.zeros([n, c], tv.float32, 0)
+    steps = max(3, args.steps // 20)
+    wms, ems = timed(lambda: native.forward(x, w, out, lists, acc=acc), steps, 2)
+    # what this algorithm has to move: per pair one input row, one fp32 accumulator row read and
+    # written, two indices; the image zeroed, read once more and the result written
+    alg = P * (c * 2 + 2 * c * 4 + 8) + n * c * (4 + 4 + 2) + 125 * c * c * 2
+    return {"voxels": n, "kernel_volume": 125, "active_pairs": P, "input_preparation_first_call_ms": round(prep_ms, 3),
+            "forward_ms": round(wms, 4), "kernel_ms_events": round(ems, 4),
+            "tflops": round(2.0 * P * c * c / (wms * 1e-3) / 1e12, 2),
+            "hbm_frac": round(alg / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "launches": int((lists.counts > 0).sum()) + 2}
+
+
 def bench_dense_gemm(args):
     """Plain matmul2, 4096^3 f16 (the only MFMA-bound shape of the path)."""
     rng3 = np.random.default_rng(SEED + 3)
@@ -471,11 +528,15 @@ def main():
     ap.add_argument("--tile-m", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the s8 / backward legs")
-    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs,gather,tuner,stack")
+    ap.add_argument("--extra-only", default="", help="comma list of extra legs to run: dgrad,wgrad,s8,gather_gemm,dense_gemm,pairs,gather,tuner,stack,native")
+    ap.add_argument("--source-hash", action="store_true", help="print the hash of the forward kernel's sources and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on 512 MiB (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
     args = ap.parse_args()
+    if args.source_hash:
+        print(kernel_source_hash())
+        return 0
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)",
               file=sys.stderr)
@@ -541,14 +602,14 @@ def main():
         "kernel_ms_events": round(ev_ms, 5),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved_gbs / PEAK_HBM_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES if tile_m == 64 else None,
+                     "traffic": measured_traffic(tile_m)[0], "traffic_source": measured_traffic(tile_m)[1],
                      "algorithmic_bytes": alg_bytes},
     }
 
     if not args.no_extra:
         extra = {}
         legs = (set(args.extra_only.split(",")) if args.extra_only
-                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather", "tuner", "stack"})
+                else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather", "tuner", "stack", "native"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)
         dout = dev(rng.normal(0, 1, size=(n, K)).astype(np.float16))
         if "dgrad" in legs:
@@ -568,6 +629,8 @@ def main():
             extra["gather_scatter_rows"] = bench_gather_scatter(args)
         if "stack" in legs:
             extra["bf16_stack_1m"] = bench_stack(args)
+        if "native" in legs:
+            extra["native_subm_5x5x5_f16"] = bench_native(args, coords)
         if "tuner" in legs:
             # the timing-based descriptor choice on the headline problem (after the timed region)
             from cumm_amd import tuner

@@ -797,7 +797,12 @@ int cumm_hip_device_synchronize(void) {
 }
 int cumm_hip_take_async_errors(int32_t *split_k_timeouts) {
   if (!split_k_timeouts) return fail(CUMM_HIP_EINVAL, "null out-param");
-  return take_async_errors(split_k_timeouts);
+  int32_t sort_give_ups = 0;
+  if (int rc = take_async_errors(split_k_timeouts, &sort_give_ups)) return rc;
+  if (sort_give_ups != 0)
+    return fail(CUMM_HIP_ERUNTIME, "mask sort: %d look-back(s) gave up waiting for an earlier chunk; the result of that "
+                "sort is invalid", (int)sort_give_ups);
+  return CUMM_HIP_OK;
 }
 int cumm_hip_set_split_k_spin_limit(int polls) {
   if (polls < 0) return fail(CUMM_HIP_EINVAL, "the number of polls must not be negative (0 = the default)");

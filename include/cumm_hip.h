@@ -189,7 +189,9 @@ int cumm_hip_stream_destroy(void *stream);
 int cumm_hip_stream_synchronize(void *stream);
 int cumm_hip_device_synchronize(void);
 /* The same count for callers that synchronise by other means (e.g. through torch): reads and
- * clears the current device's count of timed-out split-K slices.  Call after a synchronisation. */
+ * clears the current device's count of timed-out split-K slices.  Call after a synchronisation.
+ * A mask sort whose look-back gave up since the last report (cumm_hip_sort_by_mask) makes the call
+ * return CUMM_HIP_ERUNTIME, with the count of slices still written. */
 int cumm_hip_take_async_errors(int32_t *split_k_timeouts);   /* host out-param */
 /* Polls a split-K slice makes before it gives up (0 = the default of 2^24, about a second).  For
  * tests of the time-out path and for workloads with very long slices. */
