@@ -128,8 +128,9 @@ def bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops):
             "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3)}
 
 
-def bench_wgrad(args, p, dout, n, C, K, tile_m, flops, parallel):
+def bench_wgrad(args, p, dout, n, C, K, tile_m, flops, parallel, fixed_order=False):
     pw = ConvParams(3, ConvOpType.BackwardWeight)
+    pw.deterministic = fixed_order
     pw.conv_algo_desp = find_desp(tv.float16, ConvOpType.BackwardWeight, 64, 64, parallel=parallel)
     pw.input, pw.output = p.input, dout
     pw.weight = tv.zeros([K, 27, C], tv.float16, 0)
@@ -280,6 +281,10 @@ def bench_stack(args):
     pw.indices, pw.mask, pw.mask_argsort = table.indices_fwd, red, order_tv
     pw.mask_width, pw.split_k_slices = 64, 32
     wms, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), steps, warm)
+    pw.deterministic, pw.workspace = True, tv.Tensor()
+    wms_fixed, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), steps, warm)
+    pw.deterministic, pw.workspace = False, tv.Tensor()
+    res["subm_c128_backward_weight_fixed_order"] = {"ms_per_step": round(wms_fixed, 5)}
     res["subm_c128_backward_weight_balanced"] = {"ms_per_step": round(wms, 5),
                                                  "tflops": round(2.0 * pairs1 * c * c / (wms * 1e-3) / 1e12, 2)}
     p2 = ConvParams(3, ConvOpType.Forward)
@@ -309,6 +314,10 @@ def bench_stack(args):
     pw2.indices, pw2.mask, pw2.mask_argsort = table2.indices_fwd, red2, order2_tv
     pw2.mask_width, pw2.split_k_slices = 64, 32
     wms, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw2), steps, warm)
+    pw2.deterministic, pw2.workspace = True, tv.Tensor()
+    wms_fixed, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw2), steps, warm)
+    pw2.deterministic, pw2.workspace = False, tv.Tensor()
+    res["stride2_c128_c256_backward_weight_fixed_order"] = {"ms_per_step": round(wms_fixed, 5)}
     res["stride2_c128_c256_backward_weight_balanced"] = {
         "ms_per_step": round(wms, 5), "tflops": round(2.0 * pairs2 * c * 256 / (wms * 1e-3) / 1e12, 2)}
 
@@ -398,14 +407,15 @@ def bench_native(args, coords):
     w = dev(rngn.normal(0, 0.03, size=(c, 125, c)).astype(np.float16))
     out, acc = tv.zeros([n, c], tv.float16, 0), tv.zeros([n, c], tv.float32, 0)
     steps = max(3, args.steps // 20)
-    wms, ems = timed(lambda: native.forward(x, w, out, lists, acc=acc), steps, 2)
+    plan = native.plan_forward(x, w, out, lists, acc=acc)   # validated once, as a layer with a fixed geometry would
+    wms, ems = timed(plan, steps, 2)
     # what this algorithm has to move: per pair one input row, one fp32 accumulator row read and
     # written, two indices; the image zeroed, read once more and the result written
     alg = P * (c * 2 + 2 * c * 4 + 8) + n * c * (4 + 4 + 2) + 125 * c * c * 2
     return {"voxels": n, "kernel_volume": 125, "active_pairs": P, "input_preparation_first_call_ms": round(prep_ms, 3),
             "forward_ms": round(wms, 4), "kernel_ms_events": round(ems, 4),
             "tflops": round(2.0 * P * c * c / (wms * 1e-3) / 1e12, 2),
-            "hbm_frac": round(alg / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "launches": int((lists.counts > 0).sum()) + 2}
+            "hbm_frac": round(alg / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "launches": plan.launches}
 
 
 def bench_dense_gemm(args):
@@ -616,6 +626,7 @@ def main():
             extra["subm_f16_dgrad"] = bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops)
         if "wgrad" in legs:
             extra["subm_f16_wgrad_balanced_atomic"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops, True)
+            extra["subm_f16_wgrad_balanced_fixed_order"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops, True, True)
             extra["subm_f16_wgrad_serial_splitk32"] = bench_wgrad(args, p, dout, n, C, K, tile_m, flops, False)
         if "s8" in legs:
             extra["sparseconv_s8_stride2"] = bench_s8(args, tile_m)

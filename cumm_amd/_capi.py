@@ -54,7 +54,7 @@ class SparseConvArgs(C.Structure):
                 ("mask_width", C.c_int32),
                 ("ndim", C.c_int32), ("N", C.c_int32), ("C", C.c_int32), ("K", C.c_int32),
                 ("kernel_volume", C.c_int32), ("mode", C.c_int32), ("groups", C.c_int32),
-                ("d_is_bias", C.c_int32),
+                ("d_is_bias", C.c_int32), ("deterministic", C.c_int32),
                 ("bias_pointer", C.c_void_p), ("scale_pointer", C.c_void_p),
                 ("rows_in", C.c_int32), ("rows_out", C.c_int32)]
 
@@ -67,6 +67,7 @@ SYMBOLS = {
     "cumm_hip_sparse_conv_static_ws": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(SparseConvArgs), _VP]),
     "cumm_hip_query_gemm_workspace": (C.c_int64, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.c_int]),
     "cumm_hip_query_conv_workspace": (C.c_int64, [C.POINTER(ConvDesc), C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "cumm_hip_query_wgrad_ordered_workspace": (C.c_int64, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "cumm_hip_list_gemm_algos": (C.c_int, [C.POINTER(GemmDesc), C.c_int]),
     "cumm_hip_list_conv_algos": (C.c_int, [C.POINTER(ConvDesc), C.c_int]),
     "cumm_hip_gemm_supported": (C.c_int, [C.POINTER(GemmDesc)]),

@@ -181,6 +181,13 @@ class ConvMainUnitTest:
 
         workspace_size = desp.query_conv_workspace_size(mnk[0], mnk[1], mnk[2], split_k_slices,
                                                         kernel_volume)
+        ordered = bool(getattr(params, "deterministic", False)) and op_type == ConvOpType.BackwardWeight \
+            and desp.split_k_parallel and split_k_slices > 1
+        if ordered and params.workspace.empty():
+            # the fixed-order variant keeps one partial block per workgroup: sized by the library
+            workspace_size = int(_capi.lib().cumm_hip_query_wgrad_ordered_workspace(N, C, K, kernel_volume, mask_width))
+            if workspace_size < 0:
+                raise ValueError("the fixed-order backward-weight does not take these sizes")
         if static_ws:
             workspace = Tensor()
         else:
@@ -217,6 +224,7 @@ class ConvMainUnitTest:
         args.kernel_volume = kernel_volume
         args.mode, args.groups = 1, 1      # ConvMode.CrossCorrelation, ungrouped: all the reference's mask kernels do
         args.d_is_bias = int(not bias.empty())
+        args.deterministic = int(ordered)
         args.bias_pointer = _ptr(bias)
         args.scale_pointer = _ptr(scale)
         args.rows_in, args.rows_out = inp.dim(0), output.dim(0)

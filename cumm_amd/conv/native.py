@@ -25,14 +25,22 @@ from ..gemm.main import GemmMainUnitTest
 from ..tensorview.gemm import Activation, GemmParams, ShuffleStrideType
 
 
+_FOUND = {}
+
+
 def _find(dtype: int, dtype_c: int, shuffle: ShuffleStrideType, tile_m: int, tile_n: int, trans_a: bool,
           trans_b: bool):
-    for d in _descs():
-        if (d.dtype_a == dtype and d.dtype_c == dtype_c and d.shuffle_type == shuffle and
-                d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and d.trans_a == trans_a and
-                d.trans_b == trans_b and not d.trans_c):
-            return d
-    raise RuntimeError("can't find any suitable algo for your parameters.")
+    key = (dtype, dtype_c, shuffle, tile_m, tile_n, trans_a, trans_b)
+    if key not in _FOUND:
+        for d in _descs():
+            if (d.dtype_a == dtype and d.dtype_c == dtype_c and d.shuffle_type == shuffle and
+                    d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and d.trans_a == trans_a and
+                    d.trans_b == trans_b and not d.trans_c):
+                _FOUND[key] = d
+                break
+        else:
+            raise RuntimeError("can't find any suitable algo for your parameters.")
+    return _FOUND[key]
 
 
 _DESCS = None
@@ -58,10 +66,11 @@ def _check(inp, weight, lists, n_rows_out):
     return kv
 
 
-def _accumulate(a, a_inds_all, c_inds_all, counts, weight, acc, trans_b, stream):
-    """acc[c_inds[k]] += a[a_inds[k]] @ op(W[:, k, :]) for every offset with pairs."""
+def _accumulate_steps(a, a_inds_all, c_inds_all, counts, weight, acc, trans_b, stream):
+    """One validated ``GemmParams`` per offset with pairs: acc[c_inds[k]] += a[a_inds[k]] @ op(W[:, k, :])."""
     kv = weight.dim(1)
     n_ch = acc.dim(1)
+    steps = []
     for k in range(kv):
         cnt = int(counts[k])
         if cnt == 0:
@@ -75,7 +84,8 @@ def _accumulate(a, a_inds_all, c_inds_all, counts, weight, acc, trans_b, stream)
         p.c_inds = c_inds_all.select(0, k).slice_first_axis(0, cnt)
         p.alpha, p.beta = 1.0, 1.0
         p.stream = stream
-        GemmMainUnitTest.matmul2(p)
+        steps.append(p)
+    return steps
 
 
 def _finish(out, acc, bias, act_type, act_alpha, stream):
@@ -85,40 +95,73 @@ def _finish(out, acc, bias, act_type, act_alpha, stream):
         float(act_alpha), stream))
 
 
-def _fp32_image(rows, channels, acc, stream):
+def _fp32_image(rows, channels, acc):
     if acc is None or acc.empty():
         acc = tv.empty([rows, channels], tv.float32, 0)
     elif acc.dtype != tv.float32 or acc.shape != [rows, channels] or acc.device < 0:
         raise RuntimeError("acc must be a device float32 tensor [%d, %d]" % (rows, channels))
-    ctx = tv.Context()
-    ctx.set_cuda_stream(stream)
-    acc.zero_(ctx)
     return acc
+
+
+class _Plan:
+    """The launches of one pass over fixed tensors and pair lists: built (and validated) once, run
+    any number of times - a repeat run goes straight to the C entry points with the argument blocks
+    of the first one.  The plan keeps its tensors alive."""
+
+    def __init__(self, out, acc, steps, bias, act_type, act_alpha, stream):
+        self.out, self.acc, self.steps = out, acc, steps
+        self.bias, self.act_type, self.act_alpha, self.stream = bias, act_type, act_alpha, stream
+        self._ctx = tv.Context()
+        self._ctx.set_cuda_stream(stream)
+
+    def __call__(self) -> None:
+        self.acc.zero_(self._ctx)
+        for p in self.steps:
+            GemmMainUnitTest.matmul2(p)
+        _finish(self.out, self.acc, self.bias, self.act_type, self.act_alpha, self.stream)
+
+    @property
+    def launches(self) -> int:
+        return len(self.steps) + 2
+
+
+def plan_forward(inp: tv.Tensor, weight: tv.Tensor, output: tv.Tensor, lists, *, bias: Optional[tv.Tensor] = None,
+                 act_type=Activation.None_, act_alpha: float = 0.0, stream: int = 0,
+                 acc: Optional[tv.Tensor] = None) -> _Plan:
+    """The forward pass as a reusable plan (``plan()`` runs it): for a layer whose tensors and
+    geometry stay in place from call to call."""
+    _check(inp, weight, lists, output.dim(0))
+    if output.ndim != 2 or output.dim(1) != weight.dim(0) or output.dtype != inp.dtype or weight.dim(2) != inp.dim(1):
+        raise RuntimeError("error")
+    acc = _fp32_image(output.dim(0), output.dim(1), acc)
+    # W[:, k, :] is [K, C]: B stored [n, k]
+    steps = _accumulate_steps(inp, lists.pair_in, lists.pair_out, lists.counts, weight, acc, True, stream)
+    return _Plan(output, acc, steps, bias, act_type, act_alpha, stream)
+
+
+def plan_backward_input(dout: tv.Tensor, weight: tv.Tensor, dinp: tv.Tensor, lists, *, stream: int = 0,
+                        acc: Optional[tv.Tensor] = None) -> _Plan:
+    _check(dout, weight, lists, dinp.dim(0))
+    if dinp.ndim != 2 or dinp.dim(1) != weight.dim(2) or dout.dim(1) != weight.dim(0) or dinp.dtype != dout.dtype:
+        raise RuntimeError("error")
+    acc = _fp32_image(dinp.dim(0), dinp.dim(1), acc)
+    # W[:, k, :] is [K, C] with K the contraction: B stored [k, n]
+    steps = _accumulate_steps(dout, lists.pair_out, lists.pair_in, lists.counts, weight, acc, False, stream)
+    return _Plan(dinp, acc, steps, None, Activation.None_, 0.0, stream)
 
 
 def forward(inp: tv.Tensor, weight: tv.Tensor, output: tv.Tensor, lists, *, bias: Optional[tv.Tensor] = None,
             act_type=Activation.None_, act_alpha: float = 0.0, stream: int = 0, acc: Optional[tv.Tensor] = None) -> None:
     """output [N_out, K] = act(sum over offsets + bias); ``lists`` from ``pairs.pair_lists_device``
     on the forward table; ``acc``: an fp32 [N_out, K] device tensor to reuse as the image."""
-    _check(inp, weight, lists, output.dim(0))
-    if output.ndim != 2 or output.dim(1) != weight.dim(0) or output.dtype != inp.dtype or weight.dim(2) != inp.dim(1):
-        raise RuntimeError("error")
-    acc = _fp32_image(output.dim(0), output.dim(1), acc, stream)
-    # W[:, k, :] is [K, C]: B stored [n, k]
-    _accumulate(inp, lists.pair_in, lists.pair_out, lists.counts, weight, acc, True, stream)
-    _finish(output, acc, bias, act_type, act_alpha, stream)
+    plan_forward(inp, weight, output, lists, bias=bias, act_type=act_type, act_alpha=act_alpha, stream=stream,
+                 acc=acc)()
 
 
 def backward_input(dout: tv.Tensor, weight: tv.Tensor, dinp: tv.Tensor, lists, *, stream: int = 0,
                    acc: Optional[tv.Tensor] = None) -> None:
     """dinp [N_in, C] = sum over offsets of dout[pair_out[k]] @ W[:, k, :] scattered to pair_in[k]."""
-    _check(dout, weight, lists, dinp.dim(0))
-    if dinp.ndim != 2 or dinp.dim(1) != weight.dim(2) or dout.dim(1) != weight.dim(0) or dinp.dtype != dout.dtype:
-        raise RuntimeError("error")
-    acc = _fp32_image(dinp.dim(0), dinp.dim(1), acc, stream)
-    # W[:, k, :] is [K, C] with K the contraction: B stored [k, n]
-    _accumulate(dout, lists.pair_out, lists.pair_in, lists.counts, weight, acc, False, stream)
-    _finish(dinp, acc, None, Activation.None_, 0.0, stream)
+    plan_backward_input(dout, weight, dinp, lists, stream=stream, acc=acc)()
 
 
 _NO_PAIR = {}

@@ -278,6 +278,29 @@ int report_async_errors() {
 int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a, void *stream_, void *workspace,
                      size_t workspace_bytes, size_t workspace_cap);
 
+// workspace of the fixed-order backward-weight: live-tile counts (128 bytes), the table of the
+// workgroups per (offset, channel block), the live-tile lists, then the slots of partial sums
+struct OrderedLayout {
+  bool wide;
+  int num_red, kblocks, cblocks, combos, keys;
+  int64_t max_units;
+  size_t block_bytes, lists_at, slots_at;
+};
+OrderedLayout ordered_layout(int N, int C, int K, int kv, int mask_width) {
+  OrderedLayout l;
+  l.wide = K > 64 && C > 64;
+  const int blk = l.wide ? 128 : 64;
+  l.num_red = (N + mask_width - 1) / mask_width;
+  l.kblocks = (K + blk - 1) / blk; l.cblocks = (C + blk - 1) / blk;
+  l.combos = l.kblocks * l.cblocks; l.keys = kv * l.combos;
+  const int qt = kWgradMaxPos / mask_width < 1 ? 1 : kWgradMaxPos / mask_width;
+  l.max_units = ((int64_t)((l.num_red + qt - 1) / qt) * kv + kv) * l.combos;
+  l.block_bytes = sizeof(float) * blk * blk;
+  l.lists_at = 128 + (((size_t)8 * l.keys + 255) & ~(size_t)255);
+  l.slots_at = l.lists_at + ((sizeof(int32_t) * (size_t)kv * l.num_red + 255) & ~(size_t)255);
+  return l;
+}
+
 }  // namespace
 
 extern "C" {
@@ -313,6 +336,14 @@ int64_t cumm_hip_query_conv_workspace(const CummHipConvDesc *desc, int m, int n,
   if (d.split_k_serial) return (int64_t)sizeof(int32_t) * tiles_m * tiles_n;
   if (d.split_k_parallel) return (int64_t)4 * m * n * split_k_slices;
   return -1;
+}
+int64_t cumm_hip_query_wgrad_ordered_workspace(int N, int C, int K, int kernel_volume, int mask_width) {
+  if (N < 0 || C <= 0 || K <= 0 || kernel_volume <= 0 || kernel_volume > 32 || mask_width <= 0 || mask_width > kWgradMaxPos)
+    return -1;
+  const OrderedLayout l = ordered_layout(N, C, K, kernel_volume, mask_width);
+  // 512 workgroups: two per compute unit of a 256-unit part (fewer slots only mean fewer workgroups)
+  const int64_t wgs = l.max_units < 512 ? l.max_units : 512;
+  return (int64_t)l.slots_at + (wgs + l.keys) * (int64_t)l.block_bytes;
 }
 
 int cumm_hip_list_gemm_algos(CummHipGemmDesc *out, int cap) {
@@ -626,6 +657,74 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
   // backward weight: dW[K, kv, C]; A = dOut [N, K], B = input [*, C]
   const int tm = d.tile_shape[0], tn = d.tile_shape[1], tk = d.tile_shape[2];
   if (a->mask_width <= 0 || a->mask_width % tk) return fail(CUMM_HIP_ERUNTIME, "mask_width must be a positive multiple of tile k");
+  if (fam == 3 && a->deterministic && !(a->split_k_slices > 1 && a->mask_width <= kWgradMaxPos))
+    return fail(CUMM_HIP_EINVAL, "the fixed-order backward-weight needs split_k_slices > 1 and mask_width <= %d", kWgradMaxPos);
+  // The fixed-order variant (partial sums in slots, added up in a fixed order, see
+  // WgradParams::key_range) runs when the caller asks for it, and by itself where it is also the
+  // faster one: with many more units than resident workgroups a workgroup carries its sum through
+  // its run of units in registers instead of adding every unit's block into the image with atomics
+  // (0.25 against 0.29 ms for C = K = 128 at 1 M voxels) - if the workspace has room for all of its
+  // workgroups.
+  bool ordered = fam == 3 && a->deterministic;
+  if (fam == 3 && a->split_k_slices > 1 && a->mask_width <= kWgradMaxPos) {
+    const OrderedLayout lay = ordered_layout(a->N, a->C, a->K, kv, a->mask_width);
+    const int qt = kWgradMaxPos / a->mask_width < 1 ? 1 : kWgradMaxPos / a->mask_width;
+    const bool fits32 = (int64_t)a->rows_out * a->K * 2 < (int64_t)1 << 31 && (int64_t)a->rows_in * a->C * 2 < (int64_t)1 << 31 &&
+                        (int64_t)kv * a->N * 4 < (int64_t)1 << 31;
+    const int64_t unit_bound = ((int64_t)(lay.num_red + qt - 1) / qt + 1) * kv * (((int64_t)a->K + 63) / 64) * (((int64_t)a->C + 63) / 64);
+    const bool size_ok = fits32 && unit_bound < ((int64_t)1 << 22) && lay.num_red < (1 << 22);
+    const bool aligned = (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0;
+    if (ordered && !size_ok)
+      return fail(CUMM_HIP_EINVAL, "the fixed-order backward-weight does not take a problem of this size; use a split_k_serial descriptor");
+    if (ordered && !aligned) return fail(CUMM_HIP_EINVAL, "workspace must be 256-byte aligned");
+    int64_t wgs = 0;
+    if (size_ok && aligned) {
+      const int resident = dt == CUMM_HIP_F16 ? wgrad_ordered_resident_f16(lay.wide) : wgrad_ordered_resident_bf16(lay.wide);
+      if (resident < 1) return hip_fail(hipGetLastError(), "occupancy query");
+      const int64_t full = resident < lay.max_units ? resident : lay.max_units;
+      wgs = full;
+      const int64_t have = workspace && workspace_bytes > lay.slots_at ? (int64_t)((workspace_bytes - lay.slots_at) / lay.block_bytes) : 0;
+      if (have - lay.keys + 1 < wgs) wgs = have - lay.keys + 1;
+      const int64_t by_descriptor = (((int64_t)1 << 32) - 1) / (int64_t)lay.block_bytes - lay.keys + 1;
+      if (by_descriptor < wgs) wgs = by_descriptor;
+      if (!ordered && wgs == full && (lay.num_red + qt - 1) / qt >= resident) ordered = true;
+    }
+    const size_t least = lay.slots_at + (size_t)lay.keys * lay.block_bytes;
+    if (ordered && workspace_cap && least > workspace_cap)
+      return fail(CUMM_HIP_EINVAL, "this problem needs %zu bytes of workspace, the static one holds %zu", least, workspace_cap);
+    if (ordered && wgs < 1) return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", least);
+    if (ordered) {
+    char *base = reinterpret_cast<char *>(workspace);
+    WgradParams w;
+    std::memset(&w, 0, sizeof(w));
+    w.dout = a->ptr_A; w.inp = a->ptr_B; w.scratch = reinterpret_cast<float *>(base + lay.slots_at);
+    w.argsort = a->mask_argsort_ptr; w.indices = a->indice_ptr; w.red_mask = a->mask_ptr;
+    w.num_red = lay.num_red; w.mask_width = a->mask_width; w.mask_filter = a->mask_filter;
+    w.n_pos = a->N; w.n_idx = a->N; w.rows_x = a->rows_in; w.rows_y = a->rows_out;
+    w.K = a->K; w.C = a->C; w.kv = kv; w.tiles_per_wg = qt;
+    w.images = 1;
+    w.live_cnt = reinterpret_cast<int32_t *>(base);
+    w.key_range = reinterpret_cast<int32_t *>(base + 128);
+    w.live_list = reinterpret_cast<int32_t *>(base + lay.lists_at);
+    WgradPrepareParams pre;
+    std::memset(&pre, 0, sizeof(pre));
+    pre.red_mask = w.red_mask; pre.num_red = w.num_red; pre.kv = kv; pre.mask_filter = w.mask_filter;
+    pre.live_cnt = reinterpret_cast<int32_t *>(base);
+    pre.live_list = reinterpret_cast<int32_t *>(base + lay.lists_at);
+    WgradOrderedParams f;
+    std::memset(&f, 0, sizeof(f));
+    f.slots = w.scratch; f.key_range = w.key_range; f.dw = a->ptr_C; f.src = ptr_D;
+    f.total = (int64_t)a->K * kv * a->C; f.K = a->K; f.C = a->C; f.kv = kv;
+    f.block_k = f.block_c = lay.wide ? 128 : 64;
+    f.cblocks = lay.cblocks; f.per_r = lay.combos;
+    f.mask_filter = a->mask_filter; f.alpha = a->alpha; f.beta = a->beta;
+    f.slots_bytes = (uint32_t)((wgs + lay.keys - 1) * (int64_t)lay.block_bytes);
+    hipError_t e = dt == CUMM_HIP_F16 ? launch_wgrad_ordered_f16(w, pre, f, lay.wide, (int)wgs, stream)
+                                      : launch_wgrad_ordered_bf16(w, pre, f, lay.wide, (int)wgs, stream);
+    if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
+    return CUMM_HIP_OK;
+    }
+  }
   if (fam == 3 && a->split_k_slices > 1 && a->mask_width <= kWgradMaxPos) {
     const size_t need = sizeof(float) * (size_t)a->K * kv * a->C;
     if (workspace_cap && need > workspace_cap)

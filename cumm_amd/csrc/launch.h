@@ -34,6 +34,10 @@ hipError_t launch_tilegemm_wide_s8(int tm, int tn, bool xk, bool yk, const TileG
 // balanced backward-weight with fp32 atomics: main kernel then finalize (f16 / bf16 only)
 hipError_t launch_wgrad_atomic_f16(const WgradParams &p, const WgradPrepareParams &pre, const WgradFinalizeParams &f, hipStream_t s);
 hipError_t launch_wgrad_atomic_bf16(const WgradParams &p, const WgradPrepareParams &pre, const WgradFinalizeParams &f, hipStream_t s);
+int wgrad_ordered_resident_f16(bool wide);
+int wgrad_ordered_resident_bf16(bool wide);
+hipError_t launch_wgrad_ordered_f16(const WgradParams &p, const WgradPrepareParams &pre, const WgradOrderedParams &f, bool wide, int wgs, hipStream_t s);
+hipError_t launch_wgrad_ordered_bf16(const WgradParams &p, const WgradPrepareParams &pre, const WgradOrderedParams &f, bool wide, int wgs, hipStream_t s);
 
 // tile shapes the tables above hold
 inline bool rowgemm_has_tile(int tm, int tn) {

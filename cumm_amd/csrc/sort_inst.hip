@@ -129,6 +129,21 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   const int chunk = chunk_of_block;
   if (chunk >= p.chunks) return;   // (never: the grid has one workgroup per chunk)
 
+  // A digit that is the same in every key (the bits of a 32-bit filter above the kernel volume;
+  // any pass of an input with one mask value) leaves the order as it is: the chunk is copied
+  // through, without ranks and without waiting for anybody.
+  if (__syncthreads_or(total_of_bin == (uint32_t)p.n)) {
+#pragma unroll
+    for (int u = 0; u < kItems; ++u) {
+      const int64_t pos = (int64_t)chunk * kChunk + u * kSortThreads + t;
+      if (pos < p.n) {
+        p.dst_keys[pos] = p.pass == 0 ? (p.mask[pos] & p.filter) : p.src_keys[pos];
+        p.dst_vals[pos] = p.pass == 0 ? (int32_t)pos : p.src_vals[pos];
+      }
+    }
+    return;
+  }
+
   // ---- keys of this chunk, wave-striped: wave w owns positions [base_w, base_w + 64 * kItems),
   // item u of lane l is position base_w + u * 64 + l, i.e. position order = (u, l)
   const int64_t base_w = (int64_t)chunk * kChunk + (int64_t)wave * (64 * kItems);

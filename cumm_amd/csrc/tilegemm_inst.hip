@@ -128,6 +128,41 @@ hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const
   hipLaunchKernelGGL((wgrad_finalize_kernel<T>), dim3((unsigned)((f.total / 4 + 255) / 256)), dim3(256), 0, s, f);
   return hipGetLastError();
 }
+
+// Fixed-order variant: the same units, a contiguous run per workgroup, partial sums stored into
+// slots and added up in workgroup order.  `max_wgs` = workgroups the caller's slots allow.
+int CUMM_CAT(wgrad_ordered_resident_, CUMM_NAME)(bool wide) {
+  using T = CUMM_ELEM;
+  static int resident_of[2][16] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  int &resident = resident_of[wide ? 1 : 0][dev & 15];
+  if (resident == 0) {
+    int cus = 0, per_cu = 0;
+    hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess)
+      e = wide ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wgrad_units_kernel<T, 2, 2, 1, true>, 256, 0)
+               : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wgrad_units_kernel<T, 1, 1, 2, true>, 256, 0);
+    if (e != hipSuccess) return 0;
+    resident = cus * per_cu > 0 ? cus * per_cu : 1;
+  }
+  return resident;
+}
+
+hipError_t CUMM_CAT(launch_wgrad_ordered_, CUMM_NAME)(const WgradParams &p, const WgradPrepareParams &pre,
+                                                      const WgradOrderedParams &f, bool wide, int wgs, hipStream_t s) {
+  using T = CUMM_ELEM;
+  if (p.num_red == 0 || p.kv == 0 || wgs < 1) return hipSuccess;
+  hipLaunchKernelGGL(wgrad_prepare_kernel, dim3(p.kv), dim3(256), 0, s, pre);   // lists only: no image to zero
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  if (wide) hipLaunchKernelGGL((wgrad_units_kernel<T, 2, 2, 1, true>), dim3(wgs), dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((wgrad_units_kernel<T, 1, 1, 2, true>), dim3(wgs), dim3(256), 0, s, p);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL((wgrad_finalize_ordered_kernel<T>), dim3((unsigned)((f.total / 4 + 31) / 32)), dim3(256), 0, s, f);
+  return hipGetLastError();
+}
 #endif
 
 }  // namespace cummhip

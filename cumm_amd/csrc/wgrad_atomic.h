@@ -21,6 +21,10 @@
 //     every workgroup scans the reduced mask for its offset itself and surplus workgroups exit;
 //     rows pass through registers and are parked in LDS transposed with 16-bit stores.
 // The sum order is not fixed (fp32 atomics), the partial sums are never rounded to the weight type.
+//   * fixed-order variant (wgrad_units_kernel<..., true> + wgrad_finalize_ordered_kernel): the same
+//     units, but a workgroup walks a contiguous run of them, carries its accumulator from unit to
+//     unit of one (offset, channel block) and stores it into a slot of its own; the last kernel adds
+//     the slots of an element in workgroup order.  Same bits from run to run on one device.
 #pragma once
 #include "common.h"
 #include "lds_dma.h"
@@ -50,6 +54,12 @@ struct WgradParams {
   // one unit walks all 64 x 64 channel blocks of its positions in turn (the pair lists are made
   // once) instead of one block per unit; set by the launcher when the units are many anyway
   int32_t merge_blocks;
+  // fixed-order variant (wgrad_units_kernel<..., true>): workgroup b walks the units
+  // [b * q, (b + 1) * q) of the order (offset, channel block, share), keeps one accumulator while
+  // offset and channel block stay the same and stores it - plain stores, no atomics - into slot
+  // b + key (key = offset * channel blocks + channel block) of `scratch`; key_range[key] = {first
+  // workgroup, number of workgroups} tells wgrad_finalize_ordered_kernel which slots to sum.
+  int32_t *key_range;
 };
 
 constexpr int kWgradMaxPos = 1024;  // positions one workgroup handles at most (QT * mask_width)
@@ -299,7 +309,7 @@ __device__ __forceinline__ int wave_prefix_sum_dpp(int v) {
 // 64 x 64 block (four gathers of each pair at C = K = 128, where the launch is bound by that
 // traffic once dOut and In no longer fit the last-level cache); its stage holds 32 pairs (16 KB,
 // four stages, still two workgroups per CU) and a wave accumulates 64 x 64.
-template <class T, int KB, int CB, int H>
+template <class T, int KB, int CB, int H, bool DET = false>
 __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   using E = Elem<T>;
   constexpr int TK = 32 * H;          // pairs per step
@@ -321,8 +331,8 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   const int l16 = lane & 15, q = lane >> 4;
 
   const int kblocks = (p.K + 64 * KB - 1) / (64 * KB), cblocks = (p.C + 64 * CB - 1) / (64 * CB);
-  const int per_r = p.merge_blocks ? 1 : kblocks * cblocks;
-  const int combos = p.merge_blocks ? kblocks * cblocks : 1;
+  const int per_r = (!DET && p.merge_blocks) ? 1 : kblocks * cblocks;
+  const int combos = (!DET && p.merge_blocks) ? kblocks * cblocks : 1;
   // units of offset r: its workgroups (ceil(live / QT)) times the channel blocks.  Lane r of every
   // wave holds offset r's numbers (kv <= 32: one mask bit per offset); a prefix sum over the
   // lanes and a ballot locate a unit without a loop over memory.
@@ -376,13 +386,64 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   const int incl = wave_prefix_sum_dpp(my_units);
   const int total_units = __builtin_amdgcn_readlane(incl, 31);
 
-  for (int unit = blockIdx.x; unit < total_units; unit += gridDim.x) {
+  // fixed-order variant: a contiguous run of units per workgroup, and the table of the workgroups
+  // that hold a partial sum of each (offset, channel block)
+  const int run = DET ? (total_units + (int)gridDim.x - 1) / (int)gridDim.x : 1;
+  if constexpr (DET) {
+    if (blockIdx.x == 0) {
+      __shared__ int key_wgs[32], key_start[32];
+      if (tid < 32) {
+        key_wgs[tid] = my_wgs;
+        key_start[tid] = incl - my_units;
+      }
+      __syncthreads();
+      for (int key = tid; key < p.kv * per_r; key += 256) {
+        const int r = key / per_r, combo = key - r * per_r;
+        const int n = key_wgs[r], first = key_start[r] + combo * n;
+        p.key_range[2 * key] = n > 0 ? first / run : 0;
+        p.key_range[2 * key + 1] = n > 0 ? (first + n - 1) / run - first / run + 1 : 0;
+      }
+    }
+  }
+  v4f acc[NJ][NI];
+  int acc_key = -1;
+  auto store_acc = [&]() __attribute__((always_inline)) {
+    float *slot = p.scratch + (int64_t)((int)blockIdx.x + acc_key) * (64 * KB * 64 * CB);
+#pragma unroll
+    for (int i = 0; i < NJ; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j)
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+          slot[((wm * NJ + i) * 16 + 4 * q + x) * (64 * CB) + (wn * NI + j) * 16 + l16] = acc[i][j][x];
+  };
+  const int unit_begin = DET ? (int)blockIdx.x * run : (int)blockIdx.x;
+  const int unit_end = DET ? (unit_begin + run < total_units ? unit_begin + run : total_units) : total_units;
+  const int unit_step = DET ? 1 : (int)gridDim.x;
+
+  for (int unit = unit_begin; unit < unit_end; unit += unit_step) {
     const int r = __builtin_amdgcn_readfirstlane(__builtin_popcountll(__ballot(lane < 32 && incl <= unit)));
     const int u = unit - __builtin_amdgcn_readlane(incl - my_units, r);
     const int live = __builtin_amdgcn_readlane(my_live, r);
     const int n_wg = __builtin_amdgcn_readlane(my_wgs, r);
     int bx = u, cb = 0, kb = 0;
-    if (per_r > 1) {
+    if constexpr (DET) {
+      // units of an offset in the order (channel block, share): a workgroup's run stays on one
+      // accumulator for as long as possible
+      const int combo = fast_div(u, n_wg);
+      bx = u - combo * n_wg;
+      kb = fast_div(combo, cblocks);
+      cb = combo - kb * cblocks;
+      const int key = r * per_r + combo;
+      if (key != acc_key) {
+        if (acc_key >= 0) store_acc();
+        acc_key = key;
+#pragma unroll
+        for (int i = 0; i < NJ; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j) acc[i][j] = v4f{0, 0, 0, 0};
+      }
+    } else if (per_r > 1) {
       bx = fast_div(u, per_r);
       const int rest = u - bx * per_r;
       kb = fast_div(rest, cblocks);
@@ -515,11 +576,12 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
       }
     };
 
-    v4f acc[NJ][NI];
+    if constexpr (!DET) {
 #pragma unroll
-    for (int i = 0; i < NJ; ++i)
+      for (int i = 0; i < NJ; ++i)
 #pragma unroll
-      for (int j = 0; j < NI; ++j) acc[i][j] = v4f{0, 0, 0, 0};
+        for (int j = 0; j < NI; ++j) acc[i][j] = v4f{0, 0, 0, 0};
+    }
 
     wait_vmcnt<0>();   // the previous unit's atomics: from here on the counter holds ring loads only
     uint32_t yn[H][KB], xn[H][CB];
@@ -567,7 +629,7 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     // consecutive floats (one 64-byte segment per quarter).  Units that follow each other go to
     // different images, so that the many units of one offset do not all queue on the same
     // addresses.
-    if (n_steps > 0) {
+    if (!DET && n_steps > 0) {
       const int64_t ldn = (int64_t)p.kv * p.C;
       float *image = p.scratch + (int64_t)(unit % p.images) * p.image_floats;
 #pragma unroll
@@ -589,6 +651,9 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     lds_barrier();     // every wave is done with the ring before the next block's loads land in it
     }  // channel blocks
     __syncthreads();   // the LDS lists and the ring are rewritten by the next unit
+  }
+  if constexpr (DET) {
+    if (acc_key >= 0) store_acc();
   }
 }
 
@@ -634,6 +699,76 @@ __global__ __launch_bounds__(256) void wgrad_finalize_kernel(const WgradFinalize
   } else {
 #pragma unroll
     for (int x = 0; x < 4; ++x) out[x] = E::from_float(p.alpha * acc[x]);
+  }
+  *reinterpret_cast<v4h *>(reinterpret_cast<uint16_t *>(p.dw) + i) = out;
+}
+
+// dW = cvt(alpha * (sum of the slots of an element's (offset, channel block), in workgroup order) +
+// beta * src) for the fixed-order variant.  Eight lanes share four consecutive elements: lane g sums
+// the g-th eighth of the slots first to last, then the eight sums are combined pairwise (1, 2, 4
+// lanes apart): the shape of the sum depends on the number of slots only, so the result repeats bit
+// for bit from run to run.
+struct WgradOrderedParams {
+  const float *slots;
+  const int32_t *key_range;
+  void *dw;
+  const void *src;
+  int64_t total;        // K * kv * C
+  int32_t K, C, kv;
+  int32_t block_k, block_c;   // channels of a slot (64 or 128 each)
+  int32_t cblocks, per_r;
+  uint32_t mask_filter;
+  float alpha, beta;
+  uint32_t slots_bytes;
+};
+
+template <class T>
+__global__ __launch_bounds__(256) void wgrad_finalize_ordered_kernel(const WgradOrderedParams p) {
+  using E = Elem<T>;
+  const int g = threadIdx.x & 7;
+  const int64_t i = ((int64_t)blockIdx.x * 32 + (threadIdx.x >> 3)) * 4;
+  const bool in_range = i < p.total;
+  const int64_t ii = in_range ? i : 0;
+  const int nn = (int)(ii % p.C);
+  const int r = (int)((ii / p.C) % p.kv);
+  const int mm = (int)(ii / ((int64_t)p.C * p.kv));
+  const bool on = in_range && ((p.mask_filter >> r) & 1u);
+  const int kb = mm / p.block_k, cb = nn / p.block_c;
+  const int key = r * p.per_r + kb * p.cblocks + cb;
+  const int first = p.key_range[2 * key], count = on ? p.key_range[2 * key + 1] : 0;
+  const int64_t slot_floats = (int64_t)p.block_k * p.block_c;
+  const uint32_t within = (uint32_t)((mm - kb * p.block_k) * p.block_c + (nn - cb * p.block_c)) * 4u;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.slots), 0, (int)p.slots_bytes, 0x00020000);
+  const int share = (count + 7) >> 3;
+  const int lo = g * share, hi = lo + share < count ? lo + share : count;
+  v4f sum = v4f{0, 0, 0, 0};
+  for (int t0 = lo; t0 < hi; t0 += 8) {
+    v4f part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      part[u] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+          rs, t0 + u < hi ? (uint32_t)((int64_t)(first + key + t0 + u) * slot_floats * 4) + within : 0x80000000u, 0, 0));
+#pragma unroll
+    for (int u = 0; u < 8; ++u) sum += part[u];   // (a slot past the share arrives as +0)
+  }
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    float v = sum[x];
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    sum[x] = v;
+  }
+  if (!on || g != 0) return;
+  typedef uint16_t v4h __attribute__((ext_vector_type(4)));
+  v4h out;
+  if (p.beta != 0.0f) {
+    const v4h src = *reinterpret_cast<const v4h *>(reinterpret_cast<const uint16_t *>(p.src) + i);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) out[x] = E::from_float(__builtin_fmaf(p.alpha, sum[x], p.beta * E::to_float(src[x])));
+  } else {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) out[x] = E::from_float(p.alpha * sum[x]);
   }
   *reinterpret_cast<v4h *>(reinterpret_cast<uint16_t *>(p.dw) + i) = out;
 }

@@ -455,4 +455,8 @@ class ConvParams(_Versioned):
         self.indices = _empty_tensor()
         self.mask_output = _empty_tensor()
         self.stream = 0
+        # not in the reference's struct: backward-weight with a split_k_parallel descriptor adds its
+        # partial sums in a fixed order (the same bits from run to run), as the reference's serial
+        # split-K does, at the speed of the balanced kernels
+        self.deterministic = False
         self.nvrtc_params = NVRTCParams()

@@ -118,6 +118,10 @@ typedef struct CummHipSparseConvArgs {
                                        the reference's mask-based kernels implement */
   int32_t groups;                   /* must be 1 */
   int32_t d_is_bias;
+  int32_t deterministic;            /* backward-weight with a split_k_parallel descriptor: non-zero = partial sums
+                                       added in a fixed order (same bits from run to run on one device), as the
+                                       reference's serial split-K is (cumm/conv/kernel.py:1004-1014, 1068-1083);
+                                       workspace: cumm_hip_query_wgrad_ordered_workspace.  Ignored elsewhere. */
   const void *bias_pointer;         /* int8 inference: f32 [K] */
   const void *scale_pointer;        /* int8 inference: f32 [K] */
   int32_t rows_in, rows_out;        /* row counts of the input / output feature tensors */
@@ -153,6 +157,12 @@ int cumm_hip_sparse_conv_static_ws(const CummHipConvDesc *desc, const CummHipSpa
 int64_t cumm_hip_query_gemm_workspace(const CummHipGemmDesc *desc, int m, int n, int k, int split_k_slices);
 int64_t cumm_hip_query_conv_workspace(const CummHipConvDesc *desc, int m, int n, int k, int split_k_slices,
                                       int kernel_volume);
+
+/* Bytes of workspace with which the fixed-order backward-weight (CummHipSparseConvArgs.deterministic)
+ * runs at full width; 256-byte aligned.  With less it uses fewer workgroups, down to a minimum it
+ * names in its error.  -1 for arguments it does not take.  (No counterpart in the reference: its
+ * fixed-order variant is the serial split-K, sized by query_conv_workspace_size.) */
+int64_t cumm_hip_query_wgrad_ordered_workspace(int N, int C, int K, int kernel_volume, int mask_width);
 
 /* GemmMainUnitTest.get_all_algo_desp / ConvMainUnitTest.get_all_conv_algo_desp
  * (cumm/gemm/main.py:914-965, cumm/conv/main.py:467-481): the descriptors this

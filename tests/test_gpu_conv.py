@@ -12,7 +12,7 @@ import pytest
 from oracle import conv_ref
 from oracle import numerics as onm
 
-from cumm_amd import pairs, synth
+from cumm_amd import _capi, pairs, synth
 from cumm_amd import tensorview as tv
 from cumm_amd.conv.main import ConvMainUnitTest
 from cumm_amd.tensorview.gemm import Activation, ConvOpType, ConvParams
@@ -206,6 +206,68 @@ def test_backward_weight_balanced_atomic(dtype, shape, strided):
             split_k_slices=1)
     got = H.as_f32(H.host(p.weight), dtype)
     assert H.rel_err(got, H.as_f32(cur, dtype)) < TOL
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(64, 64, 64), (64, 192, 64), (128, 128, 64), (192, 136, 32), (40, 72, 128)])
+@pytest.mark.parametrize("strided", [False, True])
+def test_backward_weight_fixed_order(dtype, shape, strided):
+    """ConvParams.deterministic with the split_k_parallel descriptor: partial sums kept per workgroup
+    and added in a fixed order.  Against the oracle's once-rounded float32 sum (two mask splits,
+    alpha and beta), and the same bits on a second run and on a run with other contents in the
+    workspace; a workspace with room for fewer workgroups still gives a result within tolerance."""
+    c_in, k_out, mask_width = shape
+    print("case backward_weight_fixed_order", dtype, shape, strided, flush=True)
+    rng, coords, pt, feat, w, n_in, n_out = _case(15, 3000, c_in, k_out, dtype, strided=strided)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    red = conv_ref.tile_masks(ms, mask_width)
+    dw0 = H.to_storage(rng.normal(0, 1, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=True)
+
+    def run(workspace=None):
+        p = ConvParams(3, ConvOpType.BackwardWeight)
+        p.conv_algo_desp = desp
+        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(dw0, dtype), H.dev(dout, dtype)
+        p.indices = H.dev(pt.indices_fwd, "i32")
+        p.mask, p.mask_argsort = H.dev(red, "u32"), H.dev(order, "i32")
+        p.mask_width = mask_width
+        p.split_k_slices = 4
+        p.deterministic = True
+        if workspace is not None:
+            p.workspace = workspace
+        for filt, beta in ((0x3FFF, 0.0), (0x1FFF << 14, 1.0)):
+            p.mask_filter, p.beta, p.alpha = filt, beta, 0.5
+            ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(p.weight), p.workspace
+
+    cur = dw0
+    for filt, beta in ((0x3FFF, 0.0), (0x1FFF << 14, 1.0)):
+        cur = conv_ref.implicit_gemm_wgrad_ref(
+            dout, feat, cur, pt.indices_fwd, red, order, mask_width=mask_width, dtype_dout=dtype,
+            dtype_in=dtype, dtype_w=dtype, mask_filter=filt, alpha=0.5, beta=beta, split_k_slices=1)
+    first, ws = run()
+    assert H.rel_err(H.as_f32(first, dtype), H.as_f32(cur, dtype)) < TOL
+    again, _ = run()
+    np.testing.assert_array_equal(first, again)
+    # same size of workspace, garbage inside: nothing in it has to start at zero
+    dirty = H.dev(np.random.default_rng(1).integers(0, 255, size=ws.nbytes, dtype=np.uint8), "u8")
+    third, _ = run(dirty)
+    np.testing.assert_array_equal(first, third)
+    need = int(_capi.lib().cumm_hip_query_wgrad_ordered_workspace(n_out, c_in, k_out, 27, mask_width))
+    assert need == ws.nbytes
+    # the reference's size for four slices: room for fewer workgroups (another split of the sum:
+    # other bits, same tolerance) or, with many channel blocks, for none (the error names the least)
+    m, n, k = k_out, 27 * c_in, n_out
+    small = tv.empty([desp.query_conv_workspace_size(m, n, k, 4, 27)], tv.uint8, 0)
+    assert small.nbytes < need
+    try:
+        fourth, _ = run(small)
+        assert H.rel_err(H.as_f32(fourth, dtype), H.as_f32(cur, dtype)) < TOL
+    except RuntimeError as e:
+        assert "workspace at least" in str(e)
+    with pytest.raises(RuntimeError, match="workspace at least"):
+        run(tv.empty([4096], tv.uint8, 0))
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

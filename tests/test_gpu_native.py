@@ -128,3 +128,26 @@ def test_native_forward_against_dense_conv3d():
     wt = torch.from_numpy(w_ref.astype(np.float64)).reshape(5, 5, 5, k_out, c_in).permute(3, 4, 0, 1, 2).contiguous()
     want = F.conv3d(dense, wt, padding=2)[0, :, coords[:, 1], coords[:, 2], coords[:, 3]].T.numpy()
     assert H.rel_err(H.host(out).astype(np.float32), want.astype(np.float32)) < TOL
+
+
+def test_plan_runs_again_on_new_contents():
+    """A forward plan is validated once; a second run reads the tensors' current contents."""
+    rng = np.random.default_rng(65)
+    grid = (8, 10, 10)
+    coords = synth.clustered_voxels(rng, 300, grid, 3, sigma=2.5)
+    c_in, k_out = 16, 16
+    host = pairs.subm_pairs(coords, grid, ksize=(5, 5, 5))
+    devt = pairs.subm_pairs_device(H.dev(coords, "i32"), grid, ksize=(5, 5, 5))
+    lists_h, lists_d = pairs.pair_lists(host.indices_fwd), pairs.pair_lists_device(devt.indices_fwd)
+    n = coords.shape[0]
+    weight = rng.normal(0, 0.1, size=(k_out, 125, c_in)).astype(np.float16)
+    d_feat = tv.zeros([n, c_in], tv.float16, 0)
+    out = tv.zeros([n, k_out], tv.float16, 0)
+    plan = native.plan_forward(d_feat, H.dev(weight, "f16"), out, lists_d)
+    assert plan.launches == int((lists_h.counts > 0).sum()) + 2
+    for seed in (1, 2):
+        feat = np.random.default_rng(seed).normal(0, 1, size=(n, c_in)).astype(np.float16)
+        d_feat.copy_(tv.from_numpy(feat))
+        plan()
+        ref = native_ref.native_fwd_ref(feat, weight, lists_h.pair_in, lists_h.pair_out, lists_h.counts, n, dtype="f16")
+        assert H.rel_err(H.host(out).astype(np.float32), ref.astype(np.float32)) < TOL
