@@ -232,9 +232,13 @@ def bench_stack(args):
     ws_p = tv.empty([int(lib.cumm_hip_subm_pairs_workspace(n))], tv.uint8, 0)
     ws_s = tv.empty([int(lib.cumm_hip_sort_by_mask_workspace(max(n, n_out2)))], tv.uint8, 0)
     sorted1, sorted2 = (ms_tv, order_tv), (ms2_tv, order2_tv)
+    import ctypes
+    arr3 = ctypes.c_int32 * 3
+    ws_c = tv.empty([int(lib.cumm_hip_conv_pairs_workspace(n, 1, arr3(*grid), arr3(3, 3, 3), arr3(2, 2, 2), arr3(1, 1, 1),
+                                                           arr3(1, 1, 1)))], tv.uint8, 0)
     for name, fn in (("subm_pairs", lambda: pairs.subm_pairs_device(d_coords, grid, workspace=ws_p, out=table)),
                      ("sort_by_mask", lambda: pairs.sort_by_mask_device(table.mask_fwd, workspace=ws_s, out=sorted1)),
-                     ("sparse_conv_pairs_stride2", lambda: pairs.sparse_conv_pairs_device(d_coords, grid, batch_size=1)),
+                     ("sparse_conv_pairs_stride2", lambda: pairs.sparse_conv_pairs_device(d_coords, grid, batch_size=1, workspace=ws_c, out=table2)),
                      ("sort_by_mask_stride2", lambda: pairs.sort_by_mask_device(table2.mask_fwd, workspace=ws_s, out=sorted2))):
         wms, ems = timed(fn, 5, 2)
         prep[name] = {"wall_ms": round(wms, 4), "events_ms": round(ems, 4)}

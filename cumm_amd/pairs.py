@@ -227,11 +227,13 @@ class DeviceConvPairTable(NamedTuple):
 
 def sparse_conv_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), stride=(2, 2, 2),
                              padding=(1, 1, 1), dilation=(1, 1, 1), batch_size: int = 1, workspace=None,
-                             stream: int = 0) -> DeviceConvPairTable:
+                             stream: int = 0, out=None) -> DeviceConvPairTable:
     """GPU counterpart of :func:`sparse_conv_pairs`: ``coords`` is a device ``tv.Tensor`` [N, 4]
     int32 of unique (batch, z, y, x); the tables stay on the device.  Two library calls with one
     stream synchronisation between them (the number of active output sites sizes the tables), as
-    with spconv's generate_conv_inds_mask_stage1 / stage2.  Batch indices are 0 .. batch_size-1."""
+    with spconv's generate_conv_inds_mask_stage1 / stage2.  Batch indices are 0 .. batch_size-1.
+    ``out``: the table of an earlier call; its tensors are written again when the number of output
+    sites is the same (with ``workspace`` the call then allocates nothing)."""
     import ctypes as C
 
     from . import _capi
@@ -253,11 +255,15 @@ def sparse_conv_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 
     _capi.check(lib.cumm_hip_conv_pairs_sites(coords.byte_pointer(), n_in, int(batch_size), *geo, out_shape, C.byref(n_out),
                                               workspace.byte_pointer(), workspace.nbytes, stream))
     n = int(n_out.value)
-    out_coords = tv.empty([n, 4], tv.int32, 0)
-    ind_f = tv.empty([kv, n], tv.int32, 0)
-    ind_b = tv.empty([kv, n_in], tv.int32, 0)
-    mask_f = tv.empty([n], tv.uint32, 0) if kv <= 32 else None
-    mask_b = tv.empty([n_in], tv.uint32, 0) if kv <= 32 else None
+    if out is not None and out.indices_fwd.shape == [kv, n] and out.indices_bwd.shape == [kv, n_in] and \
+            out.out_coords.shape == [n, 4] and (out.mask_fwd is None) == (kv > 32):
+        out_coords, ind_f, ind_b, mask_f, mask_b = out.out_coords, out.indices_fwd, out.indices_bwd, out.mask_fwd, out.mask_bwd
+    else:
+        out_coords = tv.empty([n, 4], tv.int32, 0)
+        ind_f = tv.empty([kv, n], tv.int32, 0)
+        ind_b = tv.empty([kv, n_in], tv.int32, 0)
+        mask_f = tv.empty([n], tv.uint32, 0) if kv <= 32 else None
+        mask_b = tv.empty([n_in], tv.uint32, 0) if kv <= 32 else None
     _capi.check(lib.cumm_hip_conv_pairs_fill(
         coords.byte_pointer(), n_in, int(batch_size), *geo, n, out_coords.byte_pointer(), ind_f.byte_pointer(),
         ind_b.byte_pointer(), mask_f.byte_pointer() if mask_f is not None else None,

@@ -128,3 +128,26 @@ def test_workspace_queries_follow_the_descriptors():
             else:
                 assert lib.cumm_hip_query_conv_workspace(ctypes.byref(cd), m, n, k, s, kv) == \
                     d.query_conv_workspace_size(m, n, k, s, kv)
+
+
+def test_fixed_order_backward_weight_workspace_query():
+    """cumm_hip_query_wgrad_ordered_workspace: 256-byte aligned pieces (live-tile counts, the table of
+    workgroups per (offset, channel block), the live-tile lists) in front of one slot of 64 x 64
+    (or 128 x 128) floats per workgroup and per (offset, channel block); -1 for sizes it does not take."""
+    lib = _capi.lib()
+    q = lib.cumm_hip_query_wgrad_ordered_workspace
+    # 3000 positions, 64-position mask words: 47 tiles, 16 per unit at most -> (3 + 1) * 27 = 108 units
+    n, c, k, kv, mw = 3000, 64, 64, 27, 64
+    lists = 128 + 256 + ((4 * kv * 47 + 255) // 256) * 256
+    assert q(n, c, k, kv, mw) == lists + (108 + 27) * 64 * 64 * 4
+    # both channel counts above 64: slots of 128 x 128; many tiles: 512 workgroups at most
+    n = 1000000
+    tiles = (n + 63) // 64
+    lists = 128 + 256 + ((4 * kv * tiles + 255) // 256) * 256
+    assert q(n, 128, 128, kv, 64) == lists + (512 + 27) * 128 * 128 * 4
+    assert q(n, 128, 256, kv, 64) == 128 + 512 + ((4 * kv * tiles + 255) // 256) * 256 + (512 + 54) * 128 * 128 * 4
+    for bad in ((-1, 64, 64, 27, 64), (10, 0, 64, 27, 64), (10, 64, 64, 33, 64), (10, 64, 64, 27, 2048), (10, 64, 64, 27, 0)):
+        assert q(*bad) == -1
+    args = _capi.SparseConvArgs()
+    args.deterministic = 1     # the field exists (the struct keeps its size: it fills former padding)
+    assert ctypes.sizeof(args) == 176
