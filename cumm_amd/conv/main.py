@@ -99,6 +99,10 @@ class ConvMainUnitTest:
             raise RuntimeError("error")
         if not (desp.split_k_serial or desp.split_k_parallel) and split_k_slices > 1:
             raise RuntimeError("algo don't support splitk but you provide split_k_slices > 1.")
+        if int(getattr(params, "mask_int_count", 1)) != 1:
+            # (tv::gemm::ConvParams::mask_int_count, params.h:413: several 32-bit words per position
+            # for kernel volumes above 32; those go through cumm_amd.conv.native here)
+            raise RuntimeError("one 32-bit mask word per position only (mask_int_count must be 1)")
         K = weight.dim(0)
         C = inp.dim(1)
         if output.dim(1) != K:

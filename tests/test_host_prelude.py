@@ -63,6 +63,10 @@ def test_conv_prelude_errors():
     with pytest.raises(RuntimeError, match="splitk"):
         ConvMainUnitTest.implicit_gemm2(p)
     p = _fwd_params()
+    p.mask_int_count = 2                               # several mask words per position: not built
+    with pytest.raises(RuntimeError, match="mask_int_count"):
+        ConvMainUnitTest.implicit_gemm2(p)
+    p = _fwd_params()
     p.indices = tv.Tensor()
     with pytest.raises(RuntimeError):
         ConvMainUnitTest.implicit_gemm2(p)
