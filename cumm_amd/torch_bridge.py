@@ -185,6 +185,17 @@ class _SparseConvFunction(torch.autograd.Function):
             p.input, p.weight, p.output = torch2tensor(features), torch2tensor(grad_w), torch2tensor(grad_out)
             p.indices, p.mask, p.mask_argsort = g.indices_fwd, g.reduced_mask_buffer(ctx.tile_m), g.order_fwd
             p.mask_width, p.split_k_slices = ctx.tile_m, 32
+            # torch's switch for reproducible results selects the fixed-order sum of the partial blocks
+            p.deterministic = bool(torch.are_deterministic_algorithms_enabled())
+            # the workspace comes from torch's caching allocator (the prelude's own would be a
+            # device allocation per call)
+            n_pos, k_out, kv, c_in = int(grad_out.shape[0]), int(weight.shape[0]), int(weight.shape[1]), int(weight.shape[2])
+            need = p.conv_algo_desp.query_conv_workspace_size(k_out, kv * c_in, n_pos, p.split_k_slices, kv)
+            if p.deterministic:
+                need = max(need, int(lib.cumm_hip_query_wgrad_ordered_workspace(n_pos, c_in, k_out, kv, ctx.tile_m)))
+            if need > 0:
+                ws = torch.empty(need, dtype=torch.uint8, device=grad_out.device)
+                p.workspace = torch2tensor(ws)
             p.stream = stream
             ConvMainUnitTest.implicit_gemm2(p)
         if ctx.has_bias and ctx.needs_input_grad[2]:

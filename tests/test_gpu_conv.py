@@ -408,12 +408,13 @@ def test_kernel_volumes_forward_and_backward(dtype, geometry):
     zero_w = H.to_storage(np.zeros((k_out, kv, c_in), np.float32), dtype)
     ref_w = conv_ref.implicit_gemm_wgrad_ref(dout, feat, zero_w, pt.indices_fwd, red, order, mask_width=64,
                                              dtype_dout=dtype, dtype_in=dtype, dtype_w=dtype, split_k_slices=1)
-    for parallel in (True, False):
+    for parallel, fixed_order in ((True, False), (True, True), (False, False)):
         pw = ConvParams(3, ConvOpType.BackwardWeight)
         pw.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=parallel)
         pw.input, pw.weight, pw.output = p.input, H.dev(zero_w, dtype), pd.output
         pw.indices, pw.mask, pw.mask_argsort = p.indices, H.dev(red, "u32"), p.mask_argsort
         pw.mask_width, pw.split_k_slices = 64, 4 if parallel else 1
+        pw.deterministic = fixed_order
         ConvMainUnitTest.implicit_gemm2(pw)
         assert H.rel_err(H.as_f32(H.host(pw.weight), dtype), H.as_f32(ref_w, dtype)) < TOL
 

@@ -117,3 +117,31 @@ def test_module_stack_runs_and_trains_a_step():
     loss.backward()
     assert all(p.grad is not None and torch.isfinite(p.grad.float()).all() for p in params)
     assert float(l1.weight.grad.float().abs().max()) > 0
+
+
+def test_deterministic_switch_gives_the_same_weight_gradient_twice():
+    """torch.use_deterministic_algorithms(True) selects the fixed-order backward-weight: two
+    backward passes over the same tensors give the same bits (and the value stays within
+    tolerance of the default variant's)."""
+    from cumm_amd import torch_bridge as tb
+    coords, grid = H.small_cloud(23, 3000)
+    geo = tb.SparseConvGeometry(torch.as_tensor(coords, device="cuda"), grid)
+    torch.manual_seed(2)
+    layer = tb.SparseConv3d(64, 64, relu=True)
+    x = torch.randn(coords.shape[0], 64, device="cuda").half()
+
+    def weight_grad():
+        layer.zero_grad(set_to_none=True)
+        layer(x, geo).float().pow(2).mean().backward()
+        return layer.weight.grad.clone()
+
+    default = weight_grad()
+    was = torch.are_deterministic_algorithms_enabled()
+    torch.use_deterministic_algorithms(True)
+    try:
+        first, second = weight_grad(), weight_grad()
+    finally:
+        torch.use_deterministic_algorithms(was)
+    assert torch.equal(first, second)
+    scale = float(default.float().abs().max())
+    assert float((first.float() - default.float()).abs().max()) < 1e-2 * scale
