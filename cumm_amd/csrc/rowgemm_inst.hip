@@ -2,6 +2,7 @@
 #include "launch.h"
 #include "rowgemm_pipe.h"
 #include "rowgemm_lds.h"
+#include "rowgemm_wave.h"
 
 namespace cummhip {
 
@@ -115,8 +116,47 @@ static hipError_t launch_ks(int ks, bool wt, const RowGemmParams &p, hipStream_t
   return hipErrorInvalidValue;
 }
 
+// One weight matrix, no masks, a contraction of at most 128 two-byte elements: the kernel that keeps
+// the matrix in registers (rowgemm_wave.h); the descriptor's tile shape then only names the launch.
+template <class T, int KS, bool WT>
+static hipError_t launch_wave(const RowGemmParams &p, hipStream_t s) {
+  if constexpr (Elem<T>::kBytes == 2) {
+    const int n_blocks = (p.n_pos + 15) / 16;
+    if (n_blocks == 0 || p.k_out <= 0) return hipSuccess;
+    static int resident_of[16] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    int &resident = resident_of[dev & 15];
+    if (resident == 0) {
+      int cus = 0, per_cu = 0;
+      e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (e == hipSuccess) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, rowgemm_wave_kernel<T, KS, WT, kWide>, 256, 0);
+      if (e != hipSuccess) return e;
+      resident = cus * per_cu > 0 ? cus * per_cu : 1;
+    }
+    const int want = (n_blocks + 7) / 8;   // four waves, two row blocks per trip each
+    dim3 grid((unsigned)(want < resident ? want : resident), (unsigned)((p.k_out + 63) / 64), 1);
+    hipLaunchKernelGGL((rowgemm_wave_kernel<T, KS, WT, kWide>), grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+  } else {
+    return hipErrorInvalidValue;
+  }
+}
+
 hipError_t CUMM_LAUNCH_NAME(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s) {
   using T = CUMM_ELEM;
+  if constexpr (Elem<T>::kBytes == 2) {
+    // (up to 64 output channels: a second column block would gather the rows a second time)
+    if (p.mask == nullptr && p.kv == 1 && p.gather_by_pos && p.c_in <= 32 * ks && p.k_out <= 64 &&
+        (wt ? p.w_stride_n == 1 : p.w_stride_c == 1) && (tm == 64 || tm == 128) && (tn == 64 || tn == 128)) {
+      switch (ks) {
+      case 1: return wt ? launch_wave<T, 1, true>(p, s) : launch_wave<T, 1, false>(p, s);
+      case 2: return wt ? launch_wave<T, 2, true>(p, s) : launch_wave<T, 2, false>(p, s);
+      case 4: return wt ? launch_wave<T, 4, true>(p, s) : launch_wave<T, 4, false>(p, s);
+      }
+    }
+  }
   if (tm == 64 && tn == 64) return launch_ks<T, 4, 1, 64>(ks, wt, p, s);
   if (tm == 128 && tn == 64) return launch_ks<T, 4, 2, 64>(ks, wt, p, s);
   if (tm == 64 && tn == 128) return launch_ks<T, 4, 1, 128>(ks, wt, p, s);

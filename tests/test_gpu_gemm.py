@@ -155,6 +155,50 @@ def test_dense_accumulator_output(dtype, tile, trans):
             assert H.rel_err(got, ref) < 2e-3      # no output rounding: only the order of the fp32 sums differs
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("trans_b", [True, False])
+@pytest.mark.parametrize("n,k", [(64, 64), (64, 128), (40, 96), (8, 8), (56, 32), (64, 24)])
+@pytest.mark.parametrize("wide", [False, True])
+def test_shuffle_ac_one_column_block(dtype, trans_b, n, k, wide):
+    """Up to 64 output channels and 128 contraction elements: the kernel that keeps the weight matrix
+    in registers and gathers rows straight into operand registers (csrc/rowgemm_wave.h); ragged
+    row counts, identity and permuted rows, a 2-D source, a bias, ReLU, f32 outputs."""
+    print("case shuffle_ac one block", dtype, trans_b, n, k, wide, flush=True)
+    rng = np.random.default_rng(4242)
+    rows = 3000
+    out = WIDE[dtype] if wide else dtype
+    b = _rand(rng, (k, n), dtype, 0.1)
+    bb = np.ascontiguousarray(b.T) if trans_b else b
+    a = _rand(rng, (rows, k), dtype)
+    for m, with_a in ((2777, True), (33, True), (rows, False), (1, True)):
+        a_inds = rng.permutation(rows)[:m].astype(np.int32)
+        c_inds = rng.permutation(rows)[:m].astype(np.int32)
+        c0 = rng.normal(0, 1, size=(rows, n)).astype(np.float32) if wide else _rand(rng, (rows, n), dtype)
+        bias = rng.normal(0, 1, size=(n,)).astype(np.float32) if wide else _rand(rng, (n,), dtype)
+        for alpha, beta, act, use_bias in ((1.0, 0.0, Activation.None_, False), (0.5, 1.0, Activation.ReLU, False),
+                                           (1.0, 1.0, Activation.LeakyReLU, True)):
+            p = GemmParams()
+            p.algo_desp = H.find_gemm_desp(dtype, ShuffleStrideType.ShuffleAC, 64, 64, False, trans_b, dtype_c=out)
+            p.a, p.b, p.c = H.dev(a, dtype), H.dev(bb, dtype), H.dev(c0, out)
+            if with_a:
+                p.a_inds = H.dev(a_inds, "i32")
+            p.c_inds = H.dev(c_inds, "i32")
+            if use_bias:
+                p.d = H.dev(bias, out)
+            p.alpha, p.beta, p.act_type, p.act_alpha = alpha, beta, act, 0.1
+            GemmMainUnitTest.matmul2(p)
+            ref = gemm_ref.matmul2_ref(a if with_a else a[:m], bb, c0, dtype_a=dtype, dtype_b=dtype, dtype_c=out,
+                                       trans_b=trans_b, shuffle=gemm_ref.SHUFFLE_AC,
+                                       a_inds=a_inds if with_a else None, c_inds=c_inds,
+                                       d=bias if use_bias else None, alpha=alpha, beta=beta, act=act.value,
+                                       act_alpha=0.1)
+            got = H.host(p.c)
+            if wide:
+                assert H.rel_err(got, ref) < 2e-3
+            else:
+                _compare(got, ref, dtype)
+
+
 @pytest.mark.parametrize("dtype", ["s8", "f16", "bf16"])
 @pytest.mark.parametrize("tile", [(64, 64), (128, 64), (64, 128), (128, 128)])
 @pytest.mark.parametrize("trans_b", [True, False])
