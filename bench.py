@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0
 # their result lives in this summary, on a line that also carries a hash of the kernel's sources.
 TRAFFIC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
                                "rowgemm_lds_f16_subm_c64_fwd.md")
-KERNEL_SOURCES = ("rowgemm_lds.h", "rowgemm.h", "lds_dma.h", "common.h", "rowgemm_inst.hip")
+KERNEL_SOURCES = ("rowgemm_lds.h", "rowgemm.h", "lds_dma.h", "common.h", "rowgemm_inst.hip", "rowgemm_wave.h")
 
 
 def kernel_source_hash():
