@@ -4,7 +4,9 @@ backward-weight, two calls in a row, the second on a smaller input.
 
 Serial split-K is deterministic: compared bit for bit.  The balanced (split_k_parallel) kernels
 add fp32 partial sums with atomics in no fixed order: compared within the f16/bf16 tolerance of
-1e-2 (fp32 accumulate), against the existing entry point and against the oracle.
+1e-2 (fp32 accumulate), against the existing entry point and against the oracle; their fixed-order
+variant splits the sum by the number of workgroups its workspace has slots for, so it is compared
+with the oracle within the tolerance and with itself bit for bit.
 """
 import numpy as np
 import pytest
@@ -87,6 +89,25 @@ def test_static_workspace_balanced(dtype):
         assert H.rel_err(got, H.as_f32(oracle(False), dtype)) < TOL
         # an unchanged repeat call (the validated-arguments path) gives the same again
         ConvMainUnitTest.implicit_gemm2_static_workspace(p_new)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_static_workspace_fixed_order(dtype):
+    """The fixed-order backward-weight on the static workspace: as many workgroups as its 8 MiB hold
+    slots for; the same bits twice in a row, also after a call on another problem in between."""
+    desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=True)
+    results = []
+    for seed, n, c_in, k_out in ((36, 3000, 128, 128), (37, 900, 64, 72), (36, 3000, 128, 128)):
+        print("case static_ws fixed order", dtype, n, c_in, k_out, flush=True)
+        make, oracle = _wgrad_params(seed, n, c_in, k_out, dtype, desp, split_k=8)
+        p_new = make()
+        p_new.deterministic = True
+        ConvMainUnitTest.implicit_gemm2_static_workspace(p_new)
+        assert p_new.workspace.empty()
+        got = H.host(p_new.weight)
+        assert H.rel_err(H.as_f32(got, dtype), H.as_f32(oracle(False), dtype)) < TOL
+        results.append(got)
+    np.testing.assert_array_equal(results[0], results[2])
 
 
 def test_static_workspace_rejects_what_does_not_fit():
