@@ -105,14 +105,34 @@ __global__ __launch_bounds__(256) void column_partial_kernel(const ColumnSumPara
   }
 }
 
-// dst[c] = cvt(sum over blocks, in block order)
+// dst[c] = cvt(sum over blocks) in a fixed shape: sixteen threads per channel, thread j adds the j-th
+// sixteenth of the blocks in block order (eight loads in flight at a time: one thread walking all
+// 1024 blocks took 54 us), then the sixteen sums are added in order
 template <class T>
 __global__ __launch_bounds__(256) void column_final_kernel(const ColumnSumParams p) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= p.channels) return;
+  __shared__ float part[16][17];
+  const int cl = threadIdx.x & 15, j = threadIdx.x >> 4;
+  const int c = blockIdx.x * 16 + cl;
+  const int share = (p.blocks + 15) >> 4;
+  const int b0 = j * share, b1 = b0 + share < p.blocks ? b0 + share : p.blocks;
   float s = 0.0f;
-  for (int b = 0; b < p.blocks; ++b) s += p.partial[(int64_t)b * p.channels + c];
-  reinterpret_cast<uint16_t *>(p.dst)[c] = Elem<T>::from_float(s);
+  if (c < p.channels) {
+    for (int b = b0; b < b1; b += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = b + u < b1 ? p.partial[(int64_t)(b + u) * p.channels + c] : 0.0f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+  }
+  part[j][cl] = s;
+  __syncthreads();
+  if (j == 0 && c < p.channels) {
+    float total = part[0][cl];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) total += part[k][cl];
+    reinterpret_cast<uint16_t *>(p.dst)[c] = Elem<T>::from_float(total);
+  }
 }
 
 unsigned grid_for(size_t items) {
@@ -156,10 +176,10 @@ hipError_t launch_column_sum(ColumnSumParams p, bool bf16, hipStream_t s) {
   p.rows_per_block = (p.rows + p.blocks - 1) / p.blocks;
   if (bf16) {
     hipLaunchKernelGGL(column_partial_kernel<BF16>, dim3(p.blocks), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(column_final_kernel<BF16>, dim3((p.channels + 255) / 256), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(column_final_kernel<BF16>, dim3((p.channels + 15) / 16), dim3(256), 0, s, p);
   } else {
     hipLaunchKernelGGL(column_partial_kernel<F16>, dim3(p.blocks), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(column_final_kernel<F16>, dim3((p.channels + 255) / 256), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(column_final_kernel<F16>, dim3((p.channels + 15) / 16), dim3(256), 0, s, p);
   }
   return hipGetLastError();
 }

@@ -15,6 +15,15 @@ import numpy as np
 from .. import _capi
 from . import gemm  # noqa: F401  (tv.gemm.*, as in the reference)
 
+
+def _prod(shape) -> int:
+    """Product of the extents (1 for no extents); plain Python integers: this runs on every call of an operator."""
+    n = 1
+    for v in shape:
+        n *= int(v)
+    return n
+
+
 # tv::DType values are ABI: include/tensorview/dtypes.h:39-64 of the reference
 bool_ = 5
 float16 = 7
@@ -176,7 +185,7 @@ class Tensor:
             return
         self._shape = [int(s) for s in shape]
         self._stride = _contig_stride(self._shape)
-        nbytes = int(np.prod(self._shape, dtype=np.int64)) * _ITEMSIZE[self._dtype]
+        nbytes = _prod(self._shape) * _ITEMSIZE[self._dtype]
         if device == -1:
             self._storage = _HostStorage(np.empty(nbytes, dtype=np.uint8))
         else:
@@ -213,7 +222,7 @@ class Tensor:
 
     @property
     def size(self) -> int:
-        return int(np.prod(self._shape, dtype=np.int64)) if self._storage is not None else 0
+        return _prod(self._shape) if self._storage is not None else 0
 
     @property
     def itemsize(self) -> int:
@@ -257,9 +266,9 @@ class Tensor:
         assert self.is_contiguous(), "view needs a contiguous tensor"
         shape = [int(s) for s in shape]
         if -1 in shape:
-            known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+            known = _prod([s for s in shape if s != -1])
             shape[shape.index(-1)] = self.size // max(known, 1)
-        assert int(np.prod(shape, dtype=np.int64)) == self.size, (shape, self._shape)
+        assert _prod(shape) == self.size, (shape, self._shape)
         return Tensor._make(self._storage, shape, _contig_stride(shape), self._dtype, self._offset)
 
     def type_view(self, dtype: int, shape: Optional[Sequence[int]] = None) -> "Tensor":
@@ -267,7 +276,7 @@ class Tensor:
         if shape is None:
             assert _ITEMSIZE[dtype] == self.itemsize, "type_view without a shape keeps the item size"
             shape = self._shape
-        assert int(np.prod(shape, dtype=np.int64)) * _ITEMSIZE[dtype] <= self.bytesize()
+        assert _prod(shape) * _ITEMSIZE[dtype] <= self.bytesize()
         return Tensor._make(self._storage, shape, _contig_stride(shape), dtype, self._offset)
 
     def as_strided(self, shape, stride, storage_byte_offset: int = 0) -> "Tensor":

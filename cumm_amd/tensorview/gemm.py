@@ -188,7 +188,14 @@ class GemmAlgoDesp(_Versioned):
                                 lambda s, v: setattr(s, "split_k_parallel_", 1 if v else 0))
 
     def copy(self):
-        return _copy.deepcopy(self)
+        # (every field is a number, a string, an enum, a tuple or a flat list of numbers: a new
+        # object with new lists, without deepcopy's bookkeeping - this runs per operator call in
+        # the callers that build their parameter objects afresh)
+        other = object.__new__(type(self))
+        d = other.__dict__
+        for k, v in self.__dict__.items():
+            d[k] = list(v) if isinstance(v, list) else v
+        return other
 
     def _shuffle_int(self) -> int:
         st = self.shuffle_type
