@@ -232,6 +232,8 @@ class ConvMainUnitTest:
         args.bias_pointer = _ptr(bias)
         args.scale_pointer = _ptr(scale)
         args.rows_in, args.rows_out = inp.dim(0), output.dim(0)
+        args.light_prefix = max(0, min(int(getattr(params, "light_prefix", 0)), N)) \
+            if op_type != ConvOpType.BackwardWeight else 0
         cdesc = conv_desp_to_c(desp)
         name = repr(desp) if params.timer.enable else ""
         if name:

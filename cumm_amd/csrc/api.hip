@@ -633,6 +633,8 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     p.alpha = a->alpha; p.beta = a->beta; p.act_alpha = a->act_alpha; p.act_beta = a->act_beta;
     p.act = a->act_type;
     p.read_source = a->beta != 0.0f;
+    // (the hint only moves work between tile shapes; whatever it says the kernel covers every position once)
+    p.pair_tiles = a->light_prefix > 0 ? a->light_prefix / 128 : 0;
     if (c.is_int8_inference) {
       if (!a->bias_pointer || !a->scale_pointer)
         return fail(CUMM_HIP_ERUNTIME, "int8 inference must have both scale and bias");
@@ -1012,6 +1014,13 @@ int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uin
   hipError_t e = launch_sort_by_mask(mask, n, mask_filter, sorted_mask, argsort, workspace, status + 1,
                                      reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "mask sort launch");
+  return CUMM_HIP_OK;
+}
+
+int cumm_hip_light_prefix(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream) {
+  if (n < 0 || !prefix || (n > 0 && !sorted_mask)) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  hipError_t e = launch_light_prefix(sorted_mask, n, mask_filter, prefix, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "light prefix launch");
   return CUMM_HIP_OK;
 }
 

@@ -95,6 +95,7 @@ size_t conv_pairs_scan_temp_bytes(size_t n_words);
 hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t temp_bytes, hipStream_t s);
 // stable radix sort of mask & filter with its permutation (sort_inst.hip)
 size_t sort_by_mask_workspace_bytes(int n);
+hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, hipStream_t s);
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
                                void *workspace, int32_t *give_ups, hipStream_t s);
 

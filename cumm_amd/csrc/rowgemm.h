@@ -59,6 +59,9 @@ struct RowGemmParams {
   // LDS-streaming kernel only: the contraction is walked in 2^chunk_shift chunks of one stage
   // row each (a step = one kernel offset x one chunk); 0 = the whole contraction fits a row
   int32_t chunk_shift;
+  // LDS-streaming kernel, one column block: the first pair_tiles runs of 128 sorted positions are
+  // taken as 128-row tiles (rowgemm_lds_mixed_kernel); 0 = 64-row tiles throughout
+  int32_t pair_tiles;
 };
 
 // An offset no buffer contains: every operand is smaller than 2 GiB (checked on the host), and

@@ -79,6 +79,12 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   if constexpr (NS > 0 && (!WT || Elem<T>::kBytes == 2)) {
     // the LDS-streaming kernel: 2 x 2 waves, each TM/2 rows by TN/2 channels
     if (p.c_in <= chunk_e && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
+      if constexpr (TM == 64 && TN == 64 && Elem<T>::kBytes == 2 && KS <= 2 && !kWide) {
+        if (p.pair_tiles > 0 && grid.y == 1 && p.chunk_shift == 0 && p.mask != nullptr) {
+          hipLaunchKernelGGL((rowgemm_lds_mixed_kernel<T, KS, WT>), grid, dim3(256), 0, s, p);
+          return hipGetLastError();
+        }
+      }
       hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS, WT, kWide>), grid, dim3(256), 0, s, p);
       return hipGetLastError();
     }

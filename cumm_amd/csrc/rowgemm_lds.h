@@ -54,8 +54,19 @@ __device__ __forceinline__ bool run_steps(F &f, std::integer_sequence<int, Is...
 // reads make one operand.  A lane then owns channels nb*16 + 4q .. +3 of each block nb.
 // WIDE: four-byte outputs (s32 / f32: the accumulators through the linear combination, see
 // store_wide_piece in rowgemm.h).
-template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT = false, bool WIDE = false>
-__global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmParams p) {
+// The LDS a tile body works in: row part and weight part of each ring stage, and the slots of the
+// pair-table entries.  The kernels below declare the arrays (every stage its own __shared__ array,
+// see above) and hand them over; the body is inlined, so these are compile-time addresses.
+struct LdsRing {
+  v4i *rows[4];
+  v4i *weights[4];
+  int (*idx[4])[64];
+};
+
+// One tile: rows [tile * TM, tile * TM + TM) of the sorted positions, column block col.
+// HALVES: mask_out takes one word per 64 positions (a 128-row tile writes words 2 tile, 2 tile + 1).
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT, bool WIDE, bool HALVES>
+__device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const int tile, const int col, const LdsRing &lds) {
   using E = Elem<T>;
   using AccV = typename E::AccV;
   constexpr int NW = WM * WN;
@@ -86,60 +97,16 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   constexpr int WAIT_OPERANDS = 1 + (L - 1) * PER_STEP;
   static_assert(WAIT_OPERANDS < 64, "too many loads in flight for the counter");
 
-  __shared__ v4i st0[STAGE_V];
-  __shared__ v4i st1[STAGE_V];
-  __shared__ v4i st2[NS > 2 ? STAGE_V : 1];
-  __shared__ v4i st3[NS > 3 ? STAGE_V : 1];
-  // pair-table entries also travel global -> LDS directly: every vector load of the step loop is
-  // then counted by hand, none returns into a register the compiler would guard with waits of
-  // its own.  Slot [d][wave][l] is written by lane l of the wave (lanes >= RPW write zeros).
-  // (one array per slot, like the stages)
-  __shared__ int ix0[NW][64];
-  __shared__ int ix1[NW][64];
-  __shared__ int ix2[NS > 2 ? NW : 1][64];
-  __shared__ int ix3[NS > 3 ? NW : 1][64];
-  auto stage = [&](auto sc) -> v4i * {
-    constexpr int s = decltype(sc)::value;
-    if constexpr (s == 0) return st0;
-    else if constexpr (s == 1) return st1;
-    else if constexpr (s == 2) return st2;
-    else return st3;
-  };
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int m = lane & 15;
   const int q = lane >> 4;
-  auto idx_slot = [&](auto sc) -> int * {
-    constexpr int s = decltype(sc)::value;
-    if constexpr (s == 0) return ix0[wave];
-    else if constexpr (s == 1) return ix1[wave];
-    else if constexpr (s == 2) return ix2[wave];
-    else return ix3[wave];
-  };
+  auto stage = [&](auto sc) -> v4i * { return lds.rows[decltype(sc)::value]; };
+  auto stage_w = [&](auto sc) -> v4i * { return lds.weights[decltype(sc)::value]; };
+  auto idx_slot = [&](auto sc) -> int * { return lds.idx[decltype(sc)::value][wave]; };
 
-  // Workgroups are dispatched in the order of their linear number, round-robin over the 8 XCDs.
-  // With several column blocks per row tile, the workgroups of one row tile are given numbers 8
-  // apart - neighbours in time on one XCD - so that the rows one of them gathers are in that
-  // XCD's L2 for the others (as grid.y they would run a whole grid.x apart).
-  int tile_rank = (int)blockIdx.x, col = 0;
-  if (gridDim.y > 1) {
-    const int gx = (int)gridDim.x, gy = (int)gridDim.y;
-    const int lin = (int)blockIdx.y * gx + (int)blockIdx.x;
-    const int gx8 = gx & ~7;
-    if (lin < gx8 * gy) {
-      const int slot = lin >> 3;
-      tile_rank = (slot / gy) * 8 + (lin & 7);
-      col = slot % gy;
-    } else {
-      const int rest = lin - gx8 * gy;
-      tile_rank = gx8 + rest / gy;
-      col = rest % gy;
-    }
-  }
-  const int tile = (int)gridDim.x - 1 - tile_rank;  // heaviest tiles first (masks sorted ascending)
   const int n0 = col * TN;
   const int pos_base = tile * TM;
 
@@ -242,7 +209,17 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   uint32_t kmask = 1u;
   if (has_mask) {
     kmask = wave_or_dpp(mk) & p.mask_filter;
-    if (p.mask_out != nullptr && tid == 0 && col == 0) p.mask_out[tile] = kmask;
+    if constexpr (HALVES) {
+      static_assert(!HALVES || MKW == 2, "two mask words of 64 positions");
+      const uint32_t lo = wave_or_dpp((uint32_t)raw_mk[0]) & p.mask_filter;
+      const uint32_t hi = wave_or_dpp((uint32_t)raw_mk[MKW - 1]) & p.mask_filter;
+      if (p.mask_out != nullptr && tid == 0 && col == 0) {
+        p.mask_out[2 * tile] = lo;
+        if ((2 * tile + 1) * 64 < p.n_pos) p.mask_out[2 * tile + 1] = hi;
+      }
+    } else {
+      if (p.mask_out != nullptr && tid == 0 && col == 0) p.mask_out[tile] = kmask;
+    }
     if (p.exit_on_empty && kmask == 0) return;
     if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
     if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
@@ -330,7 +307,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   for (int s = 0; s < KS; ++s) {
     const int slot = m * LPR + ((s * 4 + q) ^ swz(m));
     a_rd[s] = wm * (RBW * 16) * LPR + slot;
-    w_rd[s] = A_V + wn * (NBW * 16) * LPR + slot;
+    w_rd[s] = wn * (NBW * 16) * LPR + slot;       // (relative to the weight part)
   }
   // transposing reads: byte address inside the weight part for (k-step s, half h, block nb)
   int wt_rd[WT ? KS : 1][2][WT ? NBW : 1];
@@ -348,7 +325,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
           // like the fragment order of the untransposed weights
           const int col = wn * (NBW * 16) + (m & 3) * (4 * NBW) + nb * 4;
           const int chunk = (col / PV) ^ swz_w(e);
-          wt_rd[s][h][nb] = A_V * 16 + e * (LPRW * 16) + chunk * 16 + (col % PV) * E::kBytes;
+          wt_rd[s][h][nb] = e * (LPRW * 16) + chunk * 16 + (col % PV) * E::kBytes;
         }
   }
 
@@ -405,7 +382,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     for (int t = 0; t < IPA; ++t) dst[t] = has_gather ? slot[t * RPI + lrow] : a_key[t];
   };
   constexpr int CHUNK_E = LPR * PV;      // contraction elements of a stage row
-  auto issue_operands = [&](int j, const int (&src)[IPA], v4i *st) {
+  auto issue_operands = [&](int j, const int (&src)[IPA], v4i *st, v4i *stw) {
     const int k = __builtin_amdgcn_readlane(klist, (j >> p.chunk_shift) & 63);
     const int cc = j & ((1 << p.chunk_shift) - 1);          // chunk of the contraction
     const int cc_e = cc * CHUNK_E;                           // its first element
@@ -426,7 +403,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     const uint32_t soff = (uint32_t)k * w_k_bytes + (WT ? (uint32_t)cc_e * (uint32_t)p.w_stride_c * E::kBytes : cc_b);
 #pragma unroll
     for (int t = 0; t < IPW; ++t)
-      dma_b128(rs_w, lds_addr(st + A_V + (wave * IPW + t) * 64), cc_e + w_cpos[t] < p.c_in ? w_voff[t] : kOob, soff);
+      dma_b128(rs_w, lds_addr(stw + (wave * IPW + t) * 64), cc_e + w_cpos[t] < p.c_in ? w_voff[t] : kOob, soff);
   };
 
   if (n_steps > 0) {
@@ -438,7 +415,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       wait_vmcnt<DI - 1 + j * (PER_STEP - 1)>();   // entries of offset j have landed
       int v[IPA];
       read_idx(idx_slot(std::integral_constant<int, j % DI>{}), v);
-      issue_operands(j, v, stage(std::integral_constant<int, j % NS>{}));
+      issue_operands(j, v, stage(std::integral_constant<int, j % NS>{}), stage_w(std::integral_constant<int, j % NS>{}));
       issue_idx(j + DI, idx_slot(std::integral_constant<int, j % DI>{}));
       return false;
     };
@@ -456,17 +433,18 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       lds_barrier();
       // fragment reads first: their LDS round trip overlaps the address work of the loads below
       const v4i *st = stage(std::integral_constant<int, sc>{});
+      const v4i *stw = stage_w(std::integral_constant<int, sc>{});
       v4i af[RBW][KS], wf[NBW][KS];
 #pragma unroll
       for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
           if constexpr (!WT) {
-            wf[nb][s] = st[w_rd[s] + nb * 16 * LPR];
+            wf[nb][s] = stw[w_rd[s] + nb * 16 * LPR];
           } else {
             typedef short v4s __attribute__((ext_vector_type(4)));
             typedef __attribute__((address_space(3))) v4s *lds_v4s;
-            const char *base = reinterpret_cast<const char *>(st);
+            const char *base = reinterpret_cast<const char *>(stw);
             const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(base + wt_rd[s][0][nb]));
             const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)CUMM_LDS_PTR(base + wt_rd[s][1][nb]));
             typedef short v8s __attribute__((ext_vector_type(8)));
@@ -478,7 +456,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
       for (int rb = 0; rb < RBW; ++rb)
 #pragma unroll
         for (int s = 0; s < KS; ++s) af[rb][s] = st[a_rd[s] + rb * 16 * LPR];
-      issue_operands(done + L, v, stage(std::integral_constant<int, sl>{}));
+      issue_operands(done + L, v, stage(std::integral_constant<int, sl>{}), stage_w(std::integral_constant<int, sl>{}));
       issue_idx(done + L + DI, idx_slot(std::integral_constant<int, si>{}));
 #pragma unroll
       for (int rb = 0; rb < RBW; ++rb)
@@ -598,6 +576,84 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
   case 2: with_mode(std::integral_constant<int, 2>{}); break;
   case 3: with_mode(std::integral_constant<int, 3>{}); break;
   default: with_mode(std::integral_constant<int, 0>{}); break;
+  }
+}
+
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT = false, bool WIDE = false>
+__global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmParams p) {
+  constexpr int NW = WM * WN;
+  constexpr int LPR = 4 * KS;
+  constexpr int A_V = WM * RBW * 16 * LPR;
+  constexpr int STAGE_V = (WM * RBW * 16 + WN * NBW * 16) * LPR;
+  __shared__ v4i st0[STAGE_V];
+  __shared__ v4i st1[STAGE_V];
+  __shared__ v4i st2[NS > 2 ? STAGE_V : 1];
+  __shared__ v4i st3[NS > 3 ? STAGE_V : 1];
+  // pair-table entries also travel global -> LDS directly: every vector load of the step loop is
+  // then counted by hand, none returns into a register the compiler would guard with waits of
+  // its own.  Slot [d][wave][l] is written by lane l of the wave (lanes >= RPW write zeros).
+  // (one array per slot, like the stages)
+  __shared__ int ix0[NW][64];
+  __shared__ int ix1[NW][64];
+  __shared__ int ix2[NS > 2 ? NW : 1][64];
+  __shared__ int ix3[NS > 3 ? NW : 1][64];
+  const LdsRing lds = {{st0, st1, st2, st3}, {st0 + A_V, st1 + A_V, NS > 2 ? st2 + A_V : st2, NS > 3 ? st3 + A_V : st3},
+                       {ix0, ix1, ix2, ix3}};
+
+  // Workgroups are dispatched in the order of their linear number, round-robin over the 8 XCDs.
+  // With several column blocks per row tile, the workgroups of one row tile are given numbers 8
+  // apart - neighbours in time on one XCD - so that the rows one of them gathers are in that
+  // XCD's L2 for the others (as grid.y they would run a whole grid.x apart).
+  int tile_rank = (int)blockIdx.x, col = 0;
+  if (gridDim.y > 1) {
+    const int gx = (int)gridDim.x, gy = (int)gridDim.y;
+    const int lin = (int)blockIdx.y * gx + (int)blockIdx.x;
+    const int gx8 = gx & ~7;
+    if (lin < gx8 * gy) {
+      const int slot = lin >> 3;
+      tile_rank = (slot / gy) * 8 + (lin & 7);
+      col = slot % gy;
+    } else {
+      const int rest = lin - gx8 * gy;
+      tile_rank = gx8 + rest / gy;
+      col = rest % gy;
+    }
+  }
+  const int tile = (int)gridDim.x - 1 - tile_rank;  // heaviest tiles first (masks sorted ascending)
+  rowgemm_lds_tile<T, WM, WN, RBW, NBW, KS, NS, WT, WIDE, false>(p, tile, col, lds);
+}
+
+// Tiles of two shapes in one launch, for one column block of 64 channels (grid.x = number of
+// 64-row tiles): the first p.pair_tiles runs of 128 sorted positions are taken as 128-row tiles
+// with a ring of two stages, the rest as 64-row tiles with three.  What it is for: the light end
+// of the ascending mask order (a submanifold layer's centre-only masks are the smallest mask
+// value and lead it: two thirds of the positions of a LiDAR sweep), where a tile has one or two
+// kernel offsets and its life is its three dependent memory round trips, not its bytes, so that
+// the launch is bound by how many workgroups it has to turn over.  Both rings fill the same LDS
+// (three blocks of 64 rows + 64 weight rows, or two blocks of 128 rows and both weight tiles in
+// the third), so the occupancy is that of the 64-row kernel.  Any split gives the same bits; a
+// many-offset tile in the 128-row part only runs slower (two stages).  Workgroups are dispatched
+// in the order of their number: the 64-row tiles first, heaviest first, then the pairs; the
+// numbers left over leave at once, last of all.
+template <class T, int KS, bool WT>
+__global__ __launch_bounds__(256) void rowgemm_lds_mixed_kernel(const RowGemmParams p) {
+  constexpr int R64 = 64 * 4 * KS;        // 16-byte vectors of 64 rows
+  __shared__ v4i st0[2 * R64];
+  __shared__ v4i st1[2 * R64];
+  __shared__ v4i st2[2 * R64];
+  __shared__ int ix0[4][64];
+  __shared__ int ix1[4][64];
+  __shared__ int ix2[4][64];
+  const int tiles = (int)gridDim.x;
+  const int pairs = p.pair_tiles < (tiles >> 1) ? p.pair_tiles : (tiles >> 1);
+  const int singles = tiles - 2 * pairs;
+  const int rank = (int)blockIdx.x;
+  if (rank < singles) {
+    const LdsRing lds = {{st0, st1, st2, nullptr}, {st0 + R64, st1 + R64, st2 + R64, nullptr}, {ix0, ix1, ix2, nullptr}};
+    rowgemm_lds_tile<T, 2, 2, 2, 2, KS, 3, WT, false, false>(p, tiles - 1 - rank, 0, lds);
+  } else if (rank - singles < pairs) {
+    const LdsRing lds = {{st0, st1, nullptr, nullptr}, {st2, st2 + R64, nullptr, nullptr}, {ix0, ix1, nullptr, nullptr}};
+    rowgemm_lds_tile<T, 2, 2, 4, 2, KS, 2, WT, false, true>(p, pairs - 1 - (rank - singles), 0, lds);
   }
 }
 

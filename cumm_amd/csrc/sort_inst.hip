@@ -18,6 +18,7 @@
 // always drains.
 // Integer work, bound by launch latency at 10^5 keys and by HBM / L2 traffic at 10^6 and more.
 #include "launch.h"
+#include "lds_dma.h"
 
 namespace cummhip {
 
@@ -253,6 +254,25 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   }
 }
 
+// How far the light end of a sorted mask array reaches: the number of leading runs of 128
+// positions whose two halves of 64 each have at most kLightOffsets kernel offsets in the OR of
+// their masks, as a number of positions.  One wave per run; a run that fails lowers the result
+// (which starts at the positions of all whole runs) to where it begins.
+constexpr int kLightOffsets = 2;
+
+__global__ __launch_bounds__(64) void light_prefix_init_kernel(int32_t *result, int runs) {
+  if (threadIdx.x == 0) *result = runs * 128;
+}
+
+__global__ __launch_bounds__(256) void light_prefix_kernel(const uint32_t *sorted, int runs, uint32_t filter, int32_t *result) {
+  const int lane = threadIdx.x & 63;
+  const int run = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (run >= runs) return;
+  const uint32_t lo = wave_or_dpp(sorted[(size_t)run * 128 + lane] & filter);
+  const uint32_t hi = wave_or_dpp(sorted[(size_t)run * 128 + 64 + lane] & filter);
+  if (lane == 0 && (__builtin_popcount(lo) > kLightOffsets || __builtin_popcount(hi) > kLightOffsets)) atomicMin(result, run * 128);
+}
+
 size_t align256s(size_t x) { return (x + 255) & ~(size_t)255; }
 
 int sort_passes(uint32_t filter) {
@@ -300,6 +320,13 @@ hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uin
     r.src_vals = to_out ? tmp_vals : argsort;
     hipLaunchKernelGGL(sort_pass_kernel, dim3(p.chunks), dim3(kSortThreads), 0, s, r);
   }
+  return hipGetLastError();
+}
+
+hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, hipStream_t s) {
+  const int runs = n / 128;
+  hipLaunchKernelGGL(light_prefix_init_kernel, dim3(1), dim3(64), 0, s, result, runs);
+  if (runs > 0) hipLaunchKernelGGL(light_prefix_kernel, dim3((runs + 3) / 4), dim3(256), 0, s, sorted, runs, filter, result);
   return hipGetLastError();
 }
 

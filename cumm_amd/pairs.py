@@ -146,6 +146,23 @@ def sort_by_mask(mask: np.ndarray, mask_filter: int = 0xFFFFFFFF):
     return np.ascontiguousarray(key[order]), order
 
 
+def light_prefix(sorted_mask: np.ndarray, mask_filter: int = 0xFFFFFFFF) -> int:
+    """How far the light end of a sorted mask array reaches: the number of leading positions (a
+    multiple of 128) in runs of 128 whose two halves of 64 each OR to at most two kernel offsets.
+    The value of ``ConvParams.light_prefix`` (a submanifold layer's centre-only positions lead the
+    ascending order); the reference has no such hint."""
+    key = np.asarray(sorted_mask, np.uint32) & np.uint32(mask_filter)
+    runs = key.shape[0] // 128
+    if runs == 0:
+        return 0
+    words = np.bitwise_or.reduce(key[:runs * 128].reshape(runs * 2, 64), axis=1)
+    bits = np.zeros(runs * 2, np.int64)
+    for b in range(32):
+        bits += (words >> np.uint32(b)) & np.uint32(1)
+    heavy = np.nonzero(bits.reshape(runs, 2).max(axis=1) > 2)[0]
+    return int(heavy[0] if heavy.size else runs) * 128
+
+
 class PairLists(NamedTuple):
     pair_in: np.ndarray    # [kv, N] int32: input rows of offset k's pairs, packed to the front
     pair_out: np.ndarray   # [kv, N] int32: their output rows (ascending)
@@ -297,6 +314,21 @@ def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, str
                                           out_mask.byte_pointer(), order.byte_pointer(),
                                           workspace.byte_pointer(), workspace.nbytes, stream))
     return out_mask, order
+
+
+def light_prefix_device(sorted_mask, mask_filter: int = 0xFFFFFFFF, stream: int = 0) -> int:
+    """:func:`light_prefix` of a device ``tv.Tensor`` [N] uint32, counted on the GPU; the one
+    number comes back to the host (the call waits for the stream)."""
+    from . import _capi
+    from . import tensorview as tv
+    if sorted_mask.device < 0 or sorted_mask.dtype != tv.uint32 or sorted_mask.ndim != 1:
+        raise ValueError("sorted_mask must be a device uint32 vector")
+    lib = _capi.lib()
+    res = tv.empty([1], tv.int32, 0)
+    _capi.check(lib.cumm_hip_light_prefix(sorted_mask.byte_pointer(), int(sorted_mask.shape[0]),
+                                          int(mask_filter) & 0xFFFFFFFF, res.byte_pointer(), stream))
+    _capi.check(lib.cumm_hip_stream_synchronize(stream))
+    return int(res.cpu().numpy()[0])
 
 
 class DevicePairLists(NamedTuple):

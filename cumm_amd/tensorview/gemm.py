@@ -466,4 +466,8 @@ class ConvParams(_Versioned):
         # partial sums in a fixed order (the same bits from run to run), as the reference's serial
         # split-K does, at the speed of the balanced kernels
         self.deterministic = False
+        # not in the reference's struct either: a hint for forward / backward-input, the number of
+        # leading positions of the sorted order in tiles of one or two kernel offsets
+        # (pairs.light_prefix of the sorted mask); 0 = unknown.  Any value gives the same result.
+        self.light_prefix = 0
         self.nvrtc_params = NVRTCParams()

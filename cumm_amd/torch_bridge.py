@@ -159,6 +159,10 @@ class SparseConvGeometry:
             self.mask_bwd, self.order_bwd = self.mask_fwd, self.order_fwd
         else:
             self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, stream=stream)
+        # how far the light end of each sorted order reaches (the forward / backward-input launches
+        # take it as a hint; one number each comes back to the host here)
+        self.light_fwd = pairs.light_prefix_device(self.mask_fwd, stream=stream)
+        self.light_bwd = self.light_fwd if self.subm else pairs.light_prefix_device(self.mask_bwd, stream=stream)
         self._reduced = {}
         self._launches = {}      # validated calls of the layers on this geometry, see _Launch
 
@@ -201,6 +205,7 @@ class _SparseConvFunction(torch.autograd.Function):
         p.conv_algo_desp = _desp_like(dtype, ConvOpType.Forward)
         p.input, p.weight, p.output = torch2tensor(features), torch2tensor(weight), torch2tensor(out)
         p.indices, p.mask, p.mask_argsort = geometry.indices_fwd, geometry.mask_fwd, geometry.order_fwd
+        p.light_prefix = geometry.light_fwd
         if bias is not None:
             p.bias, p.beta = torch2tensor(bias), 1.0
         if relu:
@@ -246,6 +251,7 @@ class _SparseConvFunction(torch.autograd.Function):
                 p.input, p.weight, p.output = torch2tensor(grad_in), torch2tensor(weight), torch2tensor(grad_out)
                 p.indices, p.mask, p.mask_argsort = g.indices_bwd, g.mask_bwd, g.order_bwd
                 p.reverse_mask = g.subm
+                p.light_prefix = g.light_bwd
                 p.stream = stream
                 _TUNER.tune_conv(p)
                 ConvMainUnitTest.implicit_gemm2(p)

@@ -125,6 +125,12 @@ typedef struct CummHipSparseConvArgs {
   const void *bias_pointer;         /* int8 inference: f32 [K] */
   const void *scale_pointer;        /* int8 inference: f32 [K] */
   int32_t rows_in, rows_out;        /* row counts of the input / output feature tensors */
+  int32_t light_prefix;             /* forward / backward-input, optional (0 = unknown): how many leading positions of
+                                       the sorted order sit in tiles of one or two kernel offsets, as
+                                       cumm_hip_light_prefix counts them for mask_ptr.  A hint only: it moves those
+                                       positions to 128-row tiles (fewer, longer-lived workgroups where a tile's
+                                       time is its memory round trips); any value gives the same bits, a wrong one
+                                       costs time.  No counterpart in the reference. */
 } CummHipSparseConvArgs;
 
 /* Replaces GemmMainUnitTest.matmul2 below its prelude
@@ -228,7 +234,12 @@ int cumm_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* host out-p
  *   output o gathers the input at coord[o] + (k_zyx - ksize/2) * dilation.
  *   workspace: at least cumm_hip_subm_pairs_workspace(n) bytes, 16-byte aligned.
  * cumm_hip_sort_by_mask: sorted = stable ascending sort of (mask & mask_filter), argsort = the
- *   permutation; workspace at least cumm_hip_sort_by_mask_workspace(n) bytes. */
+ *   permutation; workspace at least cumm_hip_sort_by_mask_workspace(n) bytes.
+ * cumm_hip_light_prefix: for a sorted mask array (what cumm_hip_sort_by_mask writes, what a
+ *   convolution takes as mask_ptr): the number of leading positions, a multiple of 128, in runs of
+ *   128 whose two halves of 64 each OR to at most two kernel offsets - a submanifold layer's
+ *   centre-only positions lead the ascending order.  Written to *prefix (device memory, one int32)
+ *   in stream order; the value is CummHipSparseConvArgs.light_prefix.  No counterpart in the reference. */
 size_t cumm_hip_subm_pairs_workspace(int n);
 int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_shape, const int32_t *ksize,
                         const int32_t *dilation, int32_t *indices_fwd, int32_t *indices_bwd,
@@ -237,6 +248,7 @@ int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_sha
 size_t cumm_hip_sort_by_mask_workspace(int n);
 int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
                           int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream);
+int cumm_hip_light_prefix(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream);
 
 /* Pair tables of a regular (strided) sparse convolution, in two calls like spconv's
  * generate_conv_inds_mask_stage1 / stage2 (the reference's callers take them from there; its own

@@ -31,7 +31,7 @@ def test_struct_layouts_match_the_header():
     """sizeof() of the ctypes mirrors against the C compiler's view of include/cumm_hip.h
     (a silent drift would corrupt arguments); the literal sizes guard machines without gcc."""
     sizes = [ctypes.sizeof(c) for c in (_capi.GemmDesc, _capi.ConvDesc, _capi.GemmArgs, _capi.SparseConvArgs)]
-    assert sizes == [72, 96, 160, 176]
+    assert sizes == [72, 96, 160, 184]
     import shutil
     import subprocess
     import tempfile
@@ -149,5 +149,6 @@ def test_fixed_order_backward_weight_workspace_query():
     for bad in ((-1, 64, 64, 27, 64), (10, 0, 64, 27, 64), (10, 64, 64, 33, 64), (10, 64, 64, 27, 2048), (10, 64, 64, 27, 0)):
         assert q(*bad) == -1
     args = _capi.SparseConvArgs()
-    args.deterministic = 1     # the field exists (the struct keeps its size: it fills former padding)
-    assert ctypes.sizeof(args) == 176
+    args.deterministic = 1     # the field exists (it fills former padding)
+    args.light_prefix = 128
+    assert ctypes.sizeof(args) == 184

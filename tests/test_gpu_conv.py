@@ -146,6 +146,78 @@ def test_backward_input(dtype, tile, strided):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("c_in,k_out", [(64, 64), (32, 48)])
+def test_light_prefix_hint_moves_work_not_results(dtype, c_in, k_out):
+    """ConvParams.light_prefix sends the leading positions of the sorted order to 128-row tiles:
+    whatever it says - the count pairs.light_prefix gives, too little, too much, everything - the
+    output rows and the tile masks are the same bits as without it (and those are checked
+    against the oracle)."""
+    print("case light_prefix", dtype, c_in, k_out, flush=True)
+    rng = np.random.default_rng(11)
+    grid = (16, 200, 200)
+    coords = synth.clustered_voxels(rng, 6000, grid, 8, sigma=4.0, noise_frac=0.6)
+    pt = pairs.subm_pairs(coords, grid)
+    n = coords.shape[0]
+    feat = H.to_storage(rng.normal(0, 1, size=(n, c_in)).astype(np.float32), dtype)
+    w = H.to_storage(rng.normal(0, 0.05, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    out0 = H.to_storage(rng.normal(0, 1, size=(n, k_out)).astype(np.float32), dtype)
+    dout = H.to_storage(rng.normal(0, 1, size=(n, k_out)).astype(np.float32), dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    exact = pairs.light_prefix(ms)
+    assert 256 <= exact <= n - 256, "the cloud should have a light end and a heavy end"
+    d_ms, d_order = H.dev(ms, "u32"), H.dev(order, "i32")
+    assert pairs.light_prefix_device(d_ms) == exact
+    assert pairs.light_prefix_device(d_ms, mask_filter=1 << 13) == (n // 128) * 128    # the centre alone: all light
+    tiles = (n + 63) // 64
+    hints = (0, exact, 128, exact - 128, exact + 640, n - 1, n, n + 1000)
+
+    def forward(hint, beta, relu):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, 64, 64)
+        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+        p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_fwd, "i32"), d_ms, d_order
+        p.mask_output = tv.zeros([tiles], tv.uint32, 0)
+        p.beta = beta
+        if relu:
+            p.act_type = Activation.ReLU
+        p.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(p.output), H.host(p.mask_output)
+
+    for beta, relu in ((0.0, False), (1.0, True)):
+        base, base_mo = forward(0, beta, relu)
+        ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(
+            feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype, dtype_out=dtype,
+            beta=beta, act=onm.ACT_RELU if relu else onm.ACT_NONE)
+        assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref, dtype)) < TOL
+        np.testing.assert_array_equal(base_mo, ref_mo)
+        for hint in hints[1:]:
+            got, got_mo = forward(hint, beta, relu)
+            np.testing.assert_array_equal(got.view(np.uint16), base.view(np.uint16), err_msg="hint %d" % hint)
+            np.testing.assert_array_equal(got_mo, base_mo, err_msg="hint %d" % hint)
+
+    def backward_input(hint):
+        p = ConvParams(3, ConvOpType.BackwardInput)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, 64, 64)
+        din = H.dev(H.to_storage(np.zeros((n, c_in), np.float32), dtype), dtype)
+        p.input, p.weight, p.output = din, H.dev(w, dtype), H.dev(dout, dtype)
+        p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_bwd, "i32"), d_ms, d_order
+        p.reverse_mask = True
+        p.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(din)
+
+    if k_out <= 64 and c_in <= 64:
+        base = backward_input(0)
+        ref = conv_ref.implicit_gemm_dgrad_ref(
+            dout, w, np.zeros_like(feat), pt.indices_bwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype,
+            dtype_out=dtype, reverse_mask=True)
+        assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref, dtype)) < TOL
+        for hint in hints[1:]:
+            np.testing.assert_array_equal(backward_input(hint).view(np.uint16), base.view(np.uint16), err_msg="hint %d" % hint)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 @pytest.mark.parametrize("tile", [(64, 64), (128, 128)])
 @pytest.mark.parametrize("split_k", [1, 4, 32])
 def test_backward_weight(dtype, tile, split_k):

@@ -48,6 +48,21 @@ def test_sort_by_mask_is_stable_and_filtered():
     np.testing.assert_array_equal(order2, [1, 3, 4, 0, 2, 5])
 
 
+def test_light_prefix_counts_whole_runs_of_light_halves():
+    c = np.uint32(1 << 13)
+    m = np.full(700, c, np.uint32)
+    assert pairs.light_prefix(m) == 640                 # five whole runs of 128; the rest is not counted
+    assert pairs.light_prefix(m[:127]) == 0
+    m[300] |= 1                                         # two offsets in a half are still light
+    assert pairs.light_prefix(m) == 640
+    m[310] |= 2                                         # a third offset in the same half of run 2
+    assert pairs.light_prefix(m) == 256
+    assert pairs.light_prefix(m, mask_filter=0xFFFFFFFD) == 640
+    m[5] = 7
+    assert pairs.light_prefix(m) == 0
+    assert pairs.light_prefix(np.zeros(0, np.uint32)) == 0
+
+
 def test_synthetic_cloud_is_unique_in_grid_and_seeded():
     grid = (41, 200, 176)
     a = synth.clustered_voxels(np.random.default_rng(7), 5000, grid, 8)
