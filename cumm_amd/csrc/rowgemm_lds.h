@@ -207,12 +207,14 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   }
   // ---- tile mask: OR over the tile's positions (cumm/conv/kernel.py:844-889 of the reference)
   uint32_t kmask = 1u;
+  bool half_skipped = false;   // HALVES: this wave's 64 positions would have been a skipped 64-row tile
   if (has_mask) {
     kmask = wave_or_dpp(mk) & p.mask_filter;
     if constexpr (HALVES) {
-      static_assert(!HALVES || MKW == 2, "two mask words of 64 positions");
+      static_assert(!HALVES || (MKW == 2 && WM == 2), "two mask words of 64 positions, one per row of waves");
       const uint32_t lo = wave_or_dpp((uint32_t)raw_mk[0]) & p.mask_filter;
       const uint32_t hi = wave_or_dpp((uint32_t)raw_mk[MKW - 1]) & p.mask_filter;
+      half_skipped = p.exit_on_empty && (wm == 0 ? lo : hi) == 0u;
       if (p.mask_out != nullptr && tid == 0 && col == 0) {
         p.mask_out[2 * tile] = lo;
         if ((2 * tile + 1) * 64 < p.n_pos) p.mask_out[2 * tile + 1] = hi;
@@ -476,6 +478,8 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   for (int rb = 0; rb < RBW; ++rb)
 #pragma unroll
     for (int i = 0; i < SRC_N; ++i) keep_after_wait(src_pre[rb][i]);
+  // (a 64-row tile without any offset is left alone when exit_on_empty is set: so is that half)
+  if (HALVES && half_skipped) return;
   // ---- epilogue: lane (q, m) holds, for each of its rows, channels ch0 .. ch0 + 4*NBW - 1.
   // The activation and the blend mode are lifted out of the element loops (one straight-line
   // copy per combination): tested per element they cost more issue slots than the arithmetic.

@@ -171,28 +171,31 @@ def test_light_prefix_hint_moves_work_not_results(dtype, c_in, k_out):
     tiles = (n + 63) // 64
     hints = (0, exact, 128, exact - 128, exact + 640, n - 1, n, n + 1000)
 
-    def forward(hint, beta, relu):
+    def forward(hint, beta, relu, with_bias):
         p = ConvParams(3, ConvOpType.Forward)
         p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, 64, 64)
         p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
         p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_fwd, "i32"), d_ms, d_order
         p.mask_output = tv.zeros([tiles], tv.uint32, 0)
         p.beta = beta
+        if with_bias:
+            p.bias = H.dev(bias, dtype)
         if relu:
             p.act_type = Activation.ReLU
         p.light_prefix = hint
         ConvMainUnitTest.implicit_gemm2(p)
         return H.host(p.output), H.host(p.mask_output)
 
-    for beta, relu in ((0.0, False), (1.0, True)):
-        base, base_mo = forward(0, beta, relu)
+    bias = H.to_storage(rng.normal(0, 1, size=(k_out,)).astype(np.float32), dtype)
+    for beta, relu, with_bias in ((0.0, False, False), (1.0, True, False), (1.0, True, True)):
+        base, base_mo = forward(0, beta, relu, with_bias)
         ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(
             feat, w, out0, pt.indices_fwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype, dtype_out=dtype,
-            beta=beta, act=onm.ACT_RELU if relu else onm.ACT_NONE)
+            beta=beta, bias=bias if with_bias else None, act=onm.ACT_RELU if relu else onm.ACT_NONE)
         assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref, dtype)) < TOL
         np.testing.assert_array_equal(base_mo, ref_mo)
         for hint in hints[1:]:
-            got, got_mo = forward(hint, beta, relu)
+            got, got_mo = forward(hint, beta, relu, with_bias)
             np.testing.assert_array_equal(got.view(np.uint16), base.view(np.uint16), err_msg="hint %d" % hint)
             np.testing.assert_array_equal(got_mo, base_mo, err_msg="hint %d" % hint)
 
@@ -215,6 +218,53 @@ def test_light_prefix_hint_moves_work_not_results(dtype, c_in, k_out):
         assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref, dtype)) < TOL
         for hint in hints[1:]:
             np.testing.assert_array_equal(backward_input(hint).view(np.uint16), base.view(np.uint16), err_msg="hint %d" % hint)
+
+
+def test_light_prefix_leaves_skipped_rows_alone():
+    """Backward-input of a stride-2 layer without padding: inputs on the last plane of an even axis
+    feed no output, their masks are zero and lead the sorted order, and whole 64-row tiles of them
+    are skipped (the caller zero-fills).  With the hint those positions sit in 128-row tiles: a
+    half without any offset must stay untouched there as well - the gradient buffer starts from
+    a sentinel here and has to come back the same with and without the hint."""
+    print("case light_prefix strided backward-input", flush=True)
+    dtype, c_in, k_out = "f16", 64, 64
+    rng = np.random.default_rng(12)
+    grid = (12, 40, 36)
+    coords = synth.clustered_voxels(rng, 2500, grid, 6, sigma=3.0)
+    zz, yy = np.meshgrid(np.arange(grid[0]), np.arange(grid[1]), indexing="ij")
+    plane = np.stack([np.zeros(zz.size, np.int64), zz.ravel(), yy.ravel(), np.full(zz.size, grid[2] - 1)], axis=1)
+    z2, x2 = np.meshgrid(np.arange(grid[0]), np.arange(7), indexing="ij")      # a strip of the last y plane as well
+    edge = np.stack([np.zeros(z2.size, np.int64), z2.ravel(), np.full(z2.size, grid[1] - 1), x2.ravel()], axis=1)
+    coords = np.unique(np.concatenate([coords, plane.astype(np.int32), edge.astype(np.int32)]), axis=0).astype(np.int32)
+    pt = pairs.sparse_conv_pairs(coords, grid, padding=(0, 0, 0))
+    n_in, n_out = coords.shape[0], pt.indices_fwd.shape[1]
+    ms, order = pairs.sort_by_mask(pt.mask_bwd)
+    empty = int((ms == 0).sum())
+    assert empty >= 3 * 64 and (empty // 64) % 2 == 1, "an odd number of empty tiles: one 128-run is half empty"
+    exact = pairs.light_prefix(ms)
+    assert exact >= 256
+    w = H.to_storage(rng.normal(0, 0.05, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    sentinel = H.to_storage(np.full((n_in, c_in), 7.0, np.float32), dtype)
+
+    def run(hint):
+        p = ConvParams(3, ConvOpType.BackwardInput)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, 64, 64)
+        din = H.dev(sentinel, dtype)
+        p.input, p.weight, p.output = din, H.dev(w, dtype), H.dev(dout, dtype)
+        p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_bwd, "i32"), H.dev(ms, "u32"), H.dev(order, "i32")
+        p.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(din)
+
+    base = run(0)
+    skipped = order[:(empty // 64) * 64]
+    assert (H.as_f32(base, dtype)[skipped] == 7.0).all()
+    ref = conv_ref.implicit_gemm_dgrad_ref(dout, w, sentinel, pt.indices_bwd, ms, order, tile_m=64, dtype_in=dtype,
+                                           dtype_w=dtype, dtype_out=dtype, reverse_mask=False)
+    assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref, dtype)) < TOL
+    for hint in (exact, 128, (empty // 128 + 1) * 128, n_in):
+        np.testing.assert_array_equal(run(hint).view(np.uint16), base.view(np.uint16), err_msg="hint %d" % hint)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
