@@ -154,11 +154,14 @@ class SparseConvGeometry:
             self.out_coords, self.out_shape = tensor2torch(t.out_coords, clone=False), t.out_shape
         self.indices_fwd, self.indices_bwd = t.indices_fwd, t.indices_bwd
         self.n_out = int(t.indices_fwd.dim(1))
-        self.mask_fwd, self.order_fwd = pairs.sort_by_mask_device(t.mask_fwd, stream=stream)
+        # (a mask has one bit per kernel offset: a filter of that width spares the sort the passes over
+        # the bits above it)
+        bits = (1 << self.kv) - 1 if self.kv < 32 else 0xFFFFFFFF
+        self.mask_fwd, self.order_fwd = pairs.sort_by_mask_device(t.mask_fwd, mask_filter=bits, stream=stream)
         if self.subm:      # the forward masks serve the backward-input pass, bit-reversed in the kernel
             self.mask_bwd, self.order_bwd = self.mask_fwd, self.order_fwd
         else:
-            self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, stream=stream)
+            self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, mask_filter=bits, stream=stream)
         # how far the light end of each sorted order reaches (the forward / backward-input launches
         # take it as a hint; one number each comes back to the host here)
         self.light_fwd = pairs.light_prefix_device(self.mask_fwd, stream=stream)
