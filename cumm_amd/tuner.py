@@ -42,6 +42,14 @@ def _density_bucket(num_pairs: Optional[int], n: int) -> int:
     return int(math.floor(2.0 * math.log2(max(float(num_pairs) / float(n), 1.0))))
 
 
+def _light_bucket(light_prefix: int, n: int) -> int:
+    """Quarter of the positions that the light_prefix hint covers (0 .. 4): with a long light end
+    the 64-row descriptors run two tile shapes and rank differently against the others."""
+    if n <= 0 or light_prefix <= 0:
+        return 0
+    return min(4, 1 + (4 * int(light_prefix)) // (n + 1))
+
+
 def conv_candidates(params: ConvParams, desps: Optional[List[ConvAlgoDesp]] = None) -> List[ConvAlgoDesp]:
     """Descriptors of the same kind as ``params.conv_algo_desp`` that accept the problem."""
     cur = params.conv_algo_desp
@@ -130,7 +138,7 @@ class Tuner:
         return ("conv", ConvOpType(d.op_type).value, d.dtype_a, d.dtype_b, d.dtype_c, bool(d.is_int8_inference),
                 params.input.dim(1), params.weight.dim(0), params.weight.dim(1), _bucket(n),
                 _density_bucket(num_pairs, n), params.split_k_slices > 1, params.mask_width,
-                bool(params.reverse_mask))
+                bool(params.reverse_mask), _light_bucket(getattr(params, "light_prefix", 0), n))
 
     def tune_conv(self, params: ConvParams, desps: Optional[List[ConvAlgoDesp]] = None,
                   num_pairs: Optional[int] = None) -> TuneResult:

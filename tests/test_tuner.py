@@ -51,6 +51,12 @@ def test_conv_candidates_share_the_kind_and_accept_the_problem():
     assert tuner.Tuner.conv_key(p, num_pairs=2 * n) != tuner.Tuner.conv_key(p, num_pairs=20 * n)
     assert tuner.Tuner.conv_key(p, num_pairs=2 * n) == tuner.Tuner.conv_key(p, num_pairs=int(2.2 * n))
     assert tuner.Tuner.conv_key(p, num_pairs=2 * n) != k1      # unknown density is its own class
+    # the light_prefix hint changes how the 64-row descriptors run: its share of the positions is in the key
+    hinted = tuner.Tuner.conv_key(p)
+    p.light_prefix = (n // 128) * 128
+    assert tuner.Tuner.conv_key(p) != hinted
+    p.light_prefix = 0
+    assert tuner.Tuner.conv_key(p) == hinted
 
 
 def test_gemm_candidates():
