@@ -47,6 +47,10 @@ struct SortParams {
   uint32_t *dst_keys;
   int32_t *dst_vals;
   int32_t pass;
+  // chunks are handed out by ticket (a chunk's predecessors have then always started); with no more
+  // chunks than the device runs workgroups at once every chunk is resident anyway and a chunk is
+  // its workgroup's number: one atomic round trip less per pass
+  int32_t use_tickets;
 };
 
 __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortParams p) {
@@ -75,6 +79,16 @@ __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortPara
     }
 #pragma unroll
     for (int u = 0; u < kItems; ++u) {
+      // a wave whose 64 keys are one word (the centre-only masks of a sparse cloud: most waves) adds
+      // once per digit without looking for its peers
+      const unsigned long long live = __ballot(valids[u]);
+      if (live == 0ull) continue;
+      const uint32_t first_key = (uint32_t)__builtin_amdgcn_readlane((int)keys[u], __builtin_ctzll(live));
+      if (__ballot(valids[u] && keys[u] == first_key) == live) {
+        if (lane < p.passes)
+          atomicAdd(&lds_hist[lane][(first_key >> (lane * kRadixBits)) & (kBins - 1)], (uint32_t)__popcll(live));
+        continue;
+      }
       for (int q = 0; q < p.passes; ++q) {
         const uint32_t d = (keys[u] >> (q * kRadixBits)) & (kBins - 1);
         unsigned long long peers = __ballot(valids[u]);
@@ -109,7 +123,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int shift = p.pass * kRadixBits;
 
-  if (t == 0) chunk_of_block = (int)atomicAdd(&p.tickets[p.pass], 1u);
+  if (t == 0) chunk_of_block = p.use_tickets ? (int)atomicAdd(&p.tickets[p.pass], 1u) : (int)blockIdx.x;
 #pragma unroll
   for (int w = 0; w < kSortWaves; ++w) wave_hist[w][t] = 0u;
   // exclusive prefix over the digit values of the whole input: thread = bin; a scan inside each
@@ -306,6 +320,18 @@ hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uin
   p.state = reinterpret_cast<uint32_t *>(base + 2 * words + align256s(4 * 4 * kBins) + 256);
   p.give_ups = give_ups;
   p.src_keys = nullptr; p.src_vals = nullptr; p.dst_keys = nullptr; p.dst_vals = nullptr; p.pass = 0;
+  {
+    static int cus_of[16] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    int &cus = cus_of[dev & 15];
+    if (cus == 0) {
+      e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      if (e != hipSuccess) return e;
+    }
+    p.use_tickets = p.chunks > cus ? 1 : 0;   // (a pass workgroup fits a CU: one resident per CU at least)
+  }
   hipLaunchKernelGGL(sort_clear_hist_kernel, dim3((4 * kBins + 255) / 256), dim3(256), 0, s, p.hist, 4 * kBins);
   int setup_blocks = p.chunks < 512 ? p.chunks : 512;
   hipLaunchKernelGGL(sort_setup_kernel, dim3(setup_blocks), dim3(kSortThreads), 0, s, p);
