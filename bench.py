@@ -469,6 +469,13 @@ def bench_pairs(args, coords):
     steps, warm = max(5, args.steps // 4), max(2, args.warmup // 4)
     w1, e1 = timed(pairs_step, steps, warm)
     w2, e2 = timed(sort_step, steps, warm)
+    # the light prefix of the sorted masks (the hint of the forward / backward-input launches): two small launches
+    prefix = tv.empty([1], tv.int32, 0)
+
+    def prefix_step():
+        _capi.check(lib.cumm_hip_light_prefix(smask.byte_pointer(), n, 0xFFFFFFFF, prefix.byte_pointer(), 0))
+
+    w2b, e2b = timed(prefix_step, steps, warm)
     # regular (strided) convolution on the voxel set of the s8 leg: active output sites (with the
     # one synchronisation that returns their number), then the tables
     c4 = synth.clustered_voxels(np.random.default_rng(SEED + 4), 300000, GRID, 60, sigma=15.0, noise_frac=0.10)
@@ -501,6 +508,8 @@ def bench_pairs(args, coords):
                            "hbm_frac": round(bytes1 / (e1 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
             "sort_by_mask": {"ms_per_step": round(w2, 5), "kernel_ms_events": round(e2, 5),
                              "hbm_frac": round(bytes2 / (e2 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+            "light_prefix": {"ms_per_step": round(w2b, 5), "kernel_ms_events": round(e2b, 5),
+                             "positions": int(prefix.cpu().numpy()[0])},
             "sparse_conv_pairs_stride2": {"voxels_in": n4, "voxels_out": m4, "ms_per_step": round(w3, 5),
                                           "mvoxels_per_s": round(n4 / (w3 * 1e-3) / 1e6, 1),
                                           "hbm_frac": round(bytes3 / (w3 * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
