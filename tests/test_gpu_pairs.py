@@ -201,3 +201,20 @@ def test_sort_by_mask_against_stable_argsort(n, kind):
         np.testing.assert_array_equal(H.host(order), order_ref)
     from cumm_amd.gemm.main import GemmMainUnitTest
     GemmMainUnitTest.device_synchronize()      # (would raise if a look-back had given up)
+
+
+@pytest.mark.parametrize("n", [1, 127, 128, 1000, 4096, 50001])
+def test_light_prefix_against_the_host_count(n):
+    """cumm_hip_light_prefix against pairs.light_prefix: sorted arrays whose light end has a random
+    length (centre-only words, a few with one more offset), followed by words of many offsets;
+    with filters that turn heavy words light."""
+    print("case light prefix", n, flush=True)
+    rng = np.random.default_rng(n)
+    for light_len in (0, n // 3, n - n // 7, n):
+        light = np.full(light_len, 1 << 13, np.uint32)
+        light[rng.random(light_len) < 0.05] |= np.uint32(1 << 14)
+        heavy = (rng.integers(1, 1 << 13, size=n - light_len, dtype=np.uint32) | np.uint32(1 << 13) | np.uint32(7 << 20))
+        mask = np.sort(np.concatenate([light, heavy]))
+        d = H.dev(mask, "u32")
+        for filt in (0xFFFFFFFF, 0x6000, 1 << 13, 0x1FFF):
+            assert pairs.light_prefix_device(d, mask_filter=filt) == pairs.light_prefix(mask, filt), (light_len, hex(filt))
