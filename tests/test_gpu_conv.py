@@ -452,22 +452,32 @@ def test_int8_inference_bit_exact(tile, strided):
 
 
 def test_ragged_and_empty():
-    """N not a multiple of the tile and a single voxel."""
+    """N not a multiple of the tile and a single voxel; each also with light_prefix hints that cover
+    nothing, one run of 128, everything and more (few rows: the hint is cut to the whole runs)."""
     dtype = "f16"
     desp = H.find_conv_desp(dtype, ConvOpType.Forward, 64, 64)
-    for n in (1, 65, 130):
+    for n in (1, 65, 130, 257, 300):
         rng, coords, pt, feat, w, n_in, n_out = _case(6 + n, n, 64, 64, dtype, grid=(6, 10, 10))
         ms, order = pairs.sort_by_mask(pt.mask_fwd)
         out0 = H.to_storage(np.zeros((n_out, 64), np.float32), dtype)
-        p = ConvParams(3, ConvOpType.Forward)
-        p.conv_algo_desp = desp
-        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
-        p.indices = H.dev(pt.indices_fwd, "i32")
-        p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
-        ConvMainUnitTest.implicit_gemm2(p)
-        ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64,
-                                                dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
-        assert H.rel_err(H.as_f32(H.host(p.output), dtype), H.as_f32(ref, dtype)) < TOL
+        ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=64,
+                                                     dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+        first = None
+        for hint in (0, 128, 200, n_out, n_out + 500):
+            p = ConvParams(3, ConvOpType.Forward)
+            p.conv_algo_desp = desp
+            p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+            p.indices = H.dev(pt.indices_fwd, "i32")
+            p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+            p.mask_output = tv.zeros([(n_out + 63) // 64], tv.uint32, 0)
+            p.light_prefix = hint
+            ConvMainUnitTest.implicit_gemm2(p)
+            got = H.host(p.output)
+            assert H.rel_err(H.as_f32(got, dtype), H.as_f32(ref, dtype)) < TOL
+            np.testing.assert_array_equal(H.host(p.mask_output), ref_mo)
+            if first is None:
+                first = got
+            np.testing.assert_array_equal(got.view(np.uint16), first.view(np.uint16), err_msg="n %d hint %d" % (n, hint))
 
 
 @pytest.mark.parametrize("geometry", [
