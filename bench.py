@@ -127,8 +127,10 @@ def bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops):
     w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pd), args.steps, args.warmup)
     pd.light_prefix = 0
     w0_ms, e0_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pd), args.steps, args.warmup)
+    alg = n * K * 2 + n * C * 2 + 27 * C * K * 2 + 27 * n * 4 + n * 8     # gradient rows in, rows out, weights, table, masks
     return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
-            "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3), "kernel_ms_events_without_light_prefix": round(e0_ms, 5)}
+            "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3), "kernel_ms_events_without_light_prefix": round(e0_ms, 5),
+            "hbm_frac": round(alg / (e_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
 
 def bench_wgrad(args, p, dout, n, C, K, tile_m, flops, parallel, fixed_order=False):
@@ -144,8 +146,10 @@ def bench_wgrad(args, p, dout, n, C, K, tile_m, flops, parallel, fixed_order=Fal
     div = 1 if parallel else 4
     w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), max(1, args.steps // div),
                        max(1, args.warmup // div))
+    alg = n * C * 2 + n * K * 2 + 27 * n * 4 + n * 4 + 4 * ((n + tile_m - 1) // tile_m) + 27 * C * K * 2
     return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
-            "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3)}
+            "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3),
+            "hbm_frac": round(alg / (e_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
 
 def find_gemm_desp(shuffle, tile_m, tile_n, trans_b):
