@@ -56,7 +56,8 @@ class SparseConvArgs(C.Structure):
                 ("kernel_volume", C.c_int32), ("mode", C.c_int32), ("groups", C.c_int32),
                 ("d_is_bias", C.c_int32), ("deterministic", C.c_int32),
                 ("bias_pointer", C.c_void_p), ("scale_pointer", C.c_void_p),
-                ("rows_in", C.c_int32), ("rows_out", C.c_int32), ("light_prefix", C.c_int32)]
+                ("rows_in", C.c_int32), ("rows_out", C.c_int32), ("light_prefix", C.c_int32),
+                ("ungated_rows", C.c_int32), ("indices_by_position", C.c_int32), ("reserved_", C.c_int32)]
 
 
 # every symbol include/cumm_hip.h declares: name -> (restype, argtypes)
@@ -99,6 +100,7 @@ SYMBOLS = {
                                       _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP]),
     "cumm_hip_sort_by_mask_workspace": (C.c_size_t, [C.c_int]),
     "cumm_hip_sort_by_mask": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_pairs_by_position": (C.c_int, [_VP, _VP, C.c_int, C.c_int, _VP, _VP]),
     "cumm_hip_light_prefix": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP]),
     "cumm_hip_conv_pairs_workspace": (C.c_size_t, [C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5),
     "cumm_hip_conv_pairs_sites": (C.c_int, [_VP, C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5 +

@@ -234,6 +234,9 @@ class ConvMainUnitTest:
         args.rows_in, args.rows_out = inp.dim(0), output.dim(0)
         args.light_prefix = max(0, min(int(getattr(params, "light_prefix", 0)), N)) \
             if op_type != ConvOpType.BackwardWeight else 0
+        args.ungated_rows = int(bool(getattr(params, "ungated_rows", False)))
+        args.indices_by_position = int(bool(getattr(params, "indices_by_position", False))) \
+            if op_type != ConvOpType.BackwardWeight else 0
         cdesc = conv_desp_to_c(desp)
         name = repr(desp) if params.timer.enable else ""
         if name:

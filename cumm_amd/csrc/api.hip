@@ -634,7 +634,10 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     p.act = a->act_type;
     p.read_source = a->beta != 0.0f;
     // (the hint only moves work between tile shapes; whatever it says the kernel covers every position once)
-    p.pair_tiles = a->light_prefix > 0 ? a->light_prefix / 128 : 0;
+    p.pair_tiles = a->light_prefix > 0 && !a->ungated_rows ? a->light_prefix / 128 : 0;
+    p.ungated_rows = a->ungated_rows != 0;
+    p.gather_by_pos = a->indices_by_position != 0;
+    p.n_mask_out = p.mask_out ? (a->N + d.tile_shape[0] - 1) / d.tile_shape[0] : 0;
     if (c.is_int8_inference) {
       if (!a->bias_pointer || !a->scale_pointer)
         return fail(CUMM_HIP_ERUNTIME, "int8 inference must have both scale and bias");
@@ -1219,6 +1222,17 @@ int cumm_hip_pair_lists(const int32_t *indices, int kv, int n, int32_t *pair_in,
   p.kv = kv; p.n = n; p.chunks = (n + kPairListChunk - 1) / kPairListChunk;
   hipError_t e = launch_pair_lists(p, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "pair list launch");
+  return CUMM_HIP_OK;
+}
+
+int cumm_hip_pairs_by_position(const int32_t *indices, const int32_t *mask_argsort, int kv, int n, int32_t *out,
+                               void *stream) {
+  if (kv < 0 || n < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (kv == 0 || n == 0) return CUMM_HIP_OK;
+  if (!indices || !mask_argsort || !out) return fail(CUMM_HIP_EINVAL, "indices, mask_argsort and out must not be empty");
+  if (out == indices) return fail(CUMM_HIP_EINVAL, "out must not be the table itself");
+  hipError_t e = launch_pairs_by_position(indices, mask_argsort, out, kv, n, n, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "pair table permutation launch");
   return CUMM_HIP_OK;
 }
 

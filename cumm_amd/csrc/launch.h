@@ -107,6 +107,8 @@ struct PairListsParams {
   int32_t *chunk_counts;    // [kv, chunks] scratch
   int32_t kv, n, chunks;
 };
+hipError_t launch_pairs_by_position(const int32_t *indices, const int32_t *argsort, int32_t *out, int kv, int n, int rows,
+                                    hipStream_t s);
 constexpr int kPairListChunk = 2048;   // table entries per workgroup
 hipError_t launch_pair_lists(const PairListsParams &p, hipStream_t s);
 

@@ -454,7 +454,25 @@ __global__ __launch_bounds__(256) void pair_lists_write_kernel(const PairListsPa
   }
 }
 
+// out[k][pos] = indices[k][argsort[pos]]: the pair table in the order of the sorted positions
+__global__ __launch_bounds__(256) void pairs_by_position_kernel(const int32_t *__restrict__ indices,
+                                                                const int32_t *__restrict__ argsort,
+                                                                int32_t *__restrict__ out, int n, int rows) {
+  const int pos = blockIdx.x * 256 + threadIdx.x;
+  if (pos >= n) return;
+  const int row = argsort[pos];
+  const int64_t k = blockIdx.y;
+  out[k * n + pos] = row >= 0 && row < rows ? indices[k * rows + row] : -1;
+}
+
 }  // namespace
+
+hipError_t launch_pairs_by_position(const int32_t *indices, const int32_t *argsort, int32_t *out, int kv, int n, int rows,
+                                    hipStream_t s) {
+  if (kv <= 0 || n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(pairs_by_position_kernel, dim3((n + 255) / 256, kv), dim3(256), 0, s, indices, argsort, out, n, rows);
+  return hipGetLastError();
+}
 
 hipError_t launch_pair_lists(const PairListsParams &p, hipStream_t s) {
   if (p.kv <= 0) return hipSuccess;

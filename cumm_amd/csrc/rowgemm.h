@@ -62,6 +62,12 @@ struct RowGemmParams {
   // LDS-streaming kernel, one column block: the first pair_tiles runs of 128 sorted positions are
   // taken as 128-row tiles (rowgemm_lds_mixed_kernel); 0 = 64-row tiles throughout
   int32_t pair_tiles;
+  // words the caller's mask_out array holds (a tile number beyond it is not written)
+  int32_t n_mask_out;
+  // non-zero: a row takes part in every kernel offset of its tile's mask (the reference's rule:
+  // rows are gated by their pair-table entry alone, cumm/conv/sparse_iters.py:629-631), instead of
+  // only in the offsets whose bit its own mask word has
+  int32_t ungated_rows;
 };
 
 // An offset no buffer contains: every operand is smaller than 2 GiB (checked on the host), and
@@ -153,7 +159,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_kernel(const RowGemmParams p)
     }
     kmask = wave_or(mk) & p.mask_filter;
     kmask = __builtin_amdgcn_readfirstlane(kmask);
-    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
+    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0 && tile < p.n_mask_out) p.mask_out[tile] = kmask;
     if (p.exit_on_empty && kmask == 0) return;
     if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
     if (p.kv < 32) kmask &= (1u << p.kv) - 1u;

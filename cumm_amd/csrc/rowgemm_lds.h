@@ -192,7 +192,7 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   auto row_bits = [&](int raw) -> uint32_t {
     const uint32_t w = (uint32_t)raw;
     const uint32_t wr = __builtin_bitreverse32(w) >> ((32 - p.kv) & 31);
-    return has_mask ? (p.reverse_mask ? wr : w) : ~0u;
+    return has_mask && !p.ungated_rows ? (p.reverse_mask ? wr : w) : ~0u;
   };
   // memory row of a sorted position (the position itself without an argsort), -1 past the end
   auto row_of = [&](int pos, int raw) -> int { return pos < p.n_pos ? (has_rows ? raw : pos) : -1; };
@@ -216,11 +216,11 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
       const uint32_t hi = wave_or_dpp((uint32_t)raw_mk[MKW - 1]) & p.mask_filter;
       half_skipped = p.exit_on_empty && (wm == 0 ? lo : hi) == 0u;
       if (p.mask_out != nullptr && tid == 0 && col == 0) {
-        p.mask_out[2 * tile] = lo;
-        if ((2 * tile + 1) * 64 < p.n_pos) p.mask_out[2 * tile + 1] = hi;
+        if (2 * tile < p.n_mask_out) p.mask_out[2 * tile] = lo;
+        if ((2 * tile + 1) * 64 < p.n_pos && 2 * tile + 1 < p.n_mask_out) p.mask_out[2 * tile + 1] = hi;
       }
     } else {
-      if (p.mask_out != nullptr && tid == 0 && col == 0) p.mask_out[tile] = kmask;
+      if (p.mask_out != nullptr && tid == 0 && col == 0 && tile < p.n_mask_out) p.mask_out[tile] = kmask;
     }
     if (p.exit_on_empty && kmask == 0) return;
     if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);

@@ -75,7 +75,7 @@ __global__ __launch_bounds__(NW * 64) void rowgemm_pipe_kernel(const RowGemmPara
     }
     kmask = wave_or(mk) & p.mask_filter;
     kmask = __builtin_amdgcn_readfirstlane(kmask);
-    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0) p.mask_out[tile] = kmask;
+    if (p.mask_out != nullptr && tid == 0 && blockIdx.y == 0 && tile < p.n_mask_out) p.mask_out[tile] = kmask;
     if (p.exit_on_empty && kmask == 0) return;
     if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
     if (p.kv < 32) kmask &= (1u << p.kv) - 1u;

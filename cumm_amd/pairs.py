@@ -163,6 +163,13 @@ def light_prefix(sorted_mask: np.ndarray, mask_filter: int = 0xFFFFFFFF) -> int:
     return int(heavy[0] if heavy.size else runs) * 128
 
 
+def pairs_by_position(indices: np.ndarray, mask_argsort: np.ndarray) -> np.ndarray:
+    """The pair table in the order of the sorted positions: ``out[k][pos] = indices[k][mask_argsort[pos]]``
+    (what ``ConvParams.indices_by_position`` takes; the reference's iterator forms this index per
+    access, cumm/conv/sparse_iters.py:280-357)."""
+    return np.ascontiguousarray(np.asarray(indices)[:, np.asarray(mask_argsort, np.int64)])
+
+
 class PairLists(NamedTuple):
     pair_in: np.ndarray    # [kv, N] int32: input rows of offset k's pairs, packed to the front
     pair_out: np.ndarray   # [kv, N] int32: their output rows (ascending)
@@ -329,6 +336,25 @@ def light_prefix_device(sorted_mask, mask_filter: int = 0xFFFFFFFF, stream: int 
                                           int(mask_filter) & 0xFFFFFFFF, res.byte_pointer(), stream))
     _capi.check(lib.cumm_hip_stream_synchronize(stream))
     return int(res.cpu().numpy()[0])
+
+
+def pairs_by_position_device(indices, mask_argsort, out=None, stream: int = 0):
+    """:func:`pairs_by_position` of device tensors ``indices`` [kv, N] int32 and ``mask_argsort``
+    [N] int32, in stream order; ``out`` ([kv, N] int32) is filled when given."""
+    from . import _capi
+    from . import tensorview as tv
+    if indices.device < 0 or indices.dtype != tv.int32 or indices.ndim != 2:
+        raise ValueError("indices must be a device int32 tensor [kv, N]")
+    kv, n = int(indices.shape[0]), int(indices.shape[1])
+    if mask_argsort.device < 0 or mask_argsort.dtype != tv.int32 or list(mask_argsort.shape) != [n]:
+        raise ValueError("mask_argsort must be a device int32 vector [N]")
+    if out is None:
+        out = tv.empty([kv, n], tv.int32, 0)
+    elif out.device < 0 or out.dtype != tv.int32 or list(out.shape) != [kv, n]:
+        raise ValueError("out must be a device int32 tensor [kv, N]")
+    _capi.check(_capi.lib().cumm_hip_pairs_by_position(indices.byte_pointer(), mask_argsort.byte_pointer(), kv, n,
+                                                       out.byte_pointer(), stream))
+    return out
 
 
 class DevicePairLists(NamedTuple):

@@ -470,4 +470,12 @@ class ConvParams(_Versioned):
         # leading positions of the sorted order in tiles of one or two kernel offsets
         # (pairs.light_prefix of the sorted mask); 0 = unknown.  Any value gives the same result.
         self.light_prefix = 0
+        # not in the reference's struct: True = every position of a tile takes part in every kernel
+        # offset of the tile's OR-ed mask (gated by its pair-table entry alone, the reference's
+        # rule); False (default) = only in the offsets whose bit its own mask word has, which is
+        # the same thing for masks made from the pair table and fetches less
+        self.ungated_rows = False
+        # not in the reference's struct: True = ``indices`` is the pair table in the order of the
+        # sorted positions (pairs.pairs_by_position[_device]); forward / backward-input
+        self.indices_by_position = False
         self.nvrtc_params = NVRTCParams()

@@ -131,6 +131,22 @@ typedef struct CummHipSparseConvArgs {
                                        positions to 128-row tiles (fewer, longer-lived workgroups where a tile's
                                        time is its memory round trips); any value gives the same bits, a wrong one
                                        costs time.  No counterpart in the reference. */
+  int32_t ungated_rows;             /* forward / backward-input.  0: a position takes part in kernel offset k only if its
+                                       own mask word has bit k - masks made from the pair table (bit k set wherever
+                                       indice_ptr[k][row] >= 0, as spconv makes them) lose nothing, and entries and rows
+                                       of the other offsets are never fetched.  Non-zero: every position of a tile takes
+                                       part in every offset of the tile's OR-ed mask and is gated by its pair-table entry
+                                       alone - the reference's rule (cumm/conv/sparse_iters.py:629-631), which differs
+                                       from the above only for masks with a bit clear over a valid entry; slower
+                                       (the hint light_prefix is then ignored). */
+  int32_t indices_by_position;      /* forward / backward-input.  Non-zero: indice_ptr is the pair table in the order of
+                                       the sorted positions, [kernel_volume, N] with entry [k][pos] = the reference
+                                       table's [k][mask_argsort_ptr[pos]] (cumm_hip_pairs_by_position makes it, once per
+                                       geometry and sort).  A tile's entries for one offset are then consecutive in
+                                       memory instead of one memory sector apiece.  Same results either way.  No
+                                       counterpart in the reference, whose iterator reads the table by output row
+                                       (cumm/conv/sparse_iters.py:280-357). */
+  int32_t reserved_;
 } CummHipSparseConvArgs;
 
 /* Replaces GemmMainUnitTest.matmul2 below its prelude
@@ -291,6 +307,15 @@ int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, co
 size_t cumm_hip_pair_lists_workspace(int kv, int n);
 int cumm_hip_pair_lists(const int32_t *indices, int kv, int n, int32_t *pair_in, int32_t *pair_out, int32_t *counts,
                         void *workspace, size_t workspace_bytes, void *stream);
+
+/* The pair table in the order of the sorted positions: out[k][pos] = indices[k][mask_argsort[pos]] for
+ * indices [kv, n] and mask_argsort [n] (an argsort entry outside [0, n) gives -1); out [kv, n], not the
+ * table itself.  What CummHipSparseConvArgs.indices_by_position takes: one pass per geometry and sort,
+ * after which the entries a tile reads for one kernel offset are consecutive.  No counterpart in the
+ * reference (its iterator reads indices[k][mask_argsort[pos]] per access,
+ * cumm/conv/sparse_iters.py:280-357). */
+int cumm_hip_pairs_by_position(const int32_t *indices, const int32_t *mask_argsort, int kv, int n, int32_t *out,
+                               void *stream);
 
 /* ---- stand-alone row gather / scatter-add (the "native" per-offset path around a plain GEMM)
  * cumm_hip_gather_rows: output[i, :] = input[indices[i], :] for i < m; rows of row_bytes bytes

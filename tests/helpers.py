@@ -44,10 +44,17 @@ def host(t):
 
 
 def rel_err(got_f32, ref_f32):
-    """max |got-ref| / max |ref|: the reference's own criterion
-    (cumm/gemm/main_real.py:672-677)."""
-    denom = max(float(np.max(np.abs(ref_f32))), 1e-6)
-    return float(np.max(np.abs(got_f32.astype(np.float64) - ref_f32.astype(np.float64)))) / denom
+    """The larger of two figures: max |got-ref| / max |ref| over the whole tensor - the reference's
+    own criterion (cumm/gemm/main_real.py:672-677) - and the same per row (:func:`rel_err_rows`),
+    so that a wrong row of small magnitude cannot hide under the tensor's largest value."""
+    got_f32, ref_f32 = np.asarray(got_f32), np.asarray(ref_f32)
+    denom = max(float(np.max(np.abs(ref_f32))), 1e-6) if ref_f32.size else 1.0
+    if ref_f32.size == 0:
+        return 0.0
+    whole = float(np.max(np.abs(got_f32.astype(np.float64) - ref_f32.astype(np.float64)))) / denom
+    if ref_f32.ndim == 0:
+        return whole
+    return max(whole, rel_err_rows(got_f32, ref_f32))
 
 
 def rel_err_rows(got_f32, ref_f32, floor_frac=1e-2):

@@ -711,3 +711,154 @@ def test_long_contraction_forward_and_backward_input(dtype):
         dout, w2, din0, pt.indices_bwd, ms, order, tile_m=64, dtype_in=dtype, dtype_w=dtype,
         dtype_out=dtype, reverse_mask=True)
     assert H.rel_err(H.as_f32(H.host(q.input), dtype), H.as_f32(ref_d, dtype)) < TOL
+
+
+@pytest.mark.parametrize("dtype,tile", [("f16", (64, 64)), ("bf16", (128, 128)), ("s8", (64, 128))])
+def test_mask_bit_clear_over_a_valid_entry(dtype, tile):
+    """Where this library narrows the reference's mask contract, as a tested fact.  The reference
+    walks the kernel offsets of a tile's OR-ed mask and gates each row by its pair-table entry
+    alone (cumm/conv/sparse_iters.py:629-631); the oracle does the same.  The LDS-streaming
+    kernels here let a position take part in offset k only if its OWN mask word has bit k.  For
+    masks made from the pair table (bit k wherever the entry is valid) the two rules are the
+    same thing.  This test clears bits over valid entries in a third of the words:
+      * default: the result is the oracle's on a pair table whose entries under a cleared bit
+        are removed (and it differs from the oracle on the table as given);
+      * ``ungated_rows``: the result is the oracle's on the table as given (the reference's
+        rule), with the same ``mask_output``."""
+    print("case cleared mask bits", dtype, tile, flush=True)
+    c_in, k_out = (64, 128) if dtype == "s8" else (64, 64)
+    rng, coords, pt, feat, w, n_in, n_out = _case(31, 3000, c_in, k_out, dtype)
+    mask = pt.mask_fwd.copy()
+    victims = rng.permutation(n_out)[:n_out // 3]
+    for o in victims:
+        bits = [k for k in range(27) if k != 13 and (mask[o] >> k) & 1]
+        if bits:
+            mask[o] &= ~np.uint32(1 << int(rng.choice(bits)))
+    assert (mask != pt.mask_fwd).sum() > 100
+    ms, order = pairs.sort_by_mask(mask)
+    # the table with the entries under a cleared bit removed
+    gated = pt.indices_fwd.copy()
+    for k in range(27):
+        gated[k][((mask >> np.uint32(k)) & 1) == 0] = -1
+    kw = dict(tile_m=tile[0], dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+    scale = bias = None
+    if dtype == "s8":
+        scale = rng.uniform(0.001, 0.01, size=(k_out,)).astype(np.float32)
+        bias = rng.normal(0, 1, size=(k_out,)).astype(np.float32)
+        kw.update(scale=scale, bias=bias, int8_inference=True)
+    out0 = np.zeros((n_out, k_out), np.int8) if dtype == "s8" else H.to_storage(np.zeros((n_out, k_out), np.float32), dtype)
+    ref_given, mo_given = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, **kw)
+    ref_gated, mo_gated = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, gated, ms, order, **kw)
+    np.testing.assert_array_equal(mo_given, mo_gated)
+    assert (np.asarray(ref_given) != np.asarray(ref_gated)).any(), "the case must tell the two rules apart"
+
+    def run(ungated):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, *tile, int8_inference=dtype == "s8")
+        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+        if dtype == "s8":
+            p.scale, p.bias = H.dev(scale, "f32"), H.dev(bias, "f32")
+        p.indices = H.dev(pt.indices_fwd, "i32")
+        p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+        p.mask_output = tv.zeros([(n_out + tile[0] - 1) // tile[0]], tv.uint32, 0)
+        p.ungated_rows = ungated
+        p.light_prefix = pairs.light_prefix(ms)     # (ignored with ungated_rows)
+        ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(p.output), H.host(p.mask_output)
+
+    got, mo = run(False)
+    got_u, mo_u = run(True)
+    np.testing.assert_array_equal(mo, mo_gated)
+    np.testing.assert_array_equal(mo_u, mo_given)
+    if dtype == "s8":
+        np.testing.assert_array_equal(got, ref_gated)
+        np.testing.assert_array_equal(got_u, ref_given)
+    else:
+        assert H.rel_err(H.as_f32(got, dtype), H.as_f32(ref_gated, dtype)) < TOL
+        assert H.rel_err(H.as_f32(got_u, dtype), H.as_f32(ref_given, dtype)) < TOL
+        assert H.rel_err(H.as_f32(got, dtype), H.as_f32(ref_given, dtype)) > TOL     # the divergence is real
+
+
+@pytest.mark.parametrize("dtype,tile,c_in,k_out", [("f16", (64, 64), 64, 64), ("f16", (128, 64), 32, 96),
+                                                    ("bf16", (128, 128), 128, 128), ("bf16", (64, 128), 200, 72),
+                                                    ("s8", (64, 128), 64, 128), ("s8", (128, 128), 128, 64)])
+@pytest.mark.parametrize("strided", [False, True])
+def test_pair_table_by_position(dtype, tile, c_in, k_out, strided):
+    """``indices_by_position``: the pair table permuted into the order of the sorted positions
+    (pairs.pairs_by_position_device, bit-exact against the host's fancy indexing) gives the same
+    output bits and tile masks as the table by row, forward and backward-input, with and without
+    the light_prefix hint - and the table by row is checked against the oracle."""
+    print("case pair table by position", dtype, tile, c_in, k_out, strided, flush=True)
+    rng, coords, pt, feat, w, n_in, n_out = _case(33, 3000, c_in, k_out, dtype, strided=strided)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    d_ind, d_order = H.dev(pt.indices_fwd, "i32"), H.dev(order, "i32")
+    d_pos = pairs.pairs_by_position_device(d_ind, d_order)
+    np.testing.assert_array_equal(H.host(d_pos), pairs.pairs_by_position(pt.indices_fwd, order))
+    int8 = dtype == "s8"
+    scale = bias = None
+    kw = dict(tile_m=tile[0], dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+    if int8:
+        scale = rng.uniform(0.001, 0.01, size=(k_out,)).astype(np.float32)
+        bias = rng.normal(0, 1, size=(k_out,)).astype(np.float32)
+        kw.update(scale=scale, bias=bias, int8_inference=True)
+    out0 = np.zeros((n_out, k_out), np.int8) if int8 else H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    beta = 0.0 if int8 else 1.0
+    ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, beta=beta, **kw)
+
+    def forward(by_pos, hint):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, *tile, int8_inference=int8)
+        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+        if int8:
+            p.scale, p.bias = H.dev(scale, "f32"), H.dev(bias, "f32")
+        p.indices = d_pos if by_pos else d_ind
+        p.indices_by_position = by_pos
+        p.mask, p.mask_argsort = H.dev(ms, "u32"), d_order
+        p.mask_output = tv.zeros([(n_out + tile[0] - 1) // tile[0]], tv.uint32, 0)
+        p.beta = beta
+        p.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(p.output), H.host(p.mask_output)
+
+    base, base_mo = forward(False, 0)
+    np.testing.assert_array_equal(base_mo, ref_mo)
+    if int8:
+        np.testing.assert_array_equal(base, ref)
+    else:
+        assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref, dtype)) < TOL
+    for hint in (0, pairs.light_prefix(ms)):
+        got, got_mo = forward(True, hint)
+        np.testing.assert_array_equal(got.view(np.uint8), base.view(np.uint8))
+        np.testing.assert_array_equal(got_mo, base_mo)
+
+    if int8:
+        return
+    # backward-input: the backward table by position of the sort the launch uses
+    if strided:
+        msb, orderb = pairs.sort_by_mask(pt.mask_bwd)
+        reverse = False
+    else:
+        msb, orderb = ms, order
+        reverse = True
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    d_indb, d_orderb = H.dev(pt.indices_bwd, "i32"), H.dev(orderb, "i32")
+    d_posb = pairs.pairs_by_position_device(d_indb, d_orderb)
+
+    def backward_input(by_pos):
+        p = ConvParams(3, ConvOpType.BackwardInput)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, *tile)
+        din = H.dev(H.to_storage(np.zeros((n_in, c_in), np.float32), dtype), dtype)
+        p.input, p.weight, p.output = din, H.dev(w, dtype), H.dev(dout, dtype)
+        p.indices = d_posb if by_pos else d_indb
+        p.indices_by_position = by_pos
+        p.mask, p.mask_argsort = H.dev(msb, "u32"), d_orderb
+        p.reverse_mask = reverse
+        ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(din)
+
+    base = backward_input(False)
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, np.zeros((n_in, c_in), base.dtype), pt.indices_bwd, msb, orderb,
+                                             tile_m=tile[0], dtype_in=dtype, dtype_w=dtype, dtype_out=dtype,
+                                             reverse_mask=reverse)
+    assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref_d, dtype)) < TOL
+    np.testing.assert_array_equal(backward_input(True).view(np.uint16), base.view(np.uint16))

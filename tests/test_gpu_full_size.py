@@ -79,6 +79,64 @@ def test_subm_f16_c64_forward_dgrad_full_size(tile_m):
     assert H.rel_err_rows(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_d, dtype)) < TOL
 
 
+def test_subm_f16_c64_two_tile_shapes_full_size():
+    """The launch the benchmark times: the headline voxel set with the light end of the sorted
+    order in 128-row tiles (``light_prefix`` as input preparation counts it; several hundred
+    128-row tiles next to several hundred 64-row tiles in one launch).  Forward and
+    backward-input: the same output bits and the same ``mask_output`` as the launch without the
+    hint, and within tolerance of the oracle, over the whole tensor and row by row."""
+    print("case full size subm f16, two tile shapes", flush=True)
+    dtype, tile_m = "f16", 64
+    rng, pt, feat, w, n = _subm_case(20240607, 120000, dtype, 64, 64)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    light = pairs.light_prefix(ms)
+    assert light >= 256 and light % 128 == 0 and n - light >= 64 * 100   # both shapes, hundreds of each
+    out0 = np.zeros((n, 64), np.float16)
+    tiles = (n + tile_m - 1) // tile_m
+    d_feat, d_w = H.dev(feat, dtype), H.dev(w, dtype)
+    d_ind, d_ms, d_order = H.dev(pt.indices_fwd, "i32"), H.dev(ms, "u32"), H.dev(order, "i32")
+    d_ms_check = H.dev(ms, "u32")
+    assert pairs.light_prefix_device(d_ms_check) == light
+    outs, mask_outs = [], []
+    for hint in (0, light):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, tile_m, 64)
+        p.input, p.weight, p.output = d_feat, d_w, H.dev(out0, dtype)
+        p.indices, p.mask, p.mask_argsort = d_ind, d_ms, d_order
+        p.mask_output = tv.zeros([tiles], tv.uint32, 0)
+        p.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(p)
+        outs.append(H.host(p.output))
+        mask_outs.append(H.host(p.mask_output))
+    ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=tile_m,
+                                                 dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+    np.testing.assert_array_equal(outs[1].view(np.uint16), outs[0].view(np.uint16))
+    np.testing.assert_array_equal(mask_outs[1], mask_outs[0])
+    np.testing.assert_array_equal(mask_outs[1], ref_mo)
+    got = H.as_f32(outs[1], dtype)
+    assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+    assert H.rel_err_rows(got, H.as_f32(ref, dtype)) < TOL
+
+    dout = H.to_storage(rng.normal(0, 1, size=(n, 64)).astype(np.float32), dtype)
+    din0 = np.zeros((n, 64), np.float16)
+    d_dout, d_indb = H.dev(dout, dtype), H.dev(pt.indices_bwd, "i32")
+    dins = []
+    for hint in (0, light):
+        pd = ConvParams(3, ConvOpType.BackwardInput)
+        pd.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, tile_m, 64)
+        pd.input, pd.weight, pd.output = H.dev(din0, dtype), d_w, d_dout
+        pd.indices, pd.mask, pd.mask_argsort = d_indb, d_ms, d_order
+        pd.reverse_mask = True
+        pd.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(pd)
+        dins.append(H.host(pd.input))
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, din0, pt.indices_bwd, ms, order, tile_m=tile_m,
+                                             dtype_in=dtype, dtype_w=dtype, dtype_out=dtype, reverse_mask=True)
+    np.testing.assert_array_equal(dins[1].view(np.uint16), dins[0].view(np.uint16))
+    assert H.rel_err(H.as_f32(dins[1], dtype), H.as_f32(ref_d, dtype)) < TOL
+    assert H.rel_err_rows(H.as_f32(dins[1], dtype), H.as_f32(ref_d, dtype)) < TOL
+
+
 def test_subm_f16_c64_wgrad_full_size():
     """Backward-weight at the benchmark size with the balanced descriptor and split_k_slices = 32
     (eight fp32 images), on the reduced masks that the forward pass writes."""
@@ -130,6 +188,14 @@ def test_s8_stride2_full_size_bit_exact():
                                                  dtype_w="s8", dtype_out="s8", scale=scale, bias=bias,
                                                  int8_inference=True, return_acc=True)
     np.testing.assert_array_equal(H.host(p.output), ref)
+
+    # the same launch on the pair table in the order of the sorted positions: the same bits
+    p.output = H.dev(out0, "s8")
+    p.indices = pairs.pairs_by_position_device(p.indices, p.mask_argsort)
+    p.indices_by_position = True
+    ConvMainUnitTest.implicit_gemm2(p)
+    np.testing.assert_array_equal(H.host(p.output), ref)
+    p.indices, p.indices_by_position = H.dev(pt.indices_fwd, "i32"), False
 
     # the s32 accumulators themselves ("s8,s8,s32,s32,s32"): bit-exact against the oracle's
     # exact integer sums, and through the integer linear combination with a source
