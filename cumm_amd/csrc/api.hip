@@ -217,11 +217,24 @@ int static_scratch(void **out) {
 
 // ---- failures that a kernel can only report after the fact.  Word 0 counts the serial split-K
 // slices whose bounded semaphore wait ran out (tilegemm.h), word 1 the look-backs of the mask sort
-// that ran into their bound (sort_inst.hip); the synchronising entry points read and clear them and
-// turn a non-zero count into an error.  One array per GPU, like `scratch`.
+// that ran into their bound (sort_inst.hip).  One array per GPU, like `scratch`: the counts are
+// device-wide, whichever stream the launch ran on.  The synchronising entry points take them -
+// one kernel that exchanges every word with zero (nothing counted in between is lost) and writes
+// what it found into pinned host memory, on a stream of the library's own that does not
+// synchronise with the caller's streams - and turn a non-zero count into an error.  Nothing is
+// launched or copied while no launch that could report has run since the last look.
 static __device__ int32_t async_status[4];
 int32_t *g_status_ptr[kMaxDevices] = {};
+int32_t *g_status_host[kMaxDevices] = {};       // pinned, four words per GPU
+hipStream_t g_status_stream[kMaxDevices] = {};
+std::atomic<bool> g_status_armed[kMaxDevices];
 
+__global__ void take_status_kernel(int32_t *status, int32_t *host_words) {
+  const int i = threadIdx.x;
+  if (i < 4) host_words[i] = atomicExch(&status[i], 0);
+}
+
+// The status words of the current device, for a launch that may count into them.
 int async_status_ptr(int32_t **out) {
   int dev = -1;
   HIP_TRY(hipGetDevice(&dev));
@@ -231,35 +244,56 @@ int async_status_ptr(int32_t **out) {
     void *ptr = nullptr;
     HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(async_status)));
     if (ptr == nullptr) return fail(CUMM_HIP_ERUNTIME, "hipGetSymbolAddress returned no address for the status words");
+    void *host = nullptr;
+    HIP_TRY(hipHostMalloc(&host, 4 * sizeof(int32_t), hipHostMallocDefault));
+    hipStream_t st = nullptr;
+    HIP_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));   // (default priority)
+    g_status_host[dev] = reinterpret_cast<int32_t *>(host);
+    g_status_stream[dev] = st;
     g_status_ptr[dev] = reinterpret_cast<int32_t *>(ptr);
   }
+  g_status_armed[dev].store(true);
   *out = g_status_ptr[dev];
   return CUMM_HIP_OK;
 }
 
-// After a synchronisation: anything to report on this device?  (Nothing was ever launched that
-// could report: no device access at all.)
+// After a synchronisation: anything to report on this device?
 int take_async_errors(int32_t *timeouts, int32_t *sort_give_ups = nullptr) {
   *timeouts = 0;
   if (sort_give_ups) *sort_give_ups = 0;
   int dev = -1;
   HIP_TRY(hipGetDevice(&dev));
   if (dev < 0 || dev >= kMaxDevices) return CUMM_HIP_OK;
-  int32_t *ptr;
-  {
-    std::lock_guard<std::mutex> guard(g_scratch_lock);
-    ptr = g_status_ptr[dev];
-  }
-  if (ptr == nullptr) return CUMM_HIP_OK;
-  int32_t words[4] = {0, 0, 0, 0};
-  HIP_TRY(hipMemcpy(words, ptr, sizeof(words), hipMemcpyDeviceToHost));
-  if (words[0] != 0 || words[1] != 0) {
-    const int32_t zero[4] = {0, 0, 0, 0};
-    HIP_TRY(hipMemcpy(ptr, zero, sizeof(zero), hipMemcpyHostToDevice));
-  }
-  *timeouts = words[0];
-  if (sort_give_ups) *sort_give_ups = words[1];
+  // (disarmed before the look: a launch that arms again after this point is seen by the next look)
+  if (!g_status_armed[dev].exchange(false)) return CUMM_HIP_OK;
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  hipLaunchKernelGGL(take_status_kernel, dim3(1), dim3(64), 0, g_status_stream[dev], g_status_ptr[dev], g_status_host[dev]);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipStreamSynchronize(g_status_stream[dev]));
+  *timeouts = g_status_host[dev][0];
+  if (sort_give_ups) *sort_give_ups = g_status_host[dev][1];
   return CUMM_HIP_OK;
+}
+
+// ---- the table of light-prefix hints (launch.h): one per GPU, like `scratch`
+static __device__ int32_t light_hints[kLightHintSlots][8];
+int32_t *g_hints_ptr[kMaxDevices] = {};
+
+// the slot of a sorted mask array in the current device's table; NULL (and no error) if the
+// table cannot be found: hints are optional
+int32_t *light_hint_slot_ptr(const void *sorted_mask) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (g_hints_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(light_hints)) != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_hints_ptr[dev] = reinterpret_cast<int32_t *>(ptr);
+  }
+  return g_hints_ptr[dev] + 8 * light_hint_slot(sorted_mask);
 }
 
 int report_async_errors() {
@@ -635,6 +669,9 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     p.read_source = a->beta != 0.0f;
     // (the hint only moves work between tile shapes; whatever it says the kernel covers every position once)
     p.pair_tiles = a->light_prefix > 0 && !a->ungated_rows ? a->light_prefix / 128 : 0;
+    // without a count from the caller: what input preparation left in the table for this mask array
+    if (a->light_prefix == 0 && !a->ungated_rows && d.tile_shape[0] == 64 && d.tile_shape[1] == 64)
+      p.hint_slot = light_hint_slot_ptr(a->mask_ptr);
     p.ungated_rows = a->ungated_rows != 0;
     p.gather_by_pos = a->indices_by_position != 0;
     p.n_mask_out = p.mask_out ? (a->N + d.tile_shape[0] - 1) / d.tile_shape[0] : 0;
@@ -726,6 +763,9 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     f.slots_bytes = (uint32_t)((wgs + lay.keys - 1) * (int64_t)lay.block_bytes);
     hipError_t e = dt == CUMM_HIP_F16 ? launch_wgrad_ordered_f16(w, pre, f, lay.wide, (int)wgs, stream)
                                       : launch_wgrad_ordered_bf16(w, pre, f, lay.wide, (int)wgs, stream);
+    if (e == hipErrorNotSupported)
+      return fail(CUMM_HIP_ERUNTIME, "the fixed-order backward-weight kernel of this build uses scratch memory, which its "
+                  "hand-counted waits do not allow; use a split_k_serial descriptor");
     if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
     return CUMM_HIP_OK;
     }
@@ -786,6 +826,14 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
       HIP_TRY(zero_device(workspace, need, stream));
     }
     hipError_t e = dt == CUMM_HIP_F16 ? launch_wgrad_atomic_f16(w, pre, f, stream) : launch_wgrad_atomic_bf16(w, pre, f, stream);
+    if (e == hipErrorNotSupported && w.live_list != nullptr) {
+      // the unit-walking kernel failed its load-time check (see counted_waits_hold): the scanning
+      // kernel on one image, zeroed here
+      w.live_cnt = nullptr; w.live_list = nullptr;
+      w.images = f.images = 1;
+      HIP_TRY(zero_device(workspace, need, stream));
+      e = dt == CUMM_HIP_F16 ? launch_wgrad_atomic_f16(w, pre, f, stream) : launch_wgrad_atomic_bf16(w, pre, f, stream);
+    }
     if (e != hipSuccess) return hip_fail(e, "sparse conv wgrad launch");
     return CUMM_HIP_OK;
   }
@@ -1015,15 +1063,32 @@ int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uin
   int32_t *status = nullptr;
   if (int rc = async_status_ptr(&status)) return rc;
   hipError_t e = launch_sort_by_mask(mask, n, mask_filter, sorted_mask, argsort, workspace, status + 1,
-                                     reinterpret_cast<hipStream_t>(stream));
+                                     light_hint_slot_ptr(sorted_mask), reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "mask sort launch");
   return CUMM_HIP_OK;
 }
 
 int cumm_hip_light_prefix(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream) {
-  if (n < 0 || !prefix || (n > 0 && !sorted_mask)) return fail(CUMM_HIP_EINVAL, "bad arguments");
-  hipError_t e = launch_light_prefix(sorted_mask, n, mask_filter, prefix, reinterpret_cast<hipStream_t>(stream));
+  if (n < 0 || (n > 0 && !sorted_mask)) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  hipError_t e = launch_light_prefix(sorted_mask, n, mask_filter, prefix, n > 0 ? light_hint_slot_ptr(sorted_mask) : nullptr,
+                                     reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "light prefix launch");
+  return CUMM_HIP_OK;
+}
+
+int cumm_hip_query_light_hint(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream) {
+  if (!prefix) return fail(CUMM_HIP_EINVAL, "null out-param");
+  *prefix = -1;
+  if (!sorted_mask || n <= 0) return CUMM_HIP_OK;
+  const int32_t *slot = light_hint_slot_ptr(sorted_mask);
+  if (!slot) return CUMM_HIP_OK;
+  int32_t words[8] = {};
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  HIP_TRY(hipMemcpyAsync(words, slot, sizeof(words), hipMemcpyDeviceToHost, s));
+  HIP_TRY(hipStreamSynchronize(s));
+  const uint64_t key = (uint64_t)(uint32_t)words[0] | ((uint64_t)(uint32_t)words[1] << 32);
+  if (key == (uint64_t)reinterpret_cast<uintptr_t>(sorted_mask) && words[2] == n && (uint32_t)words[3] == mask_filter)
+    *prefix = words[4];
   return CUMM_HIP_OK;
 }
 

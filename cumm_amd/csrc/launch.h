@@ -7,6 +7,26 @@
 
 namespace cummhip {
 
+// The kernels that count their vector-memory loads by hand (direct-to-LDS loads and register
+// loads issued from asm statements, waited for with s_waitcnt vmcnt(n)) are correct only while
+// the compiler adds no vector-memory access of its own between a load and its wait: a register
+// spilled to scratch memory is one (scratch accesses count in vmcnt like any other).  Checked
+// once per kernel, when it is first launched, on the code object that was actually loaded: a
+// kernel with private (scratch) memory is not launched; the caller falls back to a kernel without
+// counted waits or reports the launch as failed.
+template <auto Kernel>
+inline bool counted_waits_hold() {
+  static const bool ok = [] {
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(Kernel)) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    return attr.localSizeBytes == 0;
+  }();
+  return ok;
+}
+
 // returns hipSuccess, or hipErrorInvalidValue when no instantiation matches
 hipError_t launch_rowgemm_f16(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s);
 hipError_t launch_rowgemm_bf16(int tm, int tn, int ks, bool wt, const RowGemmParams &p, hipStream_t s);
@@ -93,11 +113,24 @@ hipError_t launch_conv_pairs_sort(const ConvPairsParams &p, unsigned long long m
 hipError_t launch_conv_pairs_fill(const ConvPairsParams &p, hipStream_t s);
 size_t conv_pairs_scan_temp_bytes(size_t n_words);
 hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t temp_bytes, hipStream_t s);
+// What input preparation knows about a sorted mask array and a later forward / backward-input
+// launch on the same array can use without being told: a table of kLightHintSlots slots of eight
+// words in device memory, one table per GPU, indexed by a hash of the array's address.  Slot =
+// {address (two words), length, filter, light prefix in positions, 0, 0, 0}.  A hint only: a
+// launch that finds another array's slot, or a stale one, or none, still computes the same bits.
+constexpr int kLightHintSlots = 256;
+inline int light_hint_slot(const void *sorted_mask) {
+  const uint64_t a = reinterpret_cast<uintptr_t>(sorted_mask) >> 8;
+  return (int)(((a * 0x9E3779B97F4A7C15ull) >> 40) & (uint64_t)(kLightHintSlots - 1));
+}
 // stable radix sort of mask & filter with its permutation (sort_inst.hip)
 size_t sort_by_mask_workspace_bytes(int n);
-hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, hipStream_t s);
+// light prefix of a sorted array into *result (may be NULL) and into hint_slot (may be NULL)
+hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, int32_t *hint_slot,
+                               hipStream_t s);
+// hint_slot: the slot of `sorted` in the current device's table (NULL = leave no hint)
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
-                               void *workspace, int32_t *give_ups, hipStream_t s);
+                               void *workspace, int32_t *give_ups, int32_t *hint_slot, hipStream_t s);
 
 // per-offset lists of (input row, output row) out of a pair table [kv, n] (pairs_inst.hip)
 struct PairListsParams {

@@ -62,6 +62,11 @@ struct RowGemmParams {
   // LDS-streaming kernel, one column block: the first pair_tiles runs of 128 sorted positions are
   // taken as 128-row tiles (rowgemm_lds_mixed_kernel); 0 = 64-row tiles throughout
   int32_t pair_tiles;
+  // ... or, when pair_tiles is 0 and this is not NULL, what the hint slot says: eight words
+  // {mask pointer (two words), n_pos, mask_filter, light prefix in positions, ...} that input
+  // preparation left for this mask array (light_hint_slot in launch.h); a slot that names another
+  // array, length or filter says nothing
+  const int32_t *hint_slot;
   // words the caller's mask_out array holds (a tile number beyond it is not written)
   int32_t n_mask_out;
   // non-zero: a row takes part in every kernel offset of its tile's mask (the reference's rule:

@@ -68,10 +68,12 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
       int shift = 0;
       while ((1 << shift) < nch) ++shift;
       if (shift <= 3 && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
-        RowGemmParams q = p;
-        q.chunk_shift = shift;
-        hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 2, NS2, WT, kWide>), grid, dim3(256), 0, s, q);
-        return hipGetLastError();
+        if (counted_waits_hold<rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 2, NS2, WT, kWide>>()) {
+          RowGemmParams q = p;
+          q.chunk_shift = shift;
+          hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 2, NS2, WT, kWide>), grid, dim3(256), 0, s, q);
+          return hipGetLastError();
+        }
       }
     }
   }
@@ -80,13 +82,16 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
     // the LDS-streaming kernel: 2 x 2 waves, each TM/2 rows by TN/2 channels
     if (p.c_in <= chunk_e && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
       if constexpr (TM == 64 && TN == 64 && Elem<T>::kBytes == 2 && KS <= 2 && !kWide) {
-        if (p.pair_tiles > 0 && grid.y == 1 && p.chunk_shift == 0 && p.mask != nullptr) {
+        if ((p.pair_tiles > 0 || p.hint_slot != nullptr) && grid.y == 1 && p.chunk_shift == 0 && p.mask != nullptr &&
+            counted_waits_hold<rowgemm_lds_mixed_kernel<T, KS, WT>>()) {
           hipLaunchKernelGGL((rowgemm_lds_mixed_kernel<T, KS, WT>), grid, dim3(256), 0, s, p);
           return hipGetLastError();
         }
       }
-      hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS, WT, kWide>), grid, dim3(256), 0, s, p);
-      return hipGetLastError();
+      if (counted_waits_hold<rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS, WT, kWide>>()) {
+        hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KS, NS, WT, kWide>), grid, dim3(256), 0, s, p);
+        return hipGetLastError();
+      }
     }
   }
   if (p.c_in <= chunk_e) {
@@ -127,6 +132,7 @@ static hipError_t launch_ks(int ks, bool wt, const RowGemmParams &p, hipStream_t
 template <class T, int KS, bool WT>
 static hipError_t launch_wave(const RowGemmParams &p, hipStream_t s) {
   if constexpr (Elem<T>::kBytes == 2) {
+    if (!counted_waits_hold<rowgemm_wave_kernel<T, KS, WT, kWide>>()) return hipErrorNotSupported;   // (the caller goes on)
     const int n_blocks = (p.n_pos + 15) / 16;
     if (n_blocks == 0 || p.k_out <= 0) return hipSuccess;
     static int resident_of[16] = {};
@@ -156,11 +162,13 @@ hipError_t CUMM_LAUNCH_NAME(int tm, int tn, int ks, bool wt, const RowGemmParams
     // (up to 64 output channels: a second column block would gather the rows a second time)
     if (p.mask == nullptr && p.kv == 1 && p.gather_by_pos && p.c_in <= 32 * ks && p.k_out <= 64 &&
         (wt ? p.w_stride_n == 1 : p.w_stride_c == 1) && (tm == 64 || tm == 128) && (tn == 64 || tn == 128)) {
+      hipError_t e = hipErrorNotSupported;
       switch (ks) {
-      case 1: return wt ? launch_wave<T, 1, true>(p, s) : launch_wave<T, 1, false>(p, s);
-      case 2: return wt ? launch_wave<T, 2, true>(p, s) : launch_wave<T, 2, false>(p, s);
-      case 4: return wt ? launch_wave<T, 4, true>(p, s) : launch_wave<T, 4, false>(p, s);
+      case 1: e = wt ? launch_wave<T, 1, true>(p, s) : launch_wave<T, 1, false>(p, s); break;
+      case 2: e = wt ? launch_wave<T, 2, true>(p, s) : launch_wave<T, 2, false>(p, s); break;
+      case 4: e = wt ? launch_wave<T, 4, true>(p, s) : launch_wave<T, 4, false>(p, s); break;
       }
+      if (e != hipErrorNotSupported) return e;
     }
   }
   if (tm == 64 && tn == 64) return launch_ks<T, 4, 1, 64>(ks, wt, p, s);

@@ -649,7 +649,15 @@ __global__ __launch_bounds__(256) void rowgemm_lds_mixed_kernel(const RowGemmPar
   __shared__ int ix1[4][64];
   __shared__ int ix2[4][64];
   const int tiles = (int)gridDim.x;
-  const int pairs = p.pair_tiles < (tiles >> 1) ? p.pair_tiles : (tiles >> 1);
+  int hinted = p.pair_tiles;
+  if (hinted == 0 && p.hint_slot != nullptr) {
+    // (uniform addresses: scalar loads, issued with the kernel arguments' own)
+    const uint64_t key = (uint64_t)(uint32_t)p.hint_slot[0] | ((uint64_t)(uint32_t)p.hint_slot[1] << 32);
+    const bool named = key == (uint64_t)p.mask && p.hint_slot[2] == p.n_pos && (uint32_t)p.hint_slot[3] == p.mask_filter;
+    const int prefix = p.hint_slot[4];
+    hinted = named && prefix > 0 ? prefix >> 7 : 0;
+  }
+  const int pairs = hinted < (tiles >> 1) ? hinted : (tiles >> 1);
   const int singles = tiles - 2 * pairs;
   const int rank = (int)blockIdx.x;
   if (rank < singles) {

@@ -7,15 +7,24 @@
 //   * sort_setup_kernel reads the keys once and makes the histograms of ALL passes (the digits of
 //     a key do not depend on the order the keys are in), clears the look-back state and the block
 //     tickets;
+//   * a pass whose digit is the same in every key (the histogram shows it: the bits of a 32-bit
+//     filter above the kernel volume, any pass of an input with one mask value) moves nothing: its
+//     workgroups leave at once, and the passes that do move keys work out among themselves which
+//     of the two buffers each reads and writes so that the last of them writes the caller's;
 //   * a pass kernel is a single sweep: a workgroup takes the next chunk of 4096 keys (by ticket,
 //     so that a chunk's predecessors have always started), ranks its keys per digit - per wave
 //     by ballot matching, in position order, which is what makes the pass stable -, publishes its
 //     per-digit counts, finds the counts of all chunks before it by looking back over what they
 //     have published (a chunk publishes its own counts at once and the running total when it
 //     knows it; a look-back stops at the first running total), and scatters.
+//   * sort_finish_kernel, behind the last pass, counts the light prefix of the sorted array into
+//     the hint slot that a later convolution launch on this array looks up (launch.h).
 // Every spin on another workgroup's state is bounded: a wave that gives up counts itself and goes
-// on (the result is then wrong, and the host says so at its next synchronisation), so the grid
-// always drains.
+// on, so the grid always drains.  The finish kernel then replaces the result by the identity
+// order (argsort = 0 .. n-1, the masks as they came): any permutation with its masks is a valid
+// input of the convolution kernels - the order only decides how light the tiles are - so what
+// follows on the stream computes the right thing, slowly, and the host reports the give-up at
+// its next synchronisation.
 // Integer work, bound by launch latency at 10^5 keys and by HBM / L2 traffic at 10^6 and more.
 #include "launch.h"
 #include "lds_dma.h"
@@ -41,16 +50,10 @@ struct SortParams {
   uint32_t *state;           // [passes][chunks][kBins] look-back words
   uint32_t *tickets;         // [passes] next chunk to hand out
   int32_t *give_ups;         // counts the look-backs that ran into their bound (the host reports them)
-  // pass p reads keys/vals from src and writes dst (pass 0 reads the masks and an implicit iota)
-  const uint32_t *src_keys;
-  const int32_t *src_vals;
-  uint32_t *dst_keys;
-  int32_t *dst_vals;
   int32_t pass;
-  // chunks are handed out by ticket (a chunk's predecessors have then always started); with no more
-  // chunks than the device runs workgroups at once every chunk is resident anyway and a chunk is
-  // its workgroup's number: one atomic round trip less per pass
-  int32_t use_tickets;
+  uint32_t *out_keys, *tmp_keys;   // the caller's arrays and the workspace's: the passes alternate between them
+  int32_t *out_vals, *tmp_vals;
+  int32_t *hint_slot;        // light-prefix hint of the sorted array (launch.h), or NULL
 };
 
 __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortParams p) {
@@ -61,6 +64,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortPara
   const size_t words = (size_t)p.passes * p.chunks * kBins;
   for (size_t i = (size_t)blockIdx.x * kSortThreads + t; i < words; i += (size_t)gridDim.x * kSortThreads) p.state[i] = 0u;
   if (blockIdx.x == 0 && t < p.passes) p.tickets[t] = 0u;
+  if (blockIdx.x == 0 && t < 8 && p.hint_slot != nullptr) p.hint_slot[t] = t == 4 ? (p.n / 128) * 128 : 0;   // names no array yet
   __syncthreads();
   // lanes of a wave with the same digit add once (most masks of a sparse cloud are the same word:
   // one add per lane would queue 64 deep on one LDS address)
@@ -123,12 +127,40 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int shift = p.pass * kRadixBits;
 
-  if (t == 0) chunk_of_block = p.use_tickets ? (int)atomicAdd(&p.tickets[p.pass], 1u) : (int)blockIdx.x;
+  // which passes move keys at all (thread = bin: a bin that holds every key makes its pass idle)
+  uint32_t tot[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) tot[q] = q < p.passes ? p.hist[q * kBins + t] : (t == 0 ? (uint32_t)p.n : 0u);
+  int movers = 0, movers_before = 0;
+  bool mine_moves = false;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const bool idle = __syncthreads_or(tot[q] == (uint32_t)p.n) != 0;
+    if (!idle) {
+      ++movers;
+      if (q < p.pass) ++movers_before;
+      if (q == p.pass) mine_moves = true;
+    }
+  }
+  // nothing moves at all (one mask value): the first pass copies the input through
+  const bool copy_through = movers == 0 && p.pass == 0;
+  if (!mine_moves && !copy_through) return;
+  // the last mover writes the caller's arrays, the ones before it alternate; the first one
+  // reads the caller's masks (and the identity order)
+  const bool first = movers_before == 0;
+  const bool to_out = copy_through || ((movers - 1 - movers_before) & 1) == 0;
+  uint32_t *const dst_keys = to_out ? p.out_keys : p.tmp_keys;
+  int32_t *const dst_vals = to_out ? p.out_vals : p.tmp_vals;
+  const uint32_t *const src_keys = to_out ? p.tmp_keys : p.out_keys;
+  const int32_t *const src_vals = to_out ? p.tmp_vals : p.out_vals;
+  // chunks are handed out by ticket: a chunk's predecessors have then always started, whatever
+  // order the workgroups are dispatched in and however many of them are resident
+  if (t == 0) chunk_of_block = (int)atomicAdd(&p.tickets[p.pass], 1u);
 #pragma unroll
   for (int w = 0; w < kSortWaves; ++w) wave_hist[w][t] = 0u;
   // exclusive prefix over the digit values of the whole input: thread = bin; a scan inside each
   // wave by lane shuffles, then the totals of the waves before
-  const uint32_t total_of_bin = p.hist[p.pass * kBins + t];
+  const uint32_t total_of_bin = p.pass == 0 ? tot[0] : (p.pass == 1 ? tot[1] : (p.pass == 2 ? tot[2] : tot[3]));
   uint32_t incl = total_of_bin;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -144,16 +176,13 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   const int chunk = chunk_of_block;
   if (chunk >= p.chunks) return;   // (never: the grid has one workgroup per chunk)
 
-  // A digit that is the same in every key (the bits of a 32-bit filter above the kernel volume;
-  // any pass of an input with one mask value) leaves the order as it is: the chunk is copied
-  // through, without ranks and without waiting for anybody.
-  if (__syncthreads_or(total_of_bin == (uint32_t)p.n)) {
+  if (copy_through) {
 #pragma unroll
     for (int u = 0; u < kItems; ++u) {
       const int64_t pos = (int64_t)chunk * kChunk + u * kSortThreads + t;
       if (pos < p.n) {
-        p.dst_keys[pos] = p.pass == 0 ? (p.mask[pos] & p.filter) : p.src_keys[pos];
-        p.dst_vals[pos] = p.pass == 0 ? (int32_t)pos : p.src_vals[pos];
+        dst_keys[pos] = p.mask[pos] & p.filter;
+        dst_vals[pos] = (int32_t)pos;
       }
     }
     return;
@@ -169,12 +198,12 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   for (int u = 0; u < kItems; ++u) {
     const int64_t pos = base_w + u * 64 + lane;
     const bool valid = pos < p.n;
-    if (p.pass == 0) {
+    if (first) {
       key[u] = valid ? (p.mask[pos] & p.filter) : 0u;
       val[u] = (int32_t)pos;
     } else {
-      key[u] = valid ? p.src_keys[pos] : 0u;
-      val[u] = valid ? p.src_vals[pos] : 0;
+      key[u] = valid ? src_keys[pos] : 0u;
+      val[u] = valid ? src_vals[pos] : 0;
     }
   }
 #pragma unroll
@@ -262,8 +291,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
     if (pos < p.n) {
       const uint32_t d = (key[u] >> shift) & (kBins - 1);
       const uint32_t dst = bin_base[d] + wave_hist[wave][d] + rank[u];
-      p.dst_keys[dst] = key[u];
-      p.dst_vals[dst] = val[u];
+      dst_keys[dst] = key[u];
+      dst_vals[dst] = val[u];
     }
   }
 }
@@ -274,17 +303,61 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
 // (which starts at the positions of all whole runs) to where it begins.
 constexpr int kLightOffsets = 2;
 
-__global__ __launch_bounds__(64) void light_prefix_init_kernel(int32_t *result, int runs) {
-  if (threadIdx.x == 0) *result = runs * 128;
+__global__ __launch_bounds__(64) void light_prefix_init_kernel(int32_t *result, int32_t *hint_slot, int runs) {
+  if (threadIdx.x == 0 && result != nullptr) *result = runs * 128;
+  if (threadIdx.x < 8 && hint_slot != nullptr) hint_slot[threadIdx.x] = threadIdx.x == 4 ? runs * 128 : 0;
 }
 
-__global__ __launch_bounds__(256) void light_prefix_kernel(const uint32_t *sorted, int runs, uint32_t filter, int32_t *result) {
+// Names the array a hint slot describes (the prefix word has been counted down by then or is
+// being counted down by the same kernel: a launch that reads the slot comes later on the stream).
+__device__ __forceinline__ void name_hint_slot(int32_t *slot, const uint32_t *sorted, int n, uint32_t filter) {
+  const uint64_t a = (uint64_t)sorted;
+  slot[0] = (int32_t)(uint32_t)a;
+  slot[1] = (int32_t)(uint32_t)(a >> 32);
+  slot[2] = n;
+  slot[3] = (int32_t)filter;
+}
+
+__global__ __launch_bounds__(256) void light_prefix_kernel(const uint32_t *sorted, int n, int runs, uint32_t filter,
+                                                           int32_t *result, int32_t *hint_slot) {
   const int lane = threadIdx.x & 63;
   const int run = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (blockIdx.x == 0 && threadIdx.x == 0 && hint_slot != nullptr) name_hint_slot(hint_slot, sorted, n, filter);
   if (run >= runs) return;
   const uint32_t lo = wave_or_dpp(sorted[(size_t)run * 128 + lane] & filter);
   const uint32_t hi = wave_or_dpp(sorted[(size_t)run * 128 + 64 + lane] & filter);
-  if (lane == 0 && (__builtin_popcount(lo) > kLightOffsets || __builtin_popcount(hi) > kLightOffsets)) atomicMin(result, run * 128);
+  if (lane == 0 && (__builtin_popcount(lo) > kLightOffsets || __builtin_popcount(hi) > kLightOffsets)) {
+    if (result != nullptr) atomicMin(result, run * 128);
+    if (hint_slot != nullptr) atomicMin(&hint_slot[4], run * 128);
+  }
+}
+
+// Behind the last pass of the sort: the light prefix of the result into the hint slot - or, when a
+// look-back of this device has given up since the host last looked, the identity order in place
+// of a result that cannot be trusted.  One wave per 128 positions, the last run may be short.
+__global__ __launch_bounds__(256) void sort_finish_kernel(const SortParams p) {
+  const int lane = threadIdx.x & 63;
+  const int run = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const bool broken = p.give_ups != nullptr && __hip_atomic_load(p.give_ups, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+  if (broken) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int64_t pos = (int64_t)run * 128 + h * 64 + lane;
+      if (pos < p.n) {
+        p.out_keys[pos] = p.mask[pos] & p.filter;
+        p.out_vals[pos] = (int32_t)pos;
+      }
+    }
+    if (p.hint_slot != nullptr && blockIdx.x == 0 && threadIdx.x < 8) p.hint_slot[threadIdx.x] = 0;
+    return;
+  }
+  if (p.hint_slot == nullptr) return;
+  if (blockIdx.x == 0 && threadIdx.x == 0) name_hint_slot(p.hint_slot, p.out_keys, p.n, p.filter);
+  if (run >= p.n / 128) return;
+  const uint32_t lo = wave_or_dpp(p.out_keys[(size_t)run * 128 + lane]);
+  const uint32_t hi = wave_or_dpp(p.out_keys[(size_t)run * 128 + 64 + lane]);
+  if (lane == 0 && (__builtin_popcount(lo) > kLightOffsets || __builtin_popcount(hi) > kLightOffsets))
+    atomicMin(&p.hint_slot[4], run * 128);
 }
 
 size_t align256s(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -305,7 +378,7 @@ size_t sort_by_mask_workspace_bytes(int n) {
 }
 
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
-                               void *workspace, int32_t *give_ups, hipStream_t s) {
+                               void *workspace, int32_t *give_ups, int32_t *hint_slot, hipStream_t s) {
   if (n <= 0) return hipSuccess;
   char *base = reinterpret_cast<char *>(workspace);
   const size_t words = align256s(4 * (size_t)n);
@@ -313,46 +386,33 @@ hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uin
   p.mask = mask; p.filter = filter; p.n = n;
   p.chunks = (n + kChunk - 1) / kChunk;
   p.passes = sort_passes(filter);
-  uint32_t *tmp_keys = reinterpret_cast<uint32_t *>(base);
-  int32_t *tmp_vals = reinterpret_cast<int32_t *>(base + words);
+  p.out_keys = sorted; p.out_vals = argsort;
+  p.tmp_keys = reinterpret_cast<uint32_t *>(base);
+  p.tmp_vals = reinterpret_cast<int32_t *>(base + words);
   p.hist = reinterpret_cast<uint32_t *>(base + 2 * words);
   p.tickets = reinterpret_cast<uint32_t *>(base + 2 * words + align256s(4 * 4 * kBins));
   p.state = reinterpret_cast<uint32_t *>(base + 2 * words + align256s(4 * 4 * kBins) + 256);
   p.give_ups = give_ups;
-  p.src_keys = nullptr; p.src_vals = nullptr; p.dst_keys = nullptr; p.dst_vals = nullptr; p.pass = 0;
-  {
-    static int cus_of[16] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    int &cus = cus_of[dev & 15];
-    if (cus == 0) {
-      e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-      if (e != hipSuccess) return e;
-    }
-    p.use_tickets = p.chunks > cus ? 1 : 0;   // (a pass workgroup fits a CU: one resident per CU at least)
-  }
+  p.hint_slot = hint_slot;
+  p.pass = 0;
   hipLaunchKernelGGL(sort_clear_hist_kernel, dim3((4 * kBins + 255) / 256), dim3(256), 0, s, p.hist, 4 * kBins);
   int setup_blocks = p.chunks < 512 ? p.chunks : 512;
   hipLaunchKernelGGL(sort_setup_kernel, dim3(setup_blocks), dim3(kSortThreads), 0, s, p);
-  // the last pass writes the caller's arrays; the passes before it alternate
   for (int q = 0; q < p.passes; ++q) {
-    const bool to_out = ((p.passes - 1 - q) & 1) == 0;
     SortParams r = p;
     r.pass = q;
-    r.dst_keys = to_out ? sorted : tmp_keys;
-    r.dst_vals = to_out ? argsort : tmp_vals;
-    r.src_keys = to_out ? tmp_keys : sorted;
-    r.src_vals = to_out ? tmp_vals : argsort;
     hipLaunchKernelGGL(sort_pass_kernel, dim3(p.chunks), dim3(kSortThreads), 0, s, r);
   }
+  hipLaunchKernelGGL(sort_finish_kernel, dim3((n + 511) / 512), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 
-hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, hipStream_t s) {
+hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, int32_t *hint_slot,
+                               hipStream_t s) {
   const int runs = n / 128;
-  hipLaunchKernelGGL(light_prefix_init_kernel, dim3(1), dim3(64), 0, s, result, runs);
-  if (runs > 0) hipLaunchKernelGGL(light_prefix_kernel, dim3((runs + 3) / 4), dim3(256), 0, s, sorted, runs, filter, result);
+  hipLaunchKernelGGL(light_prefix_init_kernel, dim3(1), dim3(64), 0, s, result, hint_slot, runs);
+  hipLaunchKernelGGL(light_prefix_kernel, dim3(runs > 0 ? (runs + 3) / 4 : 1), dim3(256), 0, s, sorted, n, runs, filter, result,
+                     hint_slot);
   return hipGetLastError();
 }
 

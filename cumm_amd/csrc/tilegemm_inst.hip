@@ -39,6 +39,7 @@ static hipError_t launch_xy(bool xk, bool yk, const TileGemmParams &p, dim3 grid
 template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS>
 static hipError_t launch_dense_ring_as(const TileGemmParams &p, hipStream_t s) {
   constexpr int TM = WM * RBW * 16, TN = WN * NBW * 16;
+  if (!counted_waits_hold<densegemm_lds_kernel<T, WM, WN, RBW, NBW, KS, NS>>()) return hipErrorNotSupported;
   const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
   hipLaunchKernelGGL((densegemm_lds_kernel<T, WM, WN, RBW, NBW, KS, NS>), dim3((unsigned)(tiles_m * tiles_n)),
                      dim3(WM * WN * 64), 0, s, p, tiles_m, tiles_n);
@@ -62,7 +63,7 @@ static bool launch_dense_ring(const TileGemmParams &p, hipStream_t s, hipError_t
     if (big_tiles >= 256) *err = launch_dense_ring_as<T, 2, 4, 8, 4, 1, 3>(p, s);       // a tile per CU at least
     else if (mid_tiles >= 64) *err = launch_dense_ring_as<T, 2, 2, 4, 4, 2, 2>(p, s);
     else return false;
-    return true;
+    return *err != hipErrorNotSupported;     // (the register-staged kernel takes over)
   }
 }
 
@@ -90,6 +91,8 @@ hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const
   const int kblocks = (p.K + cpu_ - 1) / cpu_, cblocks = (p.C + cpu_ - 1) / cpu_;
   if (groups == 0 || p.kv == 0) return hipSuccess;
   hipError_t e;
+  const bool units_ok = wide ? counted_waits_hold<wgrad_units_kernel<T, 2, 2, 1>>() : counted_waits_hold<wgrad_units_kernel<T, 1, 1, 2>>();
+  if (p.live_list != nullptr && !units_ok) return hipErrorNotSupported;
   if (p.live_list != nullptr) {
     // lists + zeroed image, then a resident grid that walks the units
     static int resident_of[2][16] = {};
@@ -153,6 +156,8 @@ hipError_t CUMM_CAT(launch_wgrad_ordered_, CUMM_NAME)(const WgradParams &p, cons
                                                       const WgradOrderedParams &f, bool wide, int wgs, hipStream_t s) {
   using T = CUMM_ELEM;
   if (p.num_red == 0 || p.kv == 0 || wgs < 1) return hipSuccess;
+  if (!(wide ? counted_waits_hold<wgrad_units_kernel<T, 2, 2, 1, true>>() : counted_waits_hold<wgrad_units_kernel<T, 1, 1, 2, true>>()))
+    return hipErrorNotSupported;
   hipLaunchKernelGGL(wgrad_prepare_kernel, dim3(p.kv), dim3(256), 0, s, pre);   // lists only: no image to zero
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;

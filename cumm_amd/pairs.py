@@ -338,6 +338,18 @@ def light_prefix_device(sorted_mask, mask_filter: int = 0xFFFFFFFF, stream: int 
     return int(res.cpu().numpy()[0])
 
 
+def light_hint_device(sorted_mask, mask_filter: int = 0xFFFFFFFF, stream: int = 0) -> int:
+    """The light prefix that the library's device-side table holds for this sorted mask tensor
+    (left there by :func:`sort_by_mask_device` or :func:`light_prefix_device`), -1 if none: what a
+    forward / backward-input launch with ``light_prefix == 0`` on this tensor will use."""
+    import ctypes
+    from . import _capi
+    out = ctypes.c_int32(-1)
+    _capi.check(_capi.lib().cumm_hip_query_light_hint(sorted_mask.byte_pointer(), int(sorted_mask.shape[0]),
+                                                      int(mask_filter) & 0xFFFFFFFF, ctypes.byref(out), stream))
+    return int(out.value)
+
+
 def pairs_by_position_device(indices, mask_argsort, out=None, stream: int = 0):
     """:func:`pairs_by_position` of device tensors ``indices`` [kv, N] int32 and ``mask_argsort``
     [N] int32, in stream order; ``out`` ([kv, N] int32) is filled when given."""

@@ -468,7 +468,9 @@ class ConvParams(_Versioned):
         self.deterministic = False
         # not in the reference's struct either: a hint for forward / backward-input, the number of
         # leading positions of the sorted order in tiles of one or two kernel offsets
-        # (pairs.light_prefix of the sorted mask); 0 = unknown.  Any value gives the same result.
+        # (pairs.light_prefix of the sorted mask).  0 = not given: the launch uses what the GPU sort
+        # (pairs.sort_by_mask_device) or pairs.light_prefix_device left for this mask array in the
+        # library's device-side table, if anything; negative = no hint.  Any value gives the same result.
         self.light_prefix = 0
         # not in the reference's struct: True = every position of a tile takes part in every kernel
         # offset of the tile's OR-ed mask (gated by its pair-table entry alone, the reference's

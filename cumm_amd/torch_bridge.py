@@ -162,10 +162,10 @@ class SparseConvGeometry:
             self.mask_bwd, self.order_bwd = self.mask_fwd, self.order_fwd
         else:
             self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, mask_filter=bits, stream=stream)
-        # how far the light end of each sorted order reaches (the forward / backward-input launches
-        # take it as a hint; one number each comes back to the host here)
-        self.light_fwd = pairs.light_prefix_device(self.mask_fwd, stream=stream)
-        self.light_bwd = self.light_fwd if self.subm else pairs.light_prefix_device(self.mask_bwd, stream=stream)
+        # (how far the light end of each sorted order reaches - the hint of the forward and
+        # backward-input launches - stays on the device: the sort leaves it in the library's table
+        # under the sorted array's address and the launches look it up there; 0 = not given here)
+        self.light_fwd = self.light_bwd = 0
         self._reduced = {}
         self._launches = {}      # validated calls of the layers on this geometry, see _Launch
 

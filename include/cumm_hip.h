@@ -125,12 +125,15 @@ typedef struct CummHipSparseConvArgs {
   const void *bias_pointer;         /* int8 inference: f32 [K] */
   const void *scale_pointer;        /* int8 inference: f32 [K] */
   int32_t rows_in, rows_out;        /* row counts of the input / output feature tensors */
-  int32_t light_prefix;             /* forward / backward-input, optional (0 = unknown): how many leading positions of
-                                       the sorted order sit in tiles of one or two kernel offsets, as
-                                       cumm_hip_light_prefix counts them for mask_ptr.  A hint only: it moves those
-                                       positions to 128-row tiles (fewer, longer-lived workgroups where a tile's
-                                       time is its memory round trips); any value gives the same bits, a wrong one
-                                       costs time.  No counterpart in the reference. */
+  int32_t light_prefix;             /* forward / backward-input, optional: how many leading positions of the sorted order
+                                       sit in tiles of one or two kernel offsets, as cumm_hip_light_prefix counts them
+                                       for mask_ptr.  A hint only: it moves those positions to 128-row tiles (fewer,
+                                       longer-lived workgroups where a tile's time is its memory round trips); any
+                                       value gives the same bits, a wrong one costs time.  0 (what a caller that fills
+                                       the reference's struct passes) = not given: the launch then uses the count that
+                                       cumm_hip_sort_by_mask or cumm_hip_light_prefix left for this mask array in the
+                                       library's own table on the device, if there is one.  Negative = no hint at all.
+                                       No counterpart in the reference. */
   int32_t ungated_rows;             /* forward / backward-input.  0: a position takes part in kernel offset k only if its
                                        own mask word has bit k - masks made from the pair table (bit k set wherever
                                        indice_ptr[k][row] >= 0, as spconv makes them) lose nothing, and entries and rows
@@ -251,11 +254,20 @@ int cumm_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* host out-p
  *   workspace: at least cumm_hip_subm_pairs_workspace(n) bytes, 16-byte aligned.
  * cumm_hip_sort_by_mask: sorted = stable ascending sort of (mask & mask_filter), argsort = the
  *   permutation; workspace at least cumm_hip_sort_by_mask_workspace(n) bytes.
+ *   The sort also counts the light prefix of its result (below) and leaves it in a table inside the
+ *   library, on the device, under the address of sorted_mask: a forward / backward-input launch
+ *   whose mask_ptr is that array finds it there by itself (no host read, no extra field to fill).
+ *   A sort whose bounded waits ran out writes the identity order instead (argsort = 0 .. n-1 with
+ *   the masks as they came: valid input for the convolutions, only slower) and the next
+ *   synchronising call reports it.
  * cumm_hip_light_prefix: for a sorted mask array (what cumm_hip_sort_by_mask writes, what a
  *   convolution takes as mask_ptr): the number of leading positions, a multiple of 128, in runs of
  *   128 whose two halves of 64 each OR to at most two kernel offsets - a submanifold layer's
- *   centre-only positions lead the ascending order.  Written to *prefix (device memory, one int32)
- *   in stream order; the value is CummHipSparseConvArgs.light_prefix.  No counterpart in the reference. */
+ *   centre-only positions lead the ascending order.  Written to *prefix (device memory, one int32;
+ *   may be NULL) in stream order - the value is CummHipSparseConvArgs.light_prefix - and into the
+ *   library's table like the sort's own count: the call for arrays that another sort made.  The
+ *   table is keyed by address, length and filter, holds 256 entries per GPU (a newer array may
+ *   replace an older one) and is never needed for correct results.  No counterpart in the reference. */
 size_t cumm_hip_subm_pairs_workspace(int n);
 int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_shape, const int32_t *ksize,
                         const int32_t *dilation, int32_t *indices_fwd, int32_t *indices_bwd,
@@ -265,6 +277,10 @@ size_t cumm_hip_sort_by_mask_workspace(int n);
 int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
                           int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream);
 int cumm_hip_light_prefix(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream);
+/* What the library's table holds for this array, length and filter: *prefix (host) = the light prefix a
+ * launch on it would find, or -1 if the table has nothing for it.  Waits for the stream.  For tests
+ * and diagnostics; no launch needs it. */
+int cumm_hip_query_light_hint(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream);
 
 /* Pair tables of a regular (strided) sparse convolution, in two calls like spconv's
  * generate_conv_inds_mask_stage1 / stage2 (the reference's callers take them from there; its own

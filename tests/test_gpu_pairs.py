@@ -218,3 +218,54 @@ def test_light_prefix_against_the_host_count(n):
         d = H.dev(mask, "u32")
         for filt in (0xFFFFFFFF, 0x6000, 1 << 13, 0x1FFF):
             assert pairs.light_prefix_device(d, mask_filter=filt) == pairs.light_prefix(mask, filt), (light_len, hex(filt))
+
+
+def test_sort_leaves_the_light_prefix_for_the_launch():
+    """The GPU sort counts the light prefix of its result and leaves it in the library's
+    device-side table under the result's address, where a forward launch with no hint of its own
+    looks: the table holds what the host count says, per filter; an array nobody prepared has no
+    entry; cumm_hip_light_prefix registers an array that another sort made; and the launch gives
+    the same bits whether it is told the count, finds it, or is told to use none."""
+    from cumm_amd.conv.main import ConvMainUnitTest
+    from cumm_amd.tensorview.gemm import ConvOpType, ConvParams
+    print("case light hint table", flush=True)
+    rng = np.random.default_rng(77)
+    grid = (16, 200, 200)
+    coords = synth.clustered_voxels(rng, 9000, grid, 8, sigma=4.0, noise_frac=0.6)
+    pt = pairs.subm_pairs(coords, grid)
+    n = coords.shape[0]
+    d_mask = H.dev(pt.mask_fwd, "u32")
+    for filt in (0xFFFFFFFF, 0x07FFFFFF, 0x3FFF):
+        ms_ref, order_ref = pairs.sort_by_mask(pt.mask_fwd, filt)
+        ms, order = pairs.sort_by_mask_device(d_mask, filt)
+        np.testing.assert_array_equal(H.host(ms), ms_ref)
+        assert pairs.light_hint_device(ms, filt) == pairs.light_prefix(ms_ref, filt)
+        assert pairs.light_hint_device(ms, filt ^ 0x10) == -1          # another filter: no entry
+    ms_ref, order_ref = pairs.sort_by_mask(pt.mask_fwd)
+    exact = pairs.light_prefix(ms_ref)
+    assert 256 <= exact <= n - 256
+    foreign = H.dev(ms_ref, "u32")                  # sorted elsewhere: nothing known about it
+    # (the slot of this address may hold an older array's entry, never this one's)
+    assert pairs.light_hint_device(foreign) in (-1, exact)
+    assert pairs.light_prefix_device(foreign) == exact
+    assert pairs.light_hint_device(foreign) == exact
+    ms, order = pairs.sort_by_mask_device(d_mask)
+    feat = H.to_storage(rng.normal(0, 1, size=(n, 64)).astype(np.float32), "f16")
+    w = H.to_storage(rng.normal(0, 0.05, size=(64, 27, 64)).astype(np.float32), "f16")
+    outs = []
+    for hint in (-1, 0, exact):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp("f16", ConvOpType.Forward, 64, 64)
+        p.input, p.weight, p.output = H.dev(feat, "f16"), H.dev(w, "f16"), tv.zeros([n, 64], tv.float16, 0)
+        p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_fwd, "i32"), ms, order
+        p.mask_output = tv.zeros([(n + 63) // 64], tv.uint32, 0)
+        p.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(p)
+        outs.append((H.host(p.output), H.host(p.mask_output)))
+    from oracle import conv_ref
+    ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, np.zeros((n, 64), np.float16), pt.indices_fwd, ms_ref, order_ref,
+                                                 tile_m=64, dtype_in="f16", dtype_w="f16", dtype_out="f16")
+    assert H.rel_err(H.as_f32(outs[0][0], "f16"), H.as_f32(ref, "f16")) < 1e-2
+    for got, mo in outs:
+        np.testing.assert_array_equal(got.view(np.uint16), outs[0][0].view(np.uint16))
+        np.testing.assert_array_equal(mo, ref_mo)
