@@ -70,11 +70,11 @@ GRID = (41, 1600, 1408)
 SEED = 20240607
 
 
-def find_desp(tv_dtype, op, tile_m, tile_n, int8=False, parallel=False):
+def find_desp(tv_dtype, op, tile_m, tile_n, int8=False, parallel=False, dynamic_mask=False):
     for d in ConvMainUnitTest.get_all_conv_algo_desp():
         if (d.dtype_a == tv_dtype and d.dtype_c == tv_dtype and ConvOpType(d.op_type) == op and d.tile_shape[0] == tile_m
                 and d.tile_shape[1] == tile_n and d.is_int8_inference == int8
-                and d.split_k_parallel == parallel):
+                and d.split_k_parallel == parallel and bool(d.dynamic_mask) == dynamic_mask):
             return d
     raise KeyError((tv_dtype, op, tile_m, tile_n, int8, parallel))
 
@@ -424,10 +424,32 @@ def bench_native(args, coords):
     # what this algorithm has to move: per pair one input row, one fp32 accumulator row read and
     # written, two indices; the image zeroed, read once more and the result written
     alg = P * (c * 2 + 2 * c * 4 + 8) + n * c * (4 + 4 + 2) + 125 * c * c * 2
-    return {"voxels": n, "kernel_volume": 125, "active_pairs": P, "input_preparation_first_call_ms": round(prep_ms, 3),
-            "forward_ms": round(wms, 4), "kernel_ms_events": round(ems, 4),
-            "tflops": round(2.0 * P * c * c / (wms * 1e-3) / 1e12, 2),
-            "hbm_frac": round(alg / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "launches": plan.launches}
+    res = {"voxels": n, "kernel_volume": 125, "active_pairs": P, "input_preparation_first_call_ms": round(prep_ms, 3),
+           "per_offset": {"forward_ms": round(wms, 4), "kernel_ms_events": round(ems, 4),
+                          "tflops": round(2.0 * P * c * c / (wms * 1e-3) / 1e12, 2),
+                          "hbm_frac": round(alg / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "launches": plan.launches}}
+    # the same layer in ONE launch: a dynamic_mask descriptor, four mask words per position
+    # (masks from the pair table, positions ordered by cumm_hip_sort_by_mask_words)
+    t0 = time.perf_counter()
+    masks = pairs.masks_from_pairs_device(table.indices_fwd)
+    ms_d, order_d = pairs.sort_by_mask_words_device(masks)
+    by_pos = pairs.pairs_by_position_device(table.indices_fwd, order_d)
+    ConvMainUnitTest_sync()
+    prep2_ms = (time.perf_counter() - t0) * 1e3
+    p = ConvParams(3, ConvOpType.Forward)
+    p.conv_algo_desp = find_desp(tv.float16, ConvOpType.Forward, 64, 64, dynamic_mask=True)
+    p.input, p.weight, p.output = x, w, tv.zeros([n, c], tv.float16, 0)
+    p.mask, p.mask_argsort = ms_d, order_d
+    # algorithmic bytes of the mask-based launch: rows in and out once, table, masks (4 words), order, weights
+    alg_m = n * c * 2 * 2 + 125 * n * 4 + n * 16 + n * 4 + 125 * c * c * 2
+    for name, table_t, flag in (("by_row", table.indices_fwd, False), ("by_position", by_pos, True)):
+        p.indices, p.indices_by_position = table_t, flag
+        wms, ems = timed(lambda: ConvMainUnitTest.implicit_gemm2(p), max(20, args.steps // 2), 5)
+        res["dynamic_mask_" + name] = {"forward_ms": round(wms, 4), "kernel_ms_events": round(ems, 4),
+                                       "tflops": round(2.0 * P * c * c / (wms * 1e-3) / 1e12, 2),
+                                       "hbm_frac": round(alg_m / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "launches": 1}
+    res["dynamic_mask_input_preparation_first_call_ms"] = round(prep2_ms, 3)
+    return res
 
 
 def bench_dense_gemm(args):

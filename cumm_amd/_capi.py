@@ -57,7 +57,7 @@ class SparseConvArgs(C.Structure):
                 ("d_is_bias", C.c_int32), ("deterministic", C.c_int32),
                 ("bias_pointer", C.c_void_p), ("scale_pointer", C.c_void_p),
                 ("rows_in", C.c_int32), ("rows_out", C.c_int32), ("light_prefix", C.c_int32),
-                ("ungated_rows", C.c_int32), ("indices_by_position", C.c_int32), ("reserved_", C.c_int32)]
+                ("ungated_rows", C.c_int32), ("indices_by_position", C.c_int32), ("mask_int_count", C.c_int32)]
 
 
 # every symbol include/cumm_hip.h declares: name -> (restype, argtypes)
@@ -100,6 +100,9 @@ SYMBOLS = {
                                       _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP]),
     "cumm_hip_sort_by_mask_workspace": (C.c_size_t, [C.c_int]),
     "cumm_hip_sort_by_mask": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_masks_from_pairs": (C.c_int, [_VP, C.c_int, C.c_int, _VP, _VP]),
+    "cumm_hip_sort_by_mask_words_workspace": (C.c_size_t, [C.c_int]),
+    "cumm_hip_sort_by_mask_words": (C.c_int, [_VP, C.c_int, C.c_int, _VP, _VP, _VP, C.c_size_t, _VP]),
     "cumm_hip_pairs_by_position": (C.c_int, [_VP, _VP, C.c_int, C.c_int, _VP, _VP]),
     "cumm_hip_query_light_hint": (C.c_int, [_VP, C.c_int, C.c_uint32, C.POINTER(C.c_int32), _VP]),
     "cumm_hip_light_prefix": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP]),

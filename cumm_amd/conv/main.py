@@ -99,10 +99,13 @@ class ConvMainUnitTest:
             raise RuntimeError("error")
         if not (desp.split_k_serial or desp.split_k_parallel) and split_k_slices > 1:
             raise RuntimeError("algo don't support splitk but you provide split_k_slices > 1.")
-        if int(getattr(params, "mask_int_count", 1)) != 1:
-            # (tv::gemm::ConvParams::mask_int_count, params.h:413: several 32-bit words per position
-            # for kernel volumes above 32; those go through cumm_amd.conv.native here)
-            raise RuntimeError("one 32-bit mask word per position only (mask_int_count must be 1)")
+        # tv::gemm::ConvParams::mask_int_count (params.h:413): 32-bit mask words per position.  As in
+        # the reference's kernels the count follows from the descriptor and the kernel volume -
+        # ceil(kernel volume / 32) with dynamic_mask, else 1 (cumm/conv/kernel.py:827-838) - and the
+        # field may say the same thing or stay at its default of 1.
+        mask_words = (weight.dim(1) + 31) // 32 if desp.dynamic_mask else 1
+        if int(getattr(params, "mask_int_count", 1)) not in (1, mask_words):
+            raise RuntimeError("mask_int_count must be %d for this descriptor and kernel volume" % mask_words)
         K = weight.dim(0)
         C = inp.dim(1)
         if output.dim(1) != K:
@@ -175,7 +178,7 @@ class ConvMainUnitTest:
         if op_type == ConvOpType.BackwardWeight:
             if mask.dim(0) < (N + mask_width - 1) // mask_width:
                 raise RuntimeError("error")
-        elif mask.dim(0) < N:
+        elif mask.size < N * mask_words or (mask.ndim == 2 and mask.dim(1) != mask_words):
             raise RuntimeError("error")
         for t in (inp, weight, output):
             if not t.is_contiguous():
@@ -216,8 +219,8 @@ class ConvMainUnitTest:
         args.mask_ptr = _ptr(mask)
         if op_type == ConvOpType.Forward and not mask_output.empty():
             tiles = (N + desp.tile_shape[0] - 1) // desp.tile_shape[0]
-            if mask_output.dim(0) < tiles:
-                raise RuntimeError("mask_output needs one word per tile of tile_shape[0] positions")
+            if mask_output.size < tiles * mask_words:
+                raise RuntimeError("mask_output needs one word (mask_int_count words) per tile of tile_shape[0] positions")
             args.mask_out_ptr = _ptr(mask_output)
         args.indice_ptr = _ptr(indices)
         args.mask_argsort_ptr = _ptr(mask_argsort)

@@ -124,11 +124,16 @@ int gemm_family(const CummHipGemmDesc &d) {
 
 int conv_family(const CummHipConvDesc &c) {
   const CummHipGemmDesc &d = c.gemm;
-  if (!c.mask_sparse || c.dynamic_mask) return 0;
+  if (!c.mask_sparse) return 0;
   if (!same_dtype3(d) || !acc_ok(d)) return 0;
   const int tm = d.tile_shape[0], tn = d.tile_shape[1], tk = d.tile_shape[2];
   const int mk = d.dtype_a == CUMM_HIP_S8 ? 64 : 32;
   if (tk != mk) return 0;
+  // several mask words per position (kernel volumes above 32): forward and backward-input of
+  // two-byte elements on square tiles
+  if (c.dynamic_mask && (!(c.op_type == CUMM_HIP_OP_FORWARD || c.op_type == CUMM_HIP_OP_BACKWARD_INPUT) || d.dtype_a == CUMM_HIP_S8 ||
+                         wide_out(d) || tm != tn || d.split_k_serial || d.split_k_parallel))
+    return 0;
   if (d.split_k_parallel) {
     // only the balanced backward-weight kernel (fp32 atomic partial sums) splits "in parallel"
     if (c.op_type != CUMM_HIP_OP_BACKWARD_WEIGHT || d.dtype_a == CUMM_HIP_S8 || d.split_k_serial || wide_out(d)) return 0;
@@ -276,7 +281,7 @@ int take_async_errors(int32_t *timeouts, int32_t *sort_give_ups = nullptr) {
 }
 
 // ---- the table of light-prefix hints (launch.h): one per GPU, like `scratch`
-static __device__ int32_t light_hints[kLightHintSlots][8];
+static __device__ __align__(32) int32_t light_hints[kLightHintSlots + 1][8];   // (+ one slot that stays zero)
 int32_t *g_hints_ptr[kMaxDevices] = {};
 
 // the slot of a sorted mask array in the current device's table; NULL (and no error) if the
@@ -294,6 +299,12 @@ int32_t *light_hint_slot_ptr(const void *sorted_mask) {
     g_hints_ptr[dev] = reinterpret_cast<int32_t *>(ptr);
   }
   return g_hints_ptr[dev] + 8 * light_hint_slot(sorted_mask);
+}
+
+// a slot that names no array: the last one of the table, which light_hint_slot never returns
+const int32_t *light_hint_no_slot() {
+  const int32_t *first = light_hint_slot_ptr(nullptr);
+  return first ? first - 8 * light_hint_slot(nullptr) + 8 * kLightHintSlots : nullptr;
 }
 
 int report_async_errors() {
@@ -436,6 +447,20 @@ int cumm_hip_list_conv_algos(CummHipConvDesc *out, int cap) {
       fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, wide != 0);
       c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
       base(c, CUMM_HIP_OP_BACKWARD_INPUT);
+      v.push_back(c);
+    }
+    for (auto &t : sq_tiles) {
+      // the same two passes with dynamic_mask: ceil(kernel volume / 32) mask words per position
+      CummHipConvDesc c;
+      fill_gemm_desc(c.gemm, dt, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
+      base(c, CUMM_HIP_OP_FORWARD);
+      c.dynamic_mask = 1;
+      v.push_back(c);
+      fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0);
+      c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
+      base(c, CUMM_HIP_OP_BACKWARD_INPUT);
+      c.dynamic_mask = 1;
       v.push_back(c);
     }
     {
@@ -627,7 +652,13 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
   if (a->mode != CUMM_HIP_CONV_CROSS_CORRELATION)
     return fail(CUMM_HIP_EINVAL, "mode must be cross-correlation (1): the mask-based kernels implement nothing else");
   if (a->groups != 1) return fail(CUMM_HIP_EINVAL, "grouped convolution has no kernel (groups must be 1)");
-  if (kv > 32) return fail(CUMM_HIP_EINVAL, "kernel volume > 32 needs dynamic_mask, which this build has no kernel for");
+  // mask words per position: one, or with a dynamic_mask descriptor ceil(kv / 32) as in the
+  // reference's kernels (cumm/conv/kernel.py:827-838)
+  const int mask_words = c.dynamic_mask ? (kv + 31) / 32 : 1;
+  if (kv > 32 && !c.dynamic_mask) return fail(CUMM_HIP_EINVAL, "kernel volume > 32 needs a dynamic_mask descriptor");
+  if (kv > kMaxKernelVolume) return fail(CUMM_HIP_EINVAL, "kernel volume above %d", kMaxKernelVolume);
+  if (a->mask_int_count != 0 && a->mask_int_count != mask_words)
+    return fail(CUMM_HIP_EINVAL, "mask_int_count must be %d for this descriptor and kernel volume", mask_words);
   if (!a->ptr_A || !a->ptr_B || !a->ptr_C) return fail(CUMM_HIP_ERUNTIME, "input, weight and output must not be empty");
   if (!a->indice_ptr || !a->mask_ptr || !a->mask_argsort_ptr)
     return fail(CUMM_HIP_ERUNTIME, "indices, mask and mask_argsort must not be empty");
@@ -669,12 +700,18 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     p.read_source = a->beta != 0.0f;
     // (the hint only moves work between tile shapes; whatever it says the kernel covers every position once)
     p.pair_tiles = a->light_prefix > 0 && !a->ungated_rows ? a->light_prefix / 128 : 0;
-    // without a count from the caller: what input preparation left in the table for this mask array
-    if (a->light_prefix == 0 && !a->ungated_rows && d.tile_shape[0] == 64 && d.tile_shape[1] == 64)
-      p.hint_slot = light_hint_slot_ptr(a->mask_ptr);
+    // without a count from the caller: what input preparation left in the table for this mask array;
+    // with one, or without a table, a slot that names no array (the kernel reads it in any case)
+    if (a->light_prefix >= 0 && !a->ungated_rows && mask_words == 1 && d.tile_shape[0] == 64 && d.tile_shape[1] == 64)
+      p.hint_slot = a->light_prefix == 0 ? light_hint_slot_ptr(a->mask_ptr) : light_hint_no_slot();
     p.ungated_rows = a->ungated_rows != 0;
+    p.mask_words = mask_words;
+    if (mask_words > 1) {
+      p.pair_tiles = 0;
+      if ((int64_t)a->N * mask_words * 4 >= (int64_t)1 << 31) return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
+    }
     p.gather_by_pos = a->indices_by_position != 0;
-    p.n_mask_out = p.mask_out ? (a->N + d.tile_shape[0] - 1) / d.tile_shape[0] : 0;
+    p.n_mask_out = p.mask_out ? (a->N + d.tile_shape[0] - 1) / d.tile_shape[0] * mask_words : 0;
     if (c.is_int8_inference) {
       if (!a->bias_pointer || !a->scale_pointer)
         return fail(CUMM_HIP_ERUNTIME, "int8 inference must have both scale and bias");
@@ -1287,6 +1324,43 @@ int cumm_hip_pair_lists(const int32_t *indices, int kv, int n, int32_t *pair_in,
   p.kv = kv; p.n = n; p.chunks = (n + kPairListChunk - 1) / kPairListChunk;
   hipError_t e = launch_pair_lists(p, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "pair list launch");
+  return CUMM_HIP_OK;
+}
+
+int cumm_hip_masks_from_pairs(const int32_t *indices, int kv, int n, uint32_t *mask, void *stream) {
+  if (kv < 0 || n < 0 || kv > kMaxKernelVolume) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (kv == 0 || n == 0) return CUMM_HIP_OK;
+  if (!indices || !mask) return fail(CUMM_HIP_EINVAL, "indices and mask must not be empty");
+  hipError_t e = launch_masks_from_pairs(indices, mask, kv, n, reinterpret_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "mask launch");
+  return CUMM_HIP_OK;
+}
+
+size_t cumm_hip_sort_by_mask_words_workspace(int n) {
+  const size_t nn = (size_t)(n > 0 ? n : 1);
+  return 2 * ((4 * nn + 255) & ~(size_t)255) + cumm_hip_sort_by_mask_workspace(n);
+}
+
+int cumm_hip_sort_by_mask_words(const uint32_t *mask, int n, int words, uint32_t *sorted_mask, int32_t *argsort,
+                                void *workspace, size_t workspace_bytes, void *stream) {
+  if (n < 0 || words < 1 || words > 4) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (n == 0) return CUMM_HIP_OK;
+  if (n >= (1 << 30)) return fail(CUMM_HIP_EINVAL, "too many positions");
+  if (!mask || !sorted_mask || !argsort) return fail(CUMM_HIP_EINVAL, "mask, sorted_mask and argsort must not be empty");
+  if (mask == sorted_mask) return fail(CUMM_HIP_EINVAL, "the sort is not in place: mask and sorted_mask must differ");
+  if (!workspace || workspace_bytes < cumm_hip_sort_by_mask_words_workspace(n))
+    return fail(CUMM_HIP_ERUNTIME, "workspace at least %zu bytes.", cumm_hip_sort_by_mask_words_workspace(n));
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(CUMM_HIP_EINVAL, "workspace must be 256-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const size_t part = (4 * (size_t)n + 255) & ~(size_t)255;
+  char *base = reinterpret_cast<char *>(workspace);
+  uint32_t *keys = reinterpret_cast<uint32_t *>(base), *sorted_keys = reinterpret_cast<uint32_t *>(base + part);
+  int32_t *status = nullptr;
+  if (int rc = async_status_ptr(&status)) return rc;
+  hipError_t e = launch_mask_words_keys(mask, keys, n, words, s);
+  if (e == hipSuccess) e = launch_sort_by_mask(keys, n, 0xFFFFFFFFu, sorted_keys, argsort, base + 2 * part, status + 1, nullptr, s);
+  if (e == hipSuccess) e = launch_mask_words_gather(mask, argsort, sorted_mask, n, words, s);
+  if (e != hipSuccess) return hip_fail(e, "mask sort launch");
   return CUMM_HIP_OK;
 }
 

@@ -140,6 +140,9 @@ struct PairListsParams {
   int32_t *chunk_counts;    // [kv, chunks] scratch
   int32_t kv, n, chunks;
 };
+hipError_t launch_masks_from_pairs(const int32_t *indices, uint32_t *mask, int kv, int n, hipStream_t s);
+hipError_t launch_mask_words_keys(const uint32_t *mask, uint32_t *keys, int n, int words, hipStream_t s);
+hipError_t launch_mask_words_gather(const uint32_t *mask, const int32_t *argsort, uint32_t *sorted, int n, int words, hipStream_t s);
 hipError_t launch_pairs_by_position(const int32_t *indices, const int32_t *argsort, int32_t *out, int kv, int n, int rows,
                                     hipStream_t s);
 constexpr int kPairListChunk = 2048;   // table entries per workgroup

@@ -454,6 +454,50 @@ __global__ __launch_bounds__(256) void pair_lists_write_kernel(const PairListsPa
   }
 }
 
+// mask[o * words + w] = bit b set wherever indices[32 w + b][o] >= 0: the masks of a pair table,
+// any kernel volume (one lane per output, walking the offsets: every table row is read coalesced)
+__global__ __launch_bounds__(256) void masks_from_pairs_kernel(const int32_t *__restrict__ indices, uint32_t *__restrict__ mask,
+                                                               int kv, int n, int words) {
+  const int o = blockIdx.x * 256 + threadIdx.x;
+  if (o >= n) return;
+  for (int w = 0; w < words; ++w) {
+    uint32_t m = 0;
+    const int hi = kv - 32 * w < 32 ? kv - 32 * w : 32;
+    for (int b = 0; b < hi; ++b) m |= indices[(int64_t)(32 * w + b) * n + o] >= 0 ? 1u << b : 0u;
+    mask[(int64_t)o * words + w] = m;
+  }
+}
+
+// Sort key of a position with several mask words: positions with few offsets first (the number
+// of offsets in the upper six bits, at most 63), equal masks next to each other (a 26-bit hash of
+// the words below it).  Any order is a valid input of the convolution kernels; this one makes the
+// tiles of the light end light.
+__device__ __forceinline__ uint32_t mask_words_key(const uint32_t *w, int words) {
+  uint32_t pc = 0, h = 0;
+  for (int i = 0; i < words; ++i) {
+    pc += (uint32_t)__builtin_popcount(w[i]);
+    const int r = (7 * i) & 31;
+    h ^= r ? (w[i] << r) | (w[i] >> (32 - r)) : w[i];
+  }
+  return ((pc < 63u ? pc : 63u) << 26) | ((h * 0x9E3779B1u) >> 6);
+}
+__global__ __launch_bounds__(256) void mask_words_keys_kernel(const uint32_t *__restrict__ mask, uint32_t *__restrict__ keys,
+                                                              int n, int words) {
+  const int o = blockIdx.x * 256 + threadIdx.x;
+  if (o >= n) return;
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  for (int i = 0; i < words && i < 4; ++i) w[i] = mask[(int64_t)o * words + i];
+  keys[o] = mask_words_key(w, words < 4 ? words : 4);
+}
+__global__ __launch_bounds__(256) void mask_words_gather_kernel(const uint32_t *__restrict__ mask, const int32_t *__restrict__ argsort,
+                                                                uint32_t *__restrict__ sorted, int n, int words) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)n * words) return;
+  const int pos = (int)(i / words), w = (int)(i % words);
+  const int row = argsort[pos];
+  sorted[i] = row >= 0 && row < n ? mask[(int64_t)row * words + w] : 0u;
+}
+
 // out[k][pos] = indices[k][argsort[pos]]: the pair table in the order of the sorted positions
 __global__ __launch_bounds__(256) void pairs_by_position_kernel(const int32_t *__restrict__ indices,
                                                                 const int32_t *__restrict__ argsort,
@@ -466,6 +510,23 @@ __global__ __launch_bounds__(256) void pairs_by_position_kernel(const int32_t *_
 }
 
 }  // namespace
+
+hipError_t launch_masks_from_pairs(const int32_t *indices, uint32_t *mask, int kv, int n, hipStream_t s) {
+  if (kv <= 0 || n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(masks_from_pairs_kernel, dim3((n + 255) / 256), dim3(256), 0, s, indices, mask, kv, n, (kv + 31) / 32);
+  return hipGetLastError();
+}
+hipError_t launch_mask_words_keys(const uint32_t *mask, uint32_t *keys, int n, int words, hipStream_t s) {
+  if (n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(mask_words_keys_kernel, dim3((n + 255) / 256), dim3(256), 0, s, mask, keys, n, words);
+  return hipGetLastError();
+}
+hipError_t launch_mask_words_gather(const uint32_t *mask, const int32_t *argsort, uint32_t *sorted, int n, int words, hipStream_t s) {
+  if (n <= 0) return hipSuccess;
+  const int64_t total = (int64_t)n * words;
+  hipLaunchKernelGGL(mask_words_gather_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, mask, argsort, sorted, n, words);
+  return hipGetLastError();
+}
 
 hipError_t launch_pairs_by_position(const int32_t *indices, const int32_t *argsort, int32_t *out, int kv, int n, int rows,
                                     hipStream_t s) {

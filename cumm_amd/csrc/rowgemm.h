@@ -67,6 +67,8 @@ struct RowGemmParams {
   // preparation left for this mask array (light_hint_slot in launch.h); a slot that names another
   // array, length or filter says nothing
   const int32_t *hint_slot;
+  // 32-bit mask words per position (1; 2 to 4 for kernel volumes above 32: see rowgemm_lds_tile)
+  int32_t mask_words;
   // words the caller's mask_out array holds (a tile number beyond it is not written)
   int32_t n_mask_out;
   // non-zero: a row takes part in every kernel offset of its tile's mask (the reference's rule:

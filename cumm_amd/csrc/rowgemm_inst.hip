@@ -51,12 +51,36 @@ constexpr int lds_stages(int TM, int TN, int KS) {
   return 3 * stage <= 65536 ? 3 : (2 * stage <= 65536 ? 2 : 0);
 }
 
+// tile shapes and element types that have a kernel for several mask words per position
+template <class T, int TM, int TN>
+constexpr bool has_mask_words_kernel() { return Elem<T>::kBytes == 2 && !kWide && TM == TN; }
+
 template <class T, int NW, int RB, int TN, int KS, bool WT>
 static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   constexpr int TM = NW * RB * 16;
   dim3 grid((p.n_pos + TM - 1) / TM, (p.k_out + TN - 1) / TN, 1);
   if (grid.x == 0 || grid.y == 0) return hipSuccess;
   constexpr int chunk_e = 4 * KS * Elem<T>::kPerVec;
+  if (p.mask_words > 1) {
+    // kernel volumes above 32 (the reference's dynamic-mask kernels): the LDS-streaming kernel
+    // with up to four mask words per position, whole contraction or chunked
+    if constexpr (has_mask_words_kernel<T, TM, TN>()) {
+      if (WT ? p.w_stride_n != 1 : p.w_stride_c != 1) return hipErrorInvalidValue;
+      constexpr int KSM = KS == 4 ? 2 : KS;
+      constexpr int NSM = lds_stages(TM, TN, KSM);
+      if constexpr (NSM > 0) {
+        constexpr int chunk_m = 4 * KSM * Elem<T>::kPerVec;
+        RowGemmParams q = p;
+        const int nch = (p.c_in + chunk_m - 1) / chunk_m;
+        while ((1 << q.chunk_shift) < nch) ++q.chunk_shift;
+        if (q.chunk_shift <= 3 && counted_waits_hold<rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KSM, NSM, WT, false, 4>>()) {
+          hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, KSM, NSM, WT, false, 4>), grid, dim3(256), 0, s, q);
+          return hipGetLastError();
+        }
+      }
+    }
+    return hipErrorInvalidValue;
+  }
   // A contraction longer than 128 bytes: the LDS-streaming kernel with 128-byte stage rows (three
   // stages fit, three workgroups per CU) walking the contraction in chunks, rather than
   // 256-byte rows with two stages or the register-gather kernels.
@@ -82,7 +106,7 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
     // the LDS-streaming kernel: 2 x 2 waves, each TM/2 rows by TN/2 channels
     if (p.c_in <= chunk_e && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
       if constexpr (TM == 64 && TN == 64 && Elem<T>::kBytes == 2 && KS <= 2 && !kWide) {
-        if ((p.pair_tiles > 0 || p.hint_slot != nullptr) && grid.y == 1 && p.chunk_shift == 0 && p.mask != nullptr &&
+        if (p.hint_slot != nullptr && grid.y == 1 && p.chunk_shift == 0 && p.mask != nullptr &&
             counted_waits_hold<rowgemm_lds_mixed_kernel<T, KS, WT>>()) {
           hipLaunchKernelGGL((rowgemm_lds_mixed_kernel<T, KS, WT>), grid, dim3(256), 0, s, p);
           return hipGetLastError();

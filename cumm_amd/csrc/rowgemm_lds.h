@@ -65,8 +65,15 @@ struct LdsRing {
 
 // One tile: rows [tile * TM, tile * TM + TM) of the sorted positions, column block col.
 // HALVES: mask_out takes one word per 64 positions (a 128-row tile writes words 2 tile, 2 tile + 1).
-template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT, bool WIDE, bool HALVES>
+// MW: 32-bit mask words per position.  1 = one word (kernel volumes up to 32).  4 = the layout
+// of the reference's dynamic-mask kernels for larger volumes (MaskIGemmIteratorMaskLoaderDynamic,
+// cumm/gemm/blockmma/mma.py:78-269): p.mask_words = ceil(kv / 32) words per position, word w of
+// position pos at mask[pos * mask_words + w] holding offsets 32 w .. 32 w + 31; mask_out likewise
+// per tile; the filter applies to every word.
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT, bool WIDE, bool HALVES, int MW = 1>
 __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const int tile, const int col, const LdsRing &lds) {
+  static_assert(MW == 1 || MW == 4, "one mask word, or up to four");
+  static_assert(MW == 1 || !HALVES, "the two tile shapes of one launch take one mask word");
   using E = Elem<T>;
   using AccV = typename E::AccV;
   constexpr int NW = WM * WN;
@@ -120,24 +127,34 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   // dependent round trips (1.3 us of a one-offset tile's 3.8) instead of one.
   const bool has_mask = p.mask != nullptr;
   const bool has_rows = p.out_rows != nullptr;
-  const v4i rsw_mask = rsrc_words(p.mask, has_mask ? (uint32_t)p.n_pos * 4u : 0u);
+  const int mic = MW == 1 ? 1 : p.mask_words;     // words per position actually there
+  const v4i rsw_mask = rsrc_words(p.mask, has_mask ? (uint32_t)p.n_pos * 4u * (uint32_t)mic : 0u);
+  // byte offset of word w of a position's mask (pos_off of the position given)
+  auto word_off = [&](uint32_t pos_off4, int w) __attribute__((always_inline)) -> uint32_t {
+    if constexpr (MW == 1) return pos_off4;
+    else return pos_off4 != kOob && w < mic ? pos_off4 * (uint32_t)mic + 4u * (uint32_t)w : kOob;
+  };
   const v4i rsw_rows = rsrc_words(p.out_rows, has_rows ? (uint32_t)p.n_pos * 4u : 0u);
-  auto pos_off = [&](int pos) -> uint32_t { return pos >= 0 && pos < p.n_pos ? (uint32_t)pos * 4u : kOob; };
+  auto pos_off = [&](int pos) __attribute__((always_inline)) -> uint32_t { return pos >= 0 && pos < p.n_pos ? (uint32_t)pos * 4u : kOob; };
   constexpr int MKW = (TM + 63) / 64;
   const int lrow = lane / LPR;             // row inside a load instruction
   const int lchunk = lane % LPR;           // LDS chunk slot inside the row
   const int key_pos = pos_base + wave * RPW + lane;   // entries: lane l < RPW fetches the entry of row wave*RPW + l
-  int raw_mk[MKW], raw_key_row, raw_key_bits, raw_a_row[IPA], raw_a_bits[IPA], raw_o_row[RBW];
+  int raw_mk[MKW][MW], raw_key_row, raw_key_bits[MW], raw_a_row[IPA], raw_a_bits[IPA][MW], raw_o_row[RBW];
 #pragma unroll
   for (int i = 0; i < MKW; ++i)
-    raw_mk[i] = load_b32_hidden(rsw_mask, i * 64 + lane < TM ? pos_off(pos_base + i * 64 + lane) : kOob);
+#pragma unroll
+    for (int w = 0; w < MW; ++w)
+      raw_mk[i][w] = load_b32_hidden(rsw_mask, word_off(i * 64 + lane < TM ? pos_off(pos_base + i * 64 + lane) : kOob, w));
   raw_key_row = load_b32_hidden(rsw_rows, pos_off(key_pos));
-  raw_key_bits = load_b32_hidden(rsw_mask, pos_off(key_pos));
+#pragma unroll
+  for (int w = 0; w < MW; ++w) raw_key_bits[w] = load_b32_hidden(rsw_mask, word_off(pos_off(key_pos), w));
 #pragma unroll
   for (int t = 0; t < IPA; ++t) {
     const int pos = pos_base + (wave * IPA + t) * RPI + lrow;
     raw_a_row[t] = load_b32_hidden(rsw_rows, pos_off(pos));
-    raw_a_bits[t] = load_b32_hidden(rsw_mask, pos_off(pos));
+#pragma unroll
+    for (int w = 0; w < MW; ++w) raw_a_bits[t][w] = load_b32_hidden(rsw_mask, word_off(pos_off(pos), w));
   }
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb)
@@ -167,19 +184,27 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
 
   wait_vmcnt<0>();
 #pragma unroll
-  for (int i = 0; i < MKW; ++i) keep_after_wait(raw_mk[i]);
+  for (int i = 0; i < MKW; ++i)
+#pragma unroll
+    for (int w = 0; w < MW; ++w) keep_after_wait(raw_mk[i][w]);
   keep_after_wait(raw_key_row);
-  keep_after_wait(raw_key_bits);
+#pragma unroll
+  for (int w = 0; w < MW; ++w) keep_after_wait(raw_key_bits[w]);
 #pragma unroll
   for (int t = 0; t < IPA; ++t) {
     keep_after_wait(raw_a_row[t]);
-    keep_after_wait(raw_a_bits[t]);
+#pragma unroll
+    for (int w = 0; w < MW; ++w) keep_after_wait(raw_a_bits[t][w]);
   }
 #pragma unroll
   for (int rb = 0; rb < RBW; ++rb) keep_after_wait(raw_o_row[rb]);
-  uint32_t mk = 0;
+  uint32_t mk[MW];
 #pragma unroll
-  for (int i = 0; i < MKW; ++i) mk |= (uint32_t)raw_mk[i];
+  for (int w = 0; w < MW; ++w) {
+    mk[w] = 0;
+#pragma unroll
+    for (int i = 0; i < MKW; ++i) mk[w] |= (uint32_t)raw_mk[i][w];
+  }
 
   // ---- loader role of this lane: rows of the tile it fetches, weight rows it fetches
   auto swz = [](int row) { return KS == 1 ? (row >> 1) & 3 : ((row * KS) >> 2) & (LPR - 1); };
@@ -189,31 +214,100 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   // what the pair table was built from: bit clear = entry -1).  Entries and rows of the others
   // are not fetched at all: the 4-byte entries are scattered over the table, one memory sector
   // each, and on sparse offsets most rows of a tile have none.
-  auto row_bits = [&](int raw) -> uint32_t {
+  auto row_bits = [&](int raw) __attribute__((always_inline)) -> uint32_t {
     const uint32_t w = (uint32_t)raw;
     const uint32_t wr = __builtin_bitreverse32(w) >> ((32 - p.kv) & 31);
     return has_mask && !p.ungated_rows ? (p.reverse_mask ? wr : w) : ~0u;
   };
+  // The same for MW words: the kv-bit string over the words reversed end for end (bit j of the
+  // result = bit kv-1-j), as the reference's loader walks a reversed mask (mma.py:196-215).
+  // (The words of a row are one vector value, not an array: an array that is indexed through a
+  // select ends up in scratch memory, whose accesses would count in vmcnt.)
+  typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+  using Words = std::conditional_t<MW == 1, uint32_t, v4u>;
+  auto reverse_words = [&](const v4u m) __attribute__((always_inline)) -> v4u {
+    const int s = (mic * 32 - p.kv) & 31;     // unused bits at the top of the last word
+    const uint32_t b0 = __builtin_bitreverse32(m[0]), b1 = __builtin_bitreverse32(m[1]);
+    const uint32_t b2 = __builtin_bitreverse32(m[2]), b3 = __builtin_bitreverse32(m[3]);
+    // word i of the reversed string before the shift = reversed word mic-1-i
+    v4u r;
+    r[0] = mic == 4 ? b3 : (mic == 3 ? b2 : (mic == 2 ? b1 : b0));
+    r[1] = mic == 4 ? b2 : (mic == 3 ? b1 : (mic == 2 ? b0 : 0u));
+    r[2] = mic == 4 ? b1 : (mic == 3 ? b0 : 0u);
+    r[3] = mic == 4 ? b0 : 0u;
+    if (s == 0) return r;
+    v4u o;
+    o[0] = (r[0] >> s) | (r[1] << (32 - s));
+    o[1] = (r[1] >> s) | (r[2] << (32 - s));
+    o[2] = (r[2] >> s) | (r[3] << (32 - s));
+    o[3] = r[3] >> s;
+    return o;
+  };
+  auto row_words = [&](const int (&raw)[MW]) __attribute__((always_inline)) -> Words {
+    if constexpr (MW == 1) {
+      return row_bits(raw[0]);
+    } else {
+      v4u m = {(uint32_t)raw[0], (uint32_t)raw[1], (uint32_t)raw[2], (uint32_t)raw[3]};
+      if (p.reverse_mask) m = reverse_words(m);
+      if (!has_mask || p.ungated_rows) m = v4u{~0u, ~0u, ~0u, ~0u};
+      return m;
+    }
+  };
+  // bit k of a row's words (k wave-uniform; k < 0 comes with a descriptor without records)
+  auto has_bit = [&](const Words m, int k) __attribute__((always_inline)) -> uint32_t {
+    if constexpr (MW == 1) {
+      return (m >> (k & 31)) & 1u;
+    } else {
+      const uint32_t v = k < 32 ? m[0] : (k < 64 ? m[1] : (k < 96 ? m[2] : m[3]));
+      return (v >> (k & 31)) & 1u;
+    }
+  };
   // memory row of a sorted position (the position itself without an argsort), -1 past the end
-  auto row_of = [&](int pos, int raw) -> int { return pos < p.n_pos ? (has_rows ? raw : pos) : -1; };
+  auto row_of = [&](int pos, int raw) __attribute__((always_inline)) -> int { return pos < p.n_pos ? (has_rows ? raw : pos) : -1; };
   uint32_t key_off = kOob;
-  uint32_t key_bits = 0;
+  Words key_bits;
   {
     const int pos = key_pos;
     const int row = row_of(pos, raw_key_row);
     const int key = lane < RPW && pos < p.n_pos ? (p.gather_by_pos ? pos : row) : -1;
     key_off = key >= 0 && key < p.n_idx ? (uint32_t)key * 4u : kOob;
-    key_bits = lane < RPW ? row_bits(raw_key_bits) : 0u;
+    key_bits = row_words(raw_key_bits);
+    if (lane >= RPW) key_bits = Words{};
   }
   // ---- tile mask: OR over the tile's positions (cumm/conv/kernel.py:844-889 of the reference)
   uint32_t kmask = 1u;
+  uint32_t kwords[MW];         // MW > 1: the tile mask, word by word (kmask is then unused)
+#pragma unroll
+  for (int w = 0; w < MW; ++w) kwords[w] = w == 0 ? 1u : 0u;
   bool half_skipped = false;   // HALVES: this wave's 64 positions would have been a skipped 64-row tile
-  if (has_mask) {
-    kmask = wave_or_dpp(mk) & p.mask_filter;
+  if constexpr (MW > 1) {
+    if (has_mask) {
+      uint32_t any = 0;
+#pragma unroll
+      for (int w = 0; w < MW; ++w) {
+        kwords[w] = wave_or_dpp(mk[w]) & p.mask_filter;
+        any |= kwords[w];
+        if (p.mask_out != nullptr && tid == 0 && col == 0 && w < mic && tile * mic + w < p.n_mask_out)
+          p.mask_out[tile * mic + w] = kwords[w];
+      }
+      if (p.exit_on_empty && any == 0) return;
+      if (p.reverse_mask) {
+        const v4u t = reverse_words(v4u{kwords[0], kwords[MW > 1 ? 1 : 0], kwords[MW > 2 ? 2 : 0], kwords[MW > 3 ? 3 : 0]});
+#pragma unroll
+        for (int w = 0; w < MW; ++w) kwords[w] = t[w];
+      }
+#pragma unroll
+      for (int w = 0; w < MW; ++w) {
+        const int left = p.kv - 32 * w;       // offsets this word may name
+        kwords[w] = left >= 32 ? kwords[w] : (left > 0 ? kwords[w] & ((1u << left) - 1u) : 0u);
+      }
+    }
+  } else if (has_mask) {
+    kmask = wave_or_dpp(mk[0]) & p.mask_filter;
     if constexpr (HALVES) {
       static_assert(!HALVES || (MKW == 2 && WM == 2), "two mask words of 64 positions, one per row of waves");
-      const uint32_t lo = wave_or_dpp((uint32_t)raw_mk[0]) & p.mask_filter;
-      const uint32_t hi = wave_or_dpp((uint32_t)raw_mk[MKW - 1]) & p.mask_filter;
+      const uint32_t lo = wave_or_dpp((uint32_t)raw_mk[0][0]) & p.mask_filter;
+      const uint32_t hi = wave_or_dpp((uint32_t)raw_mk[MKW - 1][0]) & p.mask_filter;
       half_skipped = p.exit_on_empty && (wm == 0 ? lo : hi) == 0u;
       if (p.mask_out != nullptr && tid == 0 && col == 0) {
         if (2 * tile < p.n_mask_out) p.mask_out[2 * tile] = lo;
@@ -227,7 +321,13 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
     if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
   }
   // a step = one kernel offset x one chunk of the contraction (one chunk unless chunk_shift)
-  const int n_steps = __builtin_popcount(kmask) << p.chunk_shift;
+  int n_offsets = __builtin_popcount(kmask);
+  if constexpr (MW > 1) {
+    n_offsets = 0;
+#pragma unroll
+    for (int w = 0; w < MW; ++w) n_offsets += __builtin_popcount(kwords[w]);
+  }
+  const int n_steps = n_offsets << p.chunk_shift;
 
 
   const uint32_t g_k_bytes = (uint32_t)p.n_idx * 4u;
@@ -236,17 +336,59 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   // lane j of klist holds the j-th kernel offset of the tile (-1 past the end): lane b pushes
   // b+1 to the lane of its rank among the set bits, lanes without a bit push into lane 63, which
   // nobody reads; a lane nobody pushed to reads 0.
-  int klist;
-  {
+  // With several mask words the list takes two registers (up to 128 offsets) and every lane works
+  // out its own entry: the tile's words are wave-uniform, so lane j picks the word that holds the
+  // offset of rank j and finds the position of that set bit by halving.
+  constexpr int KL = MW == 1 ? 1 : 2;
+  int klist[KL];
+  if constexpr (MW == 1) {
     const bool bit = lane < 32 && ((kmask >> lane) & 1u);
     const int rank = __builtin_popcount(kmask & ((1u << (lane & 31)) - 1u));
-    klist = __builtin_amdgcn_ds_permute(bit ? rank * 4 : 63 * 4, bit ? lane + 1 : 0) - 1;
+    klist[0] = __builtin_amdgcn_ds_permute(bit ? rank * 4 : 63 * 4, bit ? lane + 1 : 0) - 1;
+  } else {
+#pragma unroll
+    for (int h = 0; h < KL; ++h) {
+      int r = h * 64 + lane;          // rank wanted
+      uint32_t m = 0;
+      int base = 0;
+      bool found = false;
+#pragma unroll
+      for (int w = 0; w < MW; ++w) {
+        const int c = __builtin_popcount(kwords[w]);
+        const bool here = !found && r < c;
+        m = here ? kwords[w] : m;
+        base = here ? 32 * w : base;
+        found = found || here;
+        r = found ? r : r - c;
+      }
+      int pos = 0;
+#pragma unroll
+      for (int width = 16; width >= 1; width >>= 1) {
+        const int c = __builtin_popcount(m & ((1u << width) - 1u));
+        const bool up = r >= c;
+        pos += up ? width : 0;
+        r -= up ? c : 0;
+        m = up ? m >> width : m;
+      }
+      klist[h] = found ? base + pos : -1;
+    }
   }
+  // kernel offset of step j (-1 past the end of the tile's list)
+  auto k_of_step = [&](int j) __attribute__((always_inline)) -> int {
+    const int i = j >> p.chunk_shift;
+    if constexpr (MW == 1) {
+      return __builtin_amdgcn_readlane(klist[0], i & 63);
+    } else {
+      const int lo = __builtin_amdgcn_readlane(klist[0], i & 63);
+      const int hi = __builtin_amdgcn_readlane(klist[KL - 1], i & 63);
+      return i < 64 ? lo : (i < 128 ? hi : -1);
+    }
+  };
 
-  auto issue_idx = [&](int j, int *slot) {
-    const int k = __builtin_amdgcn_readlane(klist, (j >> p.chunk_shift) & 63);
+  auto issue_idx = [&](int j, int *slot) __attribute__((always_inline)) {
+    const int k = k_of_step(j);
     const v4i rs = rsrc_words(p.gather, k >= 0 ? g_bytes : 0u);
-    dma_b32(rs, lds_addr(slot), (key_bits >> (k & 31)) & 1u ? key_off : kOob, (uint32_t)k * g_k_bytes);
+    dma_b32(rs, lds_addr(slot), has_bit(key_bits, k) ? key_off : kOob, (uint32_t)k * g_k_bytes);
   };
   // The entries of the first offsets are requested now; the address work below (row chunks, weight
   // rows, fragment slots) overlaps their round trip.
@@ -260,13 +402,13 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
 
   int a_key[IPA];          // without a pair table the gathered row is the key itself
   uint32_t a_col[IPA];     // byte offset of the fetched chunk inside the gathered row, or kOob
-  uint32_t a_bits[IPA];    // mask word of the row
+  Words a_bits[IPA];       // mask words of the row
   int a_cpos[IPA];         // first contraction element of the fetched chunk (in the first chunk of the row)
 #pragma unroll
   for (int t = 0; t < IPA; ++t) {
     const int r = (wave * IPA + t) * RPI + lrow;
     const int pos = pos_base + r;
-    a_bits[t] = row_bits(raw_a_bits[t]);
+    a_bits[t] = row_words(raw_a_bits[t]);
     const int row = row_of(pos, raw_a_row[t]);
     const int key = pos < p.n_pos ? (p.gather_by_pos ? pos : row) : -1;
     a_key[t] = key >= 0 && key < p.n_idx ? key : -1;
@@ -379,13 +521,13 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   const uint32_t w_k_bytes = (uint32_t)p.w_stride_k * E::kBytes;
 
   // entries of this lane's rows out of the wave's slot (its own loads: no barrier needed)
-  auto read_idx = [&](const int *slot, int (&dst)[IPA]) {
+  auto read_idx = [&](const int *slot, int (&dst)[IPA]) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < IPA; ++t) dst[t] = has_gather ? slot[t * RPI + lrow] : a_key[t];
   };
   constexpr int CHUNK_E = LPR * PV;      // contraction elements of a stage row
-  auto issue_operands = [&](int j, const int (&src)[IPA], v4i *st, v4i *stw) {
-    const int k = __builtin_amdgcn_readlane(klist, (j >> p.chunk_shift) & 63);
+  auto issue_operands = [&](int j, const int (&src)[IPA], v4i *st, v4i *stw) __attribute__((always_inline)) {
+    const int k = k_of_step(j);
     const int cc = j & ((1 << p.chunk_shift) - 1);          // chunk of the contraction
     const int cc_e = cc * CHUNK_E;                           // its first element
     const uint32_t cc_b = (uint32_t)cc * (LPR * 16u);        // ... as bytes inside a row
@@ -396,7 +538,7 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
       // a_col is out of range already for a row without a key or a chunk past the contraction;
       // adding a row offset below 2 GiB keeps it out of range
       const uint32_t v = (uint32_t)src[t];
-      const uint32_t voff = v < (uint32_t)p.rows_a && ((a_bits[t] >> (k & 31)) & 1u) && cc_e + a_cpos[t] < p.c_in
+      const uint32_t voff = v < (uint32_t)p.rows_a && has_bit(a_bits[t], k) && cc_e + a_cpos[t] < p.c_in
                                 ? v * a_row_bytes + a_col[t] + cc_b
                                 : kOob;
       dma_b128(rs_a, lds_addr(st + (wave * IPA + t) * 64), voff, 0u);
@@ -583,7 +725,7 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   }
 }
 
-template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT = false, bool WIDE = false>
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT = false, bool WIDE = false, int MW = 1>
 __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmParams p) {
   constexpr int NW = WM * WN;
   constexpr int LPR = 4 * KS;
@@ -624,7 +766,7 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
     }
   }
   const int tile = (int)gridDim.x - 1 - tile_rank;  // heaviest tiles first (masks sorted ascending)
-  rowgemm_lds_tile<T, WM, WN, RBW, NBW, KS, NS, WT, WIDE, false>(p, tile, col, lds);
+  rowgemm_lds_tile<T, WM, WN, RBW, NBW, KS, NS, WT, WIDE, false, MW>(p, tile, col, lds);
 }
 
 // Tiles of two shapes in one launch, for one column block of 64 channels (grid.x = number of
@@ -648,15 +790,18 @@ __global__ __launch_bounds__(256) void rowgemm_lds_mixed_kernel(const RowGemmPar
   __shared__ int ix0[4][64];
   __shared__ int ix1[4][64];
   __shared__ int ix2[4][64];
-  const int tiles = (int)gridDim.x;
-  int hinted = p.pair_tiles;
-  if (hinted == 0 && p.hint_slot != nullptr) {
-    // (uniform addresses: scalar loads, issued with the kernel arguments' own)
-    const uint64_t key = (uint64_t)(uint32_t)p.hint_slot[0] | ((uint64_t)(uint32_t)p.hint_slot[1] << 32);
-    const bool named = key == (uint64_t)p.mask && p.hint_slot[2] == p.n_pos && (uint32_t)p.hint_slot[3] == p.mask_filter;
-    const int prefix = p.hint_slot[4];
-    hinted = named && prefix > 0 ? prefix >> 7 : 0;
-  }
+  const int tiles = (p.n_pos + 63) >> 6;      // = gridDim.x, without waiting for the dispatch packet's own load
+  // The slot is read whole and without conditions - one scalar load of 32 bytes, one round trip -
+  // and compared without short cuts (a chain of && became a chain of dependent loads, each with
+  // its own wait); the host always passes a slot, an all-zero one when there is no table.
+  typedef int v8i __attribute__((ext_vector_type(8)));
+  const v8i slot = *reinterpret_cast<const v8i *>(p.hint_slot);
+  const uint64_t mask_addr = (uint64_t)p.mask;
+  const bool named = (slot[0] == (int)(uint32_t)mask_addr) & (slot[1] == (int)(uint32_t)(mask_addr >> 32)) &
+                     (slot[2] == p.n_pos) & (slot[3] == (int)p.mask_filter) & (slot[4] > 0);
+  // (a count from the caller comes with a slot that names nothing: one of the two is zero, and the
+  // OR keeps the slot's load out of a branch, where it would wait for the pointer first)
+  const int hinted = p.pair_tiles | (named ? slot[4] >> 7 : 0);
   const int pairs = hinted < (tiles >> 1) ? hinted : (tiles >> 1);
   const int singles = tiles - 2 * pairs;
   const int rank = (int)blockIdx.x;

@@ -163,6 +163,41 @@ def light_prefix(sorted_mask: np.ndarray, mask_filter: int = 0xFFFFFFFF) -> int:
     return int(heavy[0] if heavy.size else runs) * 128
 
 
+def masks_from_pairs(indices: np.ndarray) -> np.ndarray:
+    """Masks of a pair table [kv, N] of any kernel volume: [N, ceil(kv / 32)] uint32, bit b of word w
+    set wherever ``indices[32 w + b][o] >= 0`` - the layout the reference's dynamic-mask kernels read
+    (``mask_ptr[mask_int_count * pos + word]``, cumm/gemm/blockmma/mma.py:176-190)."""
+    kv, n = indices.shape
+    words = (kv + 31) // 32
+    out = np.zeros((n, words), np.uint32)
+    for k in range(kv):
+        out[:, k // 32] |= np.where(indices[k] >= 0, np.uint32(1 << (k % 32)), np.uint32(0)).astype(np.uint32)
+    return out
+
+
+def mask_words_keys(mask: np.ndarray) -> np.ndarray:
+    """Sort key of positions with several mask words [N, words]: the number of offsets (at most
+    63) in the upper six bits, a 26-bit hash of the words below - few offsets first, equal masks
+    together."""
+    mask = np.asarray(mask, np.uint32)
+    pc = np.zeros(mask.shape[0], np.uint32)
+    h = np.zeros(mask.shape[0], np.uint32)
+    for i in range(mask.shape[1]):
+        w = mask[:, i]
+        for b in range(32):
+            pc += (w >> np.uint32(b)) & np.uint32(1)
+        r = (7 * i) & 31
+        h ^= ((w << np.uint32(r)) | (w >> np.uint32(32 - r))).astype(np.uint32) if r else w
+    h = ((h.astype(np.uint64) * np.uint64(0x9E3779B1)) & np.uint64(0xFFFFFFFF)).astype(np.uint32) >> np.uint32(6)
+    return ((np.minimum(pc, 63).astype(np.uint32) << np.uint32(26)) | h).astype(np.uint32)
+
+
+def sort_by_mask_words(mask: np.ndarray):
+    """(sorted masks [N, words], argsort): stable ascending sort by :func:`mask_words_keys`."""
+    order = np.argsort(mask_words_keys(mask), kind="stable").astype(np.int32)
+    return np.ascontiguousarray(np.asarray(mask, np.uint32)[order]), order
+
+
 def pairs_by_position(indices: np.ndarray, mask_argsort: np.ndarray) -> np.ndarray:
     """The pair table in the order of the sorted positions: ``out[k][pos] = indices[k][mask_argsort[pos]]``
     (what ``ConvParams.indices_by_position`` takes; the reference's iterator forms this index per
@@ -348,6 +383,36 @@ def light_hint_device(sorted_mask, mask_filter: int = 0xFFFFFFFF, stream: int = 
     _capi.check(_capi.lib().cumm_hip_query_light_hint(sorted_mask.byte_pointer(), int(sorted_mask.shape[0]),
                                                       int(mask_filter) & 0xFFFFFFFF, ctypes.byref(out), stream))
     return int(out.value)
+
+
+def masks_from_pairs_device(indices, stream: int = 0):
+    """:func:`masks_from_pairs` of a device table [kv, N]: a device tensor [N, ceil(kv / 32)] uint32."""
+    from . import _capi
+    from . import tensorview as tv
+    if indices.device < 0 or indices.dtype != tv.int32 or indices.ndim != 2:
+        raise ValueError("indices must be a device int32 tensor [kv, N]")
+    kv, n = int(indices.shape[0]), int(indices.shape[1])
+    out = tv.empty([n, (kv + 31) // 32], tv.uint32, 0)
+    _capi.check(_capi.lib().cumm_hip_masks_from_pairs(indices.byte_pointer(), kv, n, out.byte_pointer(), stream))
+    return out
+
+
+def sort_by_mask_words_device(mask, workspace=None, stream: int = 0):
+    """:func:`sort_by_mask_words` of a device tensor [N, words] uint32 (1 to 4 words)."""
+    from . import _capi
+    from . import tensorview as tv
+    if mask.device < 0 or mask.dtype != tv.uint32 or mask.ndim != 2 or not 1 <= int(mask.shape[1]) <= 4:
+        raise ValueError("mask must be a device uint32 tensor [N, 1..4]")
+    n, words = int(mask.shape[0]), int(mask.shape[1])
+    lib = _capi.lib()
+    need = int(lib.cumm_hip_sort_by_mask_words_workspace(n))
+    if workspace is None or workspace.empty():
+        workspace = tv.empty([max(need, 256)], tv.uint8, 0)
+    out_mask = tv.empty([n, words], tv.uint32, 0)
+    order = tv.empty([n], tv.int32, 0)
+    _capi.check(lib.cumm_hip_sort_by_mask_words(mask.byte_pointer(), n, words, out_mask.byte_pointer(), order.byte_pointer(),
+                                                workspace.byte_pointer(), workspace.nbytes, stream))
+    return out_mask, order
 
 
 def pairs_by_position_device(indices, mask_argsort, out=None, stream: int = 0):

@@ -91,7 +91,7 @@ def _desp_like(dtype, op, parallel=False):
     if key not in _DESP_LIKE:
         for d in ConvMainUnitTest.get_all_conv_algo_desp():
             if (d.dtype_a == dtype and d.dtype_c == dtype and ConvOpType(d.op_type) == op and not d.is_int8_inference and
-                    bool(d.split_k_parallel) == parallel and d.mask_sparse):
+                    bool(d.split_k_parallel) == parallel and d.mask_sparse and not d.dynamic_mask):
                 _DESP_LIKE[key] = d
                 break
         else:

@@ -61,7 +61,7 @@ def conv_candidates(params: ConvParams, desps: Optional[List[ConvAlgoDesp]] = No
     for d in (desps if desps is not None else ConvMainUnitTest.get_all_conv_algo_desp()):
         if (d.op_type != cur.op_type or d.ndim != cur.ndim or not d.mask_sparse or
                 (d.dtype_a, d.dtype_b, d.dtype_c) != (cur.dtype_a, cur.dtype_b, cur.dtype_c) or
-                d.is_int8_inference != cur.is_int8_inference or
+                d.is_int8_inference != cur.is_int8_inference or bool(d.dynamic_mask) != bool(cur.dynamic_mask) or
                 (d.layout_i, d.layout_w, d.layout_o) != (cur.layout_i, cur.layout_w, cur.layout_o)):
             continue
         if params.split_k_slices > 1 and not (d.split_k_serial or d.split_k_parallel):

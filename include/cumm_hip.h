@@ -149,7 +149,12 @@ typedef struct CummHipSparseConvArgs {
                                        memory instead of one memory sector apiece.  Same results either way.  No
                                        counterpart in the reference, whose iterator reads the table by output row
                                        (cumm/conv/sparse_iters.py:280-357). */
-  int32_t reserved_;
+  int32_t mask_int_count;           /* tv::gemm::ConvParams::mask_int_count (params.h:413): 32-bit mask words per position.
+                                       0 = whatever the descriptor implies: 1, or ceil(kernel_volume / 32) with a
+                                       dynamic_mask descriptor - mask_ptr is then [N, words] and mask_out_ptr
+                                       [tiles, words], word w holding offsets 32 w .. 32 w + 31, mask_filter applying to
+                                       every word (MaskIGemmIteratorMaskLoaderDynamic, cumm/gemm/blockmma/mma.py:78-269).
+                                       Any other value than that is an error. */
 } CummHipSparseConvArgs;
 
 /* Replaces GemmMainUnitTest.matmul2 below its prelude
@@ -323,6 +328,19 @@ int cumm_hip_conv_pairs_fill(const int32_t *coords, int n_in, int batch_size, co
 size_t cumm_hip_pair_lists_workspace(int kv, int n);
 int cumm_hip_pair_lists(const int32_t *indices, int kv, int n, int32_t *pair_in, int32_t *pair_out, int32_t *counts,
                         void *workspace, size_t workspace_bytes, void *stream);
+
+/* Masks of a pair table, any kernel volume up to 128: mask [n, words], words = ceil(kv / 32), bit b of
+ * word w of output o set wherever indices[32 w + b][o] >= 0 (the layout a dynamic_mask descriptor takes;
+ * one word per output for kernel volumes up to 32, where it equals what the table builders write).
+ * cumm_hip_sort_by_mask_words: an order for positions with 1 .. 4 mask words - ascending number of offsets,
+ * equal masks adjacent (a stable sort by a 32-bit key made of the two) - with sorted_mask [n, words] =
+ * the masks in that order and argsort [n]; workspace of cumm_hip_sort_by_mask_words_workspace(n) bytes,
+ * 256-byte aligned.  The reference's callers take both steps from spconv for its dynamic-mask kernels
+ * (cumm/conv/kernel.py:827-838); any order is valid input, this one keeps the light tiles light. */
+int cumm_hip_masks_from_pairs(const int32_t *indices, int kv, int n, uint32_t *mask, void *stream);
+size_t cumm_hip_sort_by_mask_words_workspace(int n);
+int cumm_hip_sort_by_mask_words(const uint32_t *mask, int n, int words, uint32_t *sorted_mask, int32_t *argsort,
+                                void *workspace, size_t workspace_bytes, void *stream);
 
 /* The pair table in the order of the sorted positions: out[k][pos] = indices[k][mask_argsort[pos]] for
  * indices [kv, n] and mask_argsort [n] (an argsort entry outside [0, n) gives -1); out [kv, n], not the

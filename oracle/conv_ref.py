@@ -25,13 +25,41 @@ def bitrev32(x):
 def tile_masks(mask_sorted, tile_m, mask_filter=0xFFFFFFFF):
     """kmask per tile of ``tile_m`` consecutive sorted positions:
     OR of the tile's mask words, AND mask_filter
-    (cumm/conv/kernel.py:844-864 of the reference)."""
+    (cumm/conv/kernel.py:844-864 of the reference).
+
+    ``mask_sorted`` [N, words] (the dynamic-mask layout for kernel volumes above 32: word w of
+    a position holds offsets 32 w .. 32 w + 31) gives [tiles, words]: every word is reduced and
+    filtered by itself (``load_mask``, cumm/gemm/blockmma/mma.py:176-204 of the reference)."""
+    if mask_sorted.ndim == 2:
+        return np.stack([tile_masks(np.ascontiguousarray(mask_sorted[:, w]), tile_m, mask_filter)
+                         for w in range(mask_sorted.shape[1])], axis=1)
     n = mask_sorted.shape[0]
     nt = (n + tile_m - 1) // tile_m
     padded = np.zeros(nt * tile_m, dtype=np.uint32)
     padded[:n] = mask_sorted
     red = np.bitwise_or.reduce(padded.reshape(nt, tile_m), axis=1)
     return (red & np.uint32(mask_filter)).astype(np.uint32)
+
+
+def _tile_has_offset(kmask_tiles, k):
+    """Per tile: does the (possibly several-word) tile mask name kernel offset k?"""
+    if kmask_tiles.ndim == 2:
+        return ((kmask_tiles[:, k // 32] >> np.uint32(k % 32)) & 1).astype(bool)
+    return ((kmask_tiles >> np.uint32(k)) & 1).astype(bool)
+
+
+def reverse_mask_words(words, kv):
+    """The kv-bit string held in 32-bit words (bit j of the string = bit j % 32 of word j // 32)
+    reversed end for end: what the reference's loader walks with ``reverse``
+    (cumm/gemm/blockmma/mma.py:141-147, 196-215: words from the last to the first, each
+    bit-reversed, starting ``words * 32 - kv`` bits in).  Written bit by bit on purpose."""
+    words = np.asarray(words, dtype=np.uint32)
+    out = np.zeros_like(words)
+    for j in range(kv):
+        src = kv - 1 - j
+        bit = (words[..., src // 32] >> np.uint32(src % 32)) & np.uint32(1)
+        out[..., j // 32] |= (bit << np.uint32(j % 32)).astype(np.uint32)
+    return out
 
 
 def _epilogue(acc, src, alpha, beta, act, act_alpha, act_beta, dtype_out):
@@ -64,7 +92,7 @@ def implicit_gemm_fwd_ref(inp, weight, output, indices, mask_sorted, mask_argsor
     acc_dtype = np.int32 if _is_int(dtype_in) else np.float32
     acc = np.zeros((n, k_out), dtype=np.float64 if _is_int(dtype_in) else np.float32)
     for k in range(kv):
-        active = ((kmask_tiles[tile_of_pos] >> np.uint32(k)) & 1).astype(bool)
+        active = _tile_has_offset(kmask_tiles, k)[tile_of_pos]
         o = rows[active]
         i = indices[k][o]
         valid = i >= 0
@@ -116,14 +144,17 @@ def implicit_gemm_dgrad_ref(dout, weight, dinp, indices_bwd, mask_sorted, mask_a
     kv = indices_bwd.shape[0]
     c_in = weight.shape[2]
     kmask_tiles = tile_masks(mask_sorted[:n], tile_m, mask_filter)
-    live_tile = kmask_tiles != 0
+    live_tile = kmask_tiles != 0 if kmask_tiles.ndim == 1 else np.any(kmask_tiles != 0, axis=1)
     if reverse_mask:
-        kmask_tiles = (bitrev32(kmask_tiles) >> np.uint32(32 - kv)).astype(np.uint32)
+        if kmask_tiles.ndim == 2:
+            kmask_tiles = reverse_mask_words(kmask_tiles, kv)
+        else:
+            kmask_tiles = (bitrev32(kmask_tiles) >> np.uint32(32 - kv)).astype(np.uint32)
     tile_of_pos = np.arange(n) // tile_m
     rows = mask_argsort[:n].astype(np.int64)
     acc = np.zeros((n, c_in), dtype=np.float32)
     for k in range(kv):
-        active = ((kmask_tiles[tile_of_pos] >> np.uint32(k)) & 1).astype(bool)
+        active = _tile_has_offset(kmask_tiles, k)[tile_of_pos]
         o = rows[active]
         i = indices_bwd[k][o]
         valid = i >= 0

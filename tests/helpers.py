@@ -69,15 +69,18 @@ def rel_err_rows(got_f32, ref_f32, floor_frac=1e-2):
     return float(np.max(np.max(np.abs(g - r), axis=1) / denom))
 
 
-def find_conv_desp(dtype, op, tile_m, tile_n, int8_inference=False, split_k_parallel=False, dtype_out=None):
-    """``dtype_out``: element type of the result when it differs from the operands' ("s32", "f32")."""
+def find_conv_desp(dtype, op, tile_m, tile_n, int8_inference=False, split_k_parallel=False, dtype_out=None,
+                   dynamic_mask=False):
+    """``dtype_out``: element type of the result when it differs from the operands' ("s32", "f32");
+    ``dynamic_mask``: the descriptors for kernel volumes above 32 (several mask words per position)."""
     for d in ConvMainUnitTest.get_all_conv_algo_desp():
         if (d.dtype_a == TV_DTYPE[dtype] and d.dtype_output == TV_DTYPE[dtype_out or dtype] and
                 d.dtype_input == TV_DTYPE[dtype] and ConvOpType(d.op_type) == op and
                 d.tile_shape[0] == tile_m and d.tile_shape[1] == tile_n and
-                d.is_int8_inference == int8_inference and d.split_k_parallel == split_k_parallel):
+                d.is_int8_inference == int8_inference and d.split_k_parallel == split_k_parallel and
+                bool(d.dynamic_mask) == dynamic_mask):
             return d
-    raise KeyError((dtype, op, tile_m, tile_n, int8_inference, split_k_parallel))
+    raise KeyError((dtype, op, tile_m, tile_n, int8_inference, split_k_parallel, dynamic_mask))
 
 
 def find_gemm_desp(dtype, shuffle, tile_m, tile_n, trans_a, trans_b, trans_c=False, dtype_c=None):

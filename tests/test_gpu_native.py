@@ -56,7 +56,8 @@ def test_pair_tables_and_lists_bit_exact(case):
         np.testing.assert_array_equal(gout[k][:n], want.pair_out[k][:n])
 
 
-def test_mask_kernels_still_reject_large_kernel_volumes():
+def test_static_mask_descriptors_reject_large_kernel_volumes():
+    """One mask word per position describes 32 offsets: a descriptor without dynamic_mask refuses more."""
     p = ConvParams(3, ConvOpType.Forward)
     p.conv_algo_desp = H.find_conv_desp("f16", ConvOpType.Forward, 64, 64)
     n = 100
@@ -66,6 +67,120 @@ def test_mask_kernels_still_reject_large_kernel_volumes():
     p.mask, p.mask_argsort = tv.zeros([n], tv.uint32, 0), tv.zeros([n], tv.int32, 0)
     with pytest.raises(ValueError, match="kernel volume"):
         ConvMainUnitTest.implicit_gemm2(p)
+    p.conv_algo_desp = H.find_conv_desp("f16", ConvOpType.Forward, 64, 64, dynamic_mask=True)
+    p.mask_int_count = 2                      # four words for 125 offsets, nothing else
+    with pytest.raises(RuntimeError, match="mask_int_count"):
+        ConvMainUnitTest.implicit_gemm2(p)
+    with pytest.raises(RuntimeError):         # masks of one word per position: too short
+        p.mask_int_count = 4
+        ConvMainUnitTest.implicit_gemm2(p)
+
+
+@pytest.mark.parametrize("case", ["subm555", "strided335", "subm333"])
+def test_masks_and_sort_for_several_words_bit_exact(case):
+    """cumm_hip_masks_from_pairs and cumm_hip_sort_by_mask_words against their host mirrors."""
+    print("case dynamic masks", case, flush=True)
+    coords, grid = H.small_cloud(66, 6000, grid=(14, 40, 36))
+    host, devt = _tables(case, coords, grid)
+    for table_h, table_d in ((host.indices_fwd, devt.indices_fwd), (host.indices_bwd, devt.indices_bwd)):
+        want = pairs.masks_from_pairs(table_h)
+        got = pairs.masks_from_pairs_device(table_d)
+        np.testing.assert_array_equal(H.host(got), want)
+        ms_ref, order_ref = pairs.sort_by_mask_words(want)
+        ms, order = pairs.sort_by_mask_words_device(got)
+        np.testing.assert_array_equal(H.host(order), order_ref)
+        np.testing.assert_array_equal(H.host(ms), ms_ref)
+
+
+@pytest.mark.parametrize("dtype,tile,c_in,k_out", [("f16", (64, 64), 64, 64), ("bf16", (128, 128), 64, 128),
+                                                    ("f16", (128, 128), 128, 128), ("bf16", (64, 64), 160, 72)])
+@pytest.mark.parametrize("case", ["subm555", "strided335"])
+def test_dynamic_mask_forward_backward_input(dtype, tile, c_in, k_out, case):
+    """Kernel volumes above 32 through implicit_gemm2 in ONE launch: a dynamic_mask descriptor,
+    ceil(kv / 32) mask words per position (masks and order from the GPU preparation, bit-exact
+    above), against the oracle - forward with bias + ReLU and the tile masks it writes,
+    backward-input on the backward masks, and for the submanifold case backward-input on the
+    forward masks reversed in the kernel; the pair table by row and by position."""
+    print("case dynamic mask conv", dtype, tile, c_in, k_out, case, flush=True)
+    from oracle import conv_ref, numerics as onm
+    coords, grid = H.small_cloud(67, 4000, grid=(14, 40, 36))
+    rng = np.random.default_rng(68)
+    host, devt = _tables(case, coords, grid)
+    kv, n_out = host.indices_fwd.shape
+    n_in = coords.shape[0]
+    words = (kv + 31) // 32
+    mf_d = pairs.masks_from_pairs_device(devt.indices_fwd)
+    ms_d, order_d = pairs.sort_by_mask_words_device(mf_d)
+    ms, order = H.host(ms_d), H.host(order_d)
+    feat = H.to_storage(rng.normal(0, 1, size=(n_in, c_in)).astype(np.float32), dtype)
+    w = H.to_storage(rng.normal(0, 0.03, size=(k_out, kv, c_in)).astype(np.float32), dtype)
+    bias = H.to_storage(rng.normal(0, 1, size=(k_out,)).astype(np.float32), dtype)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    out0 = H.to_storage(np.zeros((n_out, k_out), np.float32), dtype)
+    ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, host.indices_fwd, ms, order, tile_m=tile[0], dtype_in=dtype,
+                                                 dtype_w=dtype, dtype_out=dtype, beta=1.0, bias=bias, act=onm.ACT_RELU)
+    tiles = (n_out + tile[0] - 1) // tile[0]
+    outs = []
+    for by_pos in (False, True):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, *tile, dynamic_mask=True)
+        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+        p.bias, p.beta, p.act_type = H.dev(bias, dtype), 1.0, Activation.ReLU
+        p.indices = pairs.pairs_by_position_device(devt.indices_fwd, order_d) if by_pos else devt.indices_fwd
+        p.indices_by_position = by_pos
+        p.mask, p.mask_argsort = ms_d, order_d
+        p.mask_output = tv.zeros([tiles, words], tv.uint32, 0)
+        p.mask_int_count = words
+        ConvMainUnitTest.implicit_gemm2(p)
+        got = H.as_f32(H.host(p.output), dtype)
+        assert got.min() >= 0.0
+        assert H.rel_err(got, H.as_f32(ref, dtype)) < TOL
+        np.testing.assert_array_equal(H.host(p.mask_output), ref_mo)
+        outs.append(H.host(p.output))
+    np.testing.assert_array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+
+    # backward-input on the masks of the backward table
+    mb_d = pairs.masks_from_pairs_device(devt.indices_bwd)
+    msb_d, orderb_d = pairs.sort_by_mask_words_device(mb_d)
+    din0 = H.to_storage(np.zeros((n_in, c_in), np.float32), dtype)
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, din0, host.indices_bwd, H.host(msb_d), H.host(orderb_d), tile_m=tile[0],
+                                             dtype_in=dtype, dtype_w=dtype, dtype_out=dtype)
+    runs = [(msb_d, orderb_d, False)]
+    if case == "subm555":
+        runs.append((ms_d, order_d, True))      # the forward masks, reversed end for end in the kernel
+    for mask_d, ord_d, reverse in runs:
+        pd = ConvParams(3, ConvOpType.BackwardInput)
+        pd.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, *tile, dynamic_mask=True)
+        pd.input, pd.weight, pd.output = H.dev(din0, dtype), H.dev(w, dtype), H.dev(dout, dtype)
+        pd.indices, pd.mask, pd.mask_argsort = devt.indices_bwd, mask_d, ord_d
+        pd.reverse_mask = reverse
+        ConvMainUnitTest.implicit_gemm2(pd)
+        if reverse:
+            ref_r = conv_ref.implicit_gemm_dgrad_ref(dout, w, din0, host.indices_bwd, ms, order, tile_m=tile[0], dtype_in=dtype,
+                                                     dtype_w=dtype, dtype_out=dtype, reverse_mask=True)
+            assert H.rel_err(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_r, dtype)) < TOL
+        assert H.rel_err(H.as_f32(H.host(pd.input), dtype), H.as_f32(ref_d, dtype)) < TOL
+
+
+def test_dynamic_mask_descriptor_with_a_small_kernel_volume():
+    """A dynamic_mask descriptor on a 3 x 3 x 3 kernel has one word per position and gives what
+    the static descriptor gives, bit for bit."""
+    coords, grid = H.small_cloud(69, 3000)
+    rng = np.random.default_rng(70)
+    pt = pairs.subm_pairs(coords, grid)
+    n = coords.shape[0]
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    feat = H.to_storage(rng.normal(0, 1, size=(n, 64)).astype(np.float32), "f16")
+    w = H.to_storage(rng.normal(0, 0.05, size=(64, 27, 64)).astype(np.float32), "f16")
+    outs = []
+    for dyn in (False, True):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp("f16", ConvOpType.Forward, 64, 64, dynamic_mask=dyn)
+        p.input, p.weight, p.output = H.dev(feat, "f16"), H.dev(w, "f16"), tv.zeros([n, 64], tv.float16, 0)
+        p.indices, p.mask, p.mask_argsort = H.dev(pt.indices_fwd, "i32"), H.dev(ms, "u32"), H.dev(order, "i32")
+        ConvMainUnitTest.implicit_gemm2(p)
+        outs.append(H.host(p.output))
+    np.testing.assert_array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
