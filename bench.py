@@ -559,11 +559,22 @@ def bench_s8(args, tile_m):
     p4.bias = dev(rng4.normal(0, 1, size=(128,)).astype(np.float32))
     p4.indices, p4.mask, p4.mask_argsort = dev(pt4.indices_fwd), dev(ms4), dev(as4)
     from cumm_amd import tuner
+    # masks sorted by value and the pair table by output row - the inputs as spconv hands them over -
+    # first; then what this library's input preparation offers on top: positions ordered by offset
+    # count (cumm_hip_sort_by_mask_ordered) and the pair table in that order (indices_by_position)
+    w0_ms, e0_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(p4), args.steps, args.warmup)
+    filt = (1 << 27) - 1
+    by_row = p4.indices
+    p4.mask, p4.mask_argsort = pairs.sort_by_mask_device(dev(pt4.mask_fwd), filt, by_offset_count=True)
+    p4.indices, p4.indices_by_position = pairs.pairs_by_position_device(by_row, p4.mask_argsort), True
     best = tuner.Tuner(steps=10, warmup=2).tune_conv(p4)     # the caller's descriptor choice, by timing
     w_ms, e_ms = timed(lambda: ConvMainUnitTest.implicit_gemm2(p4), args.steps, args.warmup)
     ops4 = 2.0 * P4 * 64 * 128
     bytes4 = n_in4 * 64 + n_out4 * 128 + 27 * 64 * 128 + 27 * n_out4 * 4 + n_out4 * 8 + 2 * 128 * 4
     return {"voxels_in": n_in4, "voxels_out": n_out4, "active_pairs": P4,
+            "inputs": "positions ordered by offset count, pair table by position",
+            "by_value_order_and_row_table": {"tile_m": tile_m, "kernel_ms_events": round(e0_ms, 5),
+                                             "hbm_frac": round(bytes4 / (e0_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
             "tile": list(best.desp.tile_shape[:2]),
             "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
                            for nm, ms in best.tried},
@@ -603,7 +614,10 @@ def main():
     coords, pt, feat, weight = build_subm_f16(rng, 120000, C, K)
     n = coords.shape[0]
     P = int((pt.indices_fwd >= 0).sum())
-    mask_sorted, argsort = pairs.sort_by_mask(pt.mask_fwd)
+    # input preparation orders the positions by offset count, then mask value (the library's own
+    # order; the sort by value that spconv makes is timed beside it below)
+    FILTER = (1 << 27) - 1
+    mask_sorted, argsort = pairs.sort_by_mask(pt.mask_fwd, FILTER, by_offset_count=True)
     tile_m = args.tile_m
 
     p = ConvParams(3, ConvOpType.Forward)
@@ -615,12 +629,14 @@ def main():
     # library's device-side table, where the forward launch finds it: no field beyond the
     # reference's ConvParams is filled in here
     p.indices = dev(pt.indices_fwd)
-    p.mask, p.mask_argsort = pairs.sort_by_mask_device(dev(pt.mask_fwd))
+    d_mask_unsorted = dev(pt.mask_fwd)
+    p.mask, p.mask_argsort = pairs.sort_by_mask_device(d_mask_unsorted, FILTER, by_offset_count=True)
+    p.mask_filter = FILTER
     tiles = (n + tile_m - 1) // tile_m
     p.mask_output = tv.zeros([tiles], tv.uint32, 0)
     p.mask_width = tile_m
     p.beta = 0.0
-    light_found = pairs.light_hint_device(p.mask)      # what the launch will find (reported only)
+    light_found, heavy_found = pairs.hints_device(p.mask, FILTER)      # what the launch will find (reported only)
 
     def step():
         ConvMainUnitTest.implicit_gemm2(p)
@@ -656,7 +672,8 @@ def main():
         "config": {"workload": "SubMConv3d 3x3x3 forward, f16, Cin=Cout=64, mask-based implicit GEMM",
                    "voxels": n, "active_pairs": P, "pairs_per_voxel": round(P / n, 3),
                    "grid_zyx": list(GRID), "clusters": 60, "sigma": 15, "noise_frac": 0.1,
-                   "tile_m": tile_m, "light_prefix_found_on_device": int(light_found), "seed": SEED},
+                   "tile_m": tile_m, "position_order": "offset count, then mask value (cumm_hip_sort_by_mask_ordered)",
+                   "light_prefix_found_on_device": int(light_found), "heavy_end_found_on_device": int(heavy_found), "seed": SEED},
         "pct_mfma_peak": round(100.0 * tflops / PEAK_MFMA_F16_TFLOPS, 3),
         "kernel_ms_events": round(ev_ms, 5),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS,
@@ -680,6 +697,17 @@ def main():
             p.indices, p.indices_by_position = by_row, False
             extra["forward_pair_table_by_position"] = {"ms_per_step": round(w1_ms, 5), "kernel_ms_events": round(e1_ms, 5),
                                                        "hbm_frac": round(alg_bytes / (e1_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+            # the same layer on masks sorted by value, as spconv's sort_1d_by_key leaves them
+            keep = p.mask, p.mask_argsort
+            p.mask, p.mask_argsort = pairs.sort_by_mask_device(d_mask_unsorted, FILTER)
+            w2_ms, e2_ms = timed(step, args.steps, args.warmup)
+            p.light_prefix = -1
+            w3_ms, e3_ms = timed(step, args.steps, args.warmup)
+            p.light_prefix = 0
+            p.mask, p.mask_argsort = keep
+            extra["forward_masks_sorted_by_value"] = {"ms_per_step": round(w2_ms, 5), "kernel_ms_events": round(e2_ms, 5),
+                                                      "hbm_frac": round(alg_bytes / (e2_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                                      "kernel_ms_events_without_hints": round(e3_ms, 5)}
         legs = (set(args.extra_only.split(",")) if args.extra_only
                 else {"dgrad", "wgrad", "s8", "gather_gemm", "dense_gemm", "pairs", "gather", "tuner", "stack", "native"})
         # backward input (reverse mask, backward table) and backward weight (serial split-K)

@@ -103,8 +103,9 @@ SYMBOLS = {
     "cumm_hip_masks_from_pairs": (C.c_int, [_VP, C.c_int, C.c_int, _VP, _VP]),
     "cumm_hip_sort_by_mask_words_workspace": (C.c_size_t, [C.c_int]),
     "cumm_hip_sort_by_mask_words": (C.c_int, [_VP, C.c_int, C.c_int, _VP, _VP, _VP, C.c_size_t, _VP]),
+    "cumm_hip_sort_by_mask_ordered": (C.c_int, [_VP, C.c_int, C.c_uint32, C.c_int, _VP, _VP, _VP, C.c_size_t, _VP]),
     "cumm_hip_pairs_by_position": (C.c_int, [_VP, _VP, C.c_int, C.c_int, _VP, _VP]),
-    "cumm_hip_query_light_hint": (C.c_int, [_VP, C.c_int, C.c_uint32, C.POINTER(C.c_int32), _VP]),
+    "cumm_hip_query_light_hint": (C.c_int, [_VP, C.c_int, C.c_uint32, C.POINTER(C.c_int32), C.POINTER(C.c_int32), _VP]),
     "cumm_hip_light_prefix": (C.c_int, [_VP, C.c_int, C.c_uint32, _VP, _VP]),
     "cumm_hip_conv_pairs_workspace": (C.c_size_t, [C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5),
     "cumm_hip_conv_pairs_sites": (C.c_int, [_VP, C.c_int, C.c_int] + [C.POINTER(C.c_int32)] * 5 +

@@ -1089,7 +1089,14 @@ size_t cumm_hip_sort_by_mask_workspace(int n) { return sort_by_mask_workspace_by
 
 int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
                           int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream) {
-  if (n < 0) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  return cumm_hip_sort_by_mask_ordered(mask, n, mask_filter, 0, sorted_mask, argsort, workspace, workspace_bytes, stream);
+}
+
+int cumm_hip_sort_by_mask_ordered(const uint32_t *mask, int n, uint32_t mask_filter, int order, uint32_t *sorted_mask,
+                                  int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream) {
+  if (n < 0 || order < 0 || order > 1) return fail(CUMM_HIP_EINVAL, "bad arguments");
+  if (order == 1 && (mask_filter >> 27) != 0u)
+    return fail(CUMM_HIP_EINVAL, "the order by offset count takes filters of at most 27 bits (kernel volumes up to 27)");
   if (n == 0) return CUMM_HIP_OK;
   if (n >= (1 << 30)) return fail(CUMM_HIP_EINVAL, "too many positions");
   if (!mask || !sorted_mask || !argsort) return fail(CUMM_HIP_EINVAL, "mask, sorted_mask and argsort must not be empty");
@@ -1100,7 +1107,7 @@ int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uin
   int32_t *status = nullptr;
   if (int rc = async_status_ptr(&status)) return rc;
   hipError_t e = launch_sort_by_mask(mask, n, mask_filter, sorted_mask, argsort, workspace, status + 1,
-                                     light_hint_slot_ptr(sorted_mask), reinterpret_cast<hipStream_t>(stream));
+                                     light_hint_slot_ptr(sorted_mask), order, reinterpret_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "mask sort launch");
   return CUMM_HIP_OK;
 }
@@ -1113,9 +1120,11 @@ int cumm_hip_light_prefix(const uint32_t *sorted_mask, int n, uint32_t mask_filt
   return CUMM_HIP_OK;
 }
 
-int cumm_hip_query_light_hint(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream) {
+int cumm_hip_query_light_hint(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, int32_t *heavy_from,
+                              void *stream) {
   if (!prefix) return fail(CUMM_HIP_EINVAL, "null out-param");
   *prefix = -1;
+  if (heavy_from) *heavy_from = -1;
   if (!sorted_mask || n <= 0) return CUMM_HIP_OK;
   const int32_t *slot = light_hint_slot_ptr(sorted_mask);
   if (!slot) return CUMM_HIP_OK;
@@ -1125,7 +1134,10 @@ int cumm_hip_query_light_hint(const uint32_t *sorted_mask, int n, uint32_t mask_
   HIP_TRY(hipStreamSynchronize(s));
   const uint64_t key = (uint64_t)(uint32_t)words[0] | ((uint64_t)(uint32_t)words[1] << 32);
   if (key == (uint64_t)reinterpret_cast<uintptr_t>(sorted_mask) && words[2] == n && (uint32_t)words[3] == mask_filter)
+  {
     *prefix = words[4];
+    if (heavy_from) *heavy_from = words[5];
+  }
   return CUMM_HIP_OK;
 }
 
@@ -1358,7 +1370,7 @@ int cumm_hip_sort_by_mask_words(const uint32_t *mask, int n, int words, uint32_t
   int32_t *status = nullptr;
   if (int rc = async_status_ptr(&status)) return rc;
   hipError_t e = launch_mask_words_keys(mask, keys, n, words, s);
-  if (e == hipSuccess) e = launch_sort_by_mask(keys, n, 0xFFFFFFFFu, sorted_keys, argsort, base + 2 * part, status + 1, nullptr, s);
+  if (e == hipSuccess) e = launch_sort_by_mask(keys, n, 0xFFFFFFFFu, sorted_keys, argsort, base + 2 * part, status + 1, nullptr, 0, s);
   if (e == hipSuccess) e = launch_mask_words_gather(mask, argsort, sorted_mask, n, words, s);
   if (e != hipSuccess) return hip_fail(e, "mask sort launch");
   return CUMM_HIP_OK;

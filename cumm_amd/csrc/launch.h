@@ -116,7 +116,8 @@ hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t t
 // What input preparation knows about a sorted mask array and a later forward / backward-input
 // launch on the same array can use without being told: a table of kLightHintSlots slots of eight
 // words in device memory, one table per GPU, indexed by a hash of the array's address.  Slot =
-// {address (two words), length, filter, light prefix in positions, 0, 0, 0}.  A hint only: a
+// {address (two words), length, filter, light prefix in positions, first position of the heavy
+// end (the length rounded up to 64 = none), 1 if sorted by offset count, 0}.  A hint only: a
 // launch that finds another array's slot, or a stale one, or none, still computes the same bits.
 constexpr int kLightHintSlots = 256;
 inline int light_hint_slot(const void *sorted_mask) {
@@ -129,8 +130,9 @@ size_t sort_by_mask_workspace_bytes(int n);
 hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, int32_t *hint_slot,
                                hipStream_t s);
 // hint_slot: the slot of `sorted` in the current device's table (NULL = leave no hint)
+// order 0: ascending mask value; 1: ascending number of offsets, then value (filter below 2^27)
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
-                               void *workspace, int32_t *give_ups, int32_t *hint_slot, hipStream_t s);
+                               void *workspace, int32_t *give_ups, int32_t *hint_slot, int order, hipStream_t s);
 
 // per-offset lists of (input row, output row) out of a pair table [kv, n] (pairs_inst.hip)
 struct PairListsParams {

@@ -108,7 +108,8 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
       if constexpr (TM == 64 && TN == 64 && Elem<T>::kBytes == 2 && KS <= 2 && !kWide) {
         if (p.hint_slot != nullptr && grid.y == 1 && p.chunk_shift == 0 && p.mask != nullptr &&
             counted_waits_hold<rowgemm_lds_mixed_kernel<T, KS, WT>>()) {
-          hipLaunchKernelGGL((rowgemm_lds_mixed_kernel<T, KS, WT>), grid, dim3(256), 0, s, p);
+          const dim3 with_spare(grid.x + (unsigned)mixed_spare_tiles((int)grid.x), 1, 1);
+          hipLaunchKernelGGL((rowgemm_lds_mixed_kernel<T, KS, WT>), with_spare, dim3(256), 0, s, p);
           return hipGetLastError();
         }
       }

@@ -65,15 +65,19 @@ struct LdsRing {
 
 // One tile: rows [tile * TM, tile * TM + TM) of the sorted positions, column block col.
 // HALVES: mask_out takes one word per 64 positions (a 128-row tile writes words 2 tile, 2 tile + 1).
+// HALF32 (TM = 32): the tile is one half of a 64-row tile, whose word of mask_out (the OR over
+// all 64 positions, written by the even half) and whose skip rule (left alone only if the whole
+// 64-row tile has no offset) it keeps, so that the launch gives what 64-row tiles give.
 // MW: 32-bit mask words per position.  1 = one word (kernel volumes up to 32).  4 = the layout
 // of the reference's dynamic-mask kernels for larger volumes (MaskIGemmIteratorMaskLoaderDynamic,
 // cumm/gemm/blockmma/mma.py:78-269): p.mask_words = ceil(kv / 32) words per position, word w of
 // position pos at mask[pos * mask_words + w] holding offsets 32 w .. 32 w + 31; mask_out likewise
 // per tile; the filter applies to every word.
-template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT, bool WIDE, bool HALVES, int MW = 1>
+template <class T, int WM, int WN, int RBW, int NBW, int KS, int NS, bool WT, bool WIDE, bool HALVES, int MW = 1, bool HALF32 = false>
 __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const int tile, const int col, const LdsRing &lds) {
   static_assert(MW == 1 || MW == 4, "one mask word, or up to four");
-  static_assert(MW == 1 || !HALVES, "the two tile shapes of one launch take one mask word");
+  static_assert(MW == 1 || (!HALVES && !HALF32), "the tile shapes of a mixed launch take one mask word");
+  static_assert(!HALF32 || (WM * RBW * 16 == 32 && !HALVES), "a half of a 64-row tile has 32 rows");
   using E = Elem<T>;
   using AccV = typename E::AccV;
   constexpr int NW = WM * WN;
@@ -146,6 +150,9 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
 #pragma unroll
     for (int w = 0; w < MW; ++w)
       raw_mk[i][w] = load_b32_hidden(rsw_mask, word_off(i * 64 + lane < TM ? pos_off(pos_base + i * 64 + lane) : kOob, w));
+  // HALF32: the masks of the other half of the 64-row tile (lanes 0 .. 31)
+  int raw_other = 0;
+  if constexpr (HALF32) raw_other = load_b32_hidden(rsw_mask, lane < 32 ? pos_off((pos_base ^ 32) + lane) : kOob);
   raw_key_row = load_b32_hidden(rsw_rows, pos_off(key_pos));
 #pragma unroll
   for (int w = 0; w < MW; ++w) raw_key_bits[w] = load_b32_hidden(rsw_mask, word_off(pos_off(key_pos), w));
@@ -187,6 +194,7 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
   for (int i = 0; i < MKW; ++i)
 #pragma unroll
     for (int w = 0; w < MW; ++w) keep_after_wait(raw_mk[i][w]);
+  if constexpr (HALF32) keep_after_wait(raw_other);
   keep_after_wait(raw_key_row);
 #pragma unroll
   for (int w = 0; w < MW; ++w) keep_after_wait(raw_key_bits[w]);
@@ -313,10 +321,14 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
         if (2 * tile < p.n_mask_out) p.mask_out[2 * tile] = lo;
         if ((2 * tile + 1) * 64 < p.n_pos && 2 * tile + 1 < p.n_mask_out) p.mask_out[2 * tile + 1] = hi;
       }
+    } else if constexpr (HALF32) {
+      const uint32_t whole = kmask | (wave_or_dpp((uint32_t)raw_other) & p.mask_filter);
+      if (p.mask_out != nullptr && tid == 0 && col == 0 && (tile & 1) == 0 && (tile >> 1) < p.n_mask_out) p.mask_out[tile >> 1] = whole;
+      if (p.exit_on_empty && whole == 0) return;
     } else {
       if (p.mask_out != nullptr && tid == 0 && col == 0 && tile < p.n_mask_out) p.mask_out[tile] = kmask;
     }
-    if (p.exit_on_empty && kmask == 0) return;
+    if (!HALF32 && p.exit_on_empty && kmask == 0) return;
     if (p.reverse_mask) kmask = __builtin_bitreverse32(kmask) >> (32 - p.kv);
     if (p.kv < 32) kmask &= (1u << p.kv) - 1u;
   }
@@ -781,6 +793,9 @@ __global__ __launch_bounds__(WM *WN * 64) void rowgemm_lds_kernel(const RowGemmP
 // many-offset tile in the 128-row part only runs slower (two stages).  Workgroups are dispatched
 // in the order of their number: the 64-row tiles first, heaviest first, then the pairs; the
 // numbers left over leave at once, last of all.
+// workgroups a mixed launch has beyond one per 64-row tile: for the halves of the heavy end
+__host__ __device__ constexpr int mixed_spare_tiles(int tiles) { return tiles / 8; }
+
 template <class T, int KS, bool WT>
 __global__ __launch_bounds__(256) void rowgemm_lds_mixed_kernel(const RowGemmParams p) {
   constexpr int R64 = 64 * 4 * KS;        // 16-byte vectors of 64 rows
@@ -797,20 +812,37 @@ __global__ __launch_bounds__(256) void rowgemm_lds_mixed_kernel(const RowGemmPar
   typedef int v8i __attribute__((ext_vector_type(8)));
   const v8i slot = *reinterpret_cast<const v8i *>(p.hint_slot);
   const uint64_t mask_addr = (uint64_t)p.mask;
+  // (the two filters have to agree on the bits a mask can have: those of the kernel volume)
+  const uint32_t live_bits = p.kv < 32 ? (1u << p.kv) - 1u : ~0u;
   const bool named = (slot[0] == (int)(uint32_t)mask_addr) & (slot[1] == (int)(uint32_t)(mask_addr >> 32)) &
-                     (slot[2] == p.n_pos) & (slot[3] == (int)p.mask_filter) & (slot[4] > 0);
+                     (slot[2] == p.n_pos) & ((((uint32_t)slot[3] ^ p.mask_filter) & live_bits) == 0u);
   // (a count from the caller comes with a slot that names nothing: one of the two is zero, and the
   // OR keeps the slot's load out of a branch, where it would wait for the pointer first)
-  const int hinted = p.pair_tiles | (named ? slot[4] >> 7 : 0);
+  const int hinted = p.pair_tiles | (named & (slot[4] > 0) ? slot[4] >> 7 : 0);
   const int pairs = hinted < (tiles >> 1) ? hinted : (tiles >> 1);
-  const int singles = tiles - 2 * pairs;
+  // The heavy end: the 64-row tiles from slot word 5 on are taken as two halves of 32 rows each,
+  // which halves the life of the launch's longest tiles - when they are few (an eighth of the
+  // tiles at most: the grid has that many workgroups to spare) and lie behind the pairs.
+  // (rows of 64 bytes: a 32-row stage is less than one load instruction per wave - no halves)
+  const int heavy_tile = named && KS == 2 ? slot[5] >> 6 : tiles;
+  const int heavy = heavy_tile >= 2 * pairs && heavy_tile < tiles && tiles - heavy_tile <= mixed_spare_tiles(tiles) ? tiles - heavy_tile : 0;
+  const int halves = 2 * heavy;
+  const int singles = tiles - 2 * pairs - heavy;
   const int rank = (int)blockIdx.x;
-  if (rank < singles) {
+  // dispatch order: the halves of the heavy end (last positions first), the 64-row tiles, heaviest
+  // first, then the pairs; the workgroup numbers left over leave at once, last of all
+  if (rank < halves) {
+    if constexpr (KS == 2) {
+      constexpr int R32 = 32 * 4 * KS;      // 16-byte vectors of 32 rows
+      const LdsRing lds = {{st0, st1, st2, nullptr}, {st0 + R32, st1 + R32, st2 + R32, nullptr}, {ix0, ix1, ix2, nullptr}};
+      rowgemm_lds_tile<T, 2, 2, 1, 2, KS, 3, WT, false, false, 1, true>(p, 2 * tiles - 1 - rank, 0, lds);
+    }
+  } else if (rank - halves < singles) {
     const LdsRing lds = {{st0, st1, st2, nullptr}, {st0 + R64, st1 + R64, st2 + R64, nullptr}, {ix0, ix1, ix2, nullptr}};
-    rowgemm_lds_tile<T, 2, 2, 2, 2, KS, 3, WT, false, false>(p, tiles - 1 - rank, 0, lds);
-  } else if (rank - singles < pairs) {
+    rowgemm_lds_tile<T, 2, 2, 2, 2, KS, 3, WT, false, false>(p, tiles - heavy - 1 - (rank - halves), 0, lds);
+  } else if (rank - halves - singles < pairs) {
     const LdsRing lds = {{st0, st1, nullptr, nullptr}, {st2, st2 + R64, nullptr, nullptr}, {ix0, ix1, nullptr, nullptr}};
-    rowgemm_lds_tile<T, 2, 2, 4, 2, KS, 2, WT, false, true>(p, pairs - 1 - (rank - singles), 0, lds);
+    rowgemm_lds_tile<T, 2, 2, 4, 2, KS, 2, WT, false, true>(p, pairs - 1 - (rank - halves - singles), 0, lds);
   }
 }
 

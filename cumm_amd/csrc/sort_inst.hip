@@ -54,7 +54,23 @@ struct SortParams {
   uint32_t *out_keys, *tmp_keys;   // the caller's arrays and the workspace's: the passes alternate between them
   int32_t *out_vals, *tmp_vals;
   int32_t *hint_slot;        // light-prefix hint of the sorted array (launch.h), or NULL
+  // 0: ascending mask value (spconv's sort_1d_by_key).  1: ascending number of kernel offsets, then
+  // ascending value (the filter has at most kCountShift significant bits): positions of few
+  // offsets first, the few of many offsets last - tiles of the heavy end then OR together masks
+  // of similar weight, and the many-offset tiles of a launch form a short run at its end.
+  int32_t count_major;
 };
+
+constexpr int kCountShift = 27;
+// sort key of a mask word
+__device__ __forceinline__ uint32_t sort_key(const SortParams &p, uint32_t mask_word) {
+  const uint32_t m = mask_word & p.filter;
+  return p.count_major ? ((uint32_t)__builtin_popcount(m) << kCountShift) | m : m;
+}
+// ... and the mask word back out of it
+__device__ __forceinline__ uint32_t key_mask(const SortParams &p, uint32_t key) {
+  return p.count_major ? key & ((1u << kCountShift) - 1u) : key;
+}
 
 __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortParams p) {
   __shared__ uint32_t lds_hist[4][kBins];
@@ -64,7 +80,8 @@ __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortPara
   const size_t words = (size_t)p.passes * p.chunks * kBins;
   for (size_t i = (size_t)blockIdx.x * kSortThreads + t; i < words; i += (size_t)gridDim.x * kSortThreads) p.state[i] = 0u;
   if (blockIdx.x == 0 && t < p.passes) p.tickets[t] = 0u;
-  if (blockIdx.x == 0 && t < 8 && p.hint_slot != nullptr) p.hint_slot[t] = t == 4 ? (p.n / 128) * 128 : 0;   // names no array yet
+  if (blockIdx.x == 0 && t < 8 && p.hint_slot != nullptr)   // names no array yet; the two counts start at "everything" / "nothing"
+    p.hint_slot[t] = t == 4 ? (p.n / 128) * 128 : (t == 5 ? ((p.n + 63) / 64) * 64 : 0);
   __syncthreads();
   // lanes of a wave with the same digit add once (most masks of a sparse cloud are the same word:
   // one add per lane would queue 64 deep on one LDS address)
@@ -79,7 +96,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_setup_kernel(const SortPara
     for (int u = 0; u < kItems; ++u) {
       const int64_t i = (r0 + u) * span + (int64_t)blockIdx.x * kSortThreads + t;
       valids[u] = r0 + u < rounds && i < p.n;
-      keys[u] = valids[u] ? (p.mask[i] & p.filter) : 0u;
+      keys[u] = valids[u] ? sort_key(p, p.mask[i]) : 0u;
     }
 #pragma unroll
     for (int u = 0; u < kItems; ++u) {
@@ -148,6 +165,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
   // the last mover writes the caller's arrays, the ones before it alternate; the first one
   // reads the caller's masks (and the identity order)
   const bool first = movers_before == 0;
+  const bool last = movers - 1 - movers_before == 0;
   const bool to_out = copy_through || ((movers - 1 - movers_before) & 1) == 0;
   uint32_t *const dst_keys = to_out ? p.out_keys : p.tmp_keys;
   int32_t *const dst_vals = to_out ? p.out_vals : p.tmp_vals;
@@ -181,7 +199,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
     for (int u = 0; u < kItems; ++u) {
       const int64_t pos = (int64_t)chunk * kChunk + u * kSortThreads + t;
       if (pos < p.n) {
-        dst_keys[pos] = p.mask[pos] & p.filter;
+        dst_keys[pos] = p.mask[pos] & p.filter;      // (nothing moves: the masks themselves)
         dst_vals[pos] = (int32_t)pos;
       }
     }
@@ -199,7 +217,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
     const int64_t pos = base_w + u * 64 + lane;
     const bool valid = pos < p.n;
     if (first) {
-      key[u] = valid ? (p.mask[pos] & p.filter) : 0u;
+      key[u] = valid ? sort_key(p, p.mask[pos]) : 0u;
       val[u] = (int32_t)pos;
     } else {
       key[u] = valid ? src_keys[pos] : 0u;
@@ -291,25 +309,32 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
     if (pos < p.n) {
       const uint32_t d = (key[u] >> shift) & (kBins - 1);
       const uint32_t dst = bin_base[d] + wave_hist[wave][d] + rank[u];
-      dst_keys[dst] = key[u];
+      dst_keys[dst] = last ? key_mask(p, key[u]) : key[u];     // the caller gets masks, not keys
       dst_vals[dst] = val[u];
     }
   }
 }
 
-// How far the light end of a sorted mask array reaches: the number of leading runs of 128
-// positions whose two halves of 64 each have at most kLightOffsets kernel offsets in the OR of
-// their masks, as a number of positions.  One wave per run; a run that fails lowers the result
-// (which starts at the positions of all whole runs) to where it begins.
-constexpr int kLightOffsets = 2;
+// What a later launch can use about a sorted mask array, counted here into its hint slot:
+//   * the light prefix (slot word 4): the number of leading runs of 128 positions whose two halves
+//     of 64 each have at most `light` kernel offsets in the OR of their masks, as a number of
+//     positions - those go to 128-row tiles.  `light` is 2 for the order by value; in the order by
+//     offset count the runs of equal two-offset masks follow one another, and the tile at each
+//     seam has three: 3 there.
+//   * where the heavy end begins (slot word 5): the first tile of 64 positions with kHeavyOffsets or
+//     more kernel offsets, as a position - a launch may take the tiles from there on in halves of
+//     32 rows when they are few (in the order by offset count they are the last few tiles).
+// One wave per run of 128; a run that fails lowers a count that starts at "all" / "none".
+constexpr int kLightOffsets = 2, kLightOffsetsByCount = 3, kHeavyOffsets = 10;
 
-__global__ __launch_bounds__(64) void light_prefix_init_kernel(int32_t *result, int32_t *hint_slot, int runs) {
-  if (threadIdx.x == 0 && result != nullptr) *result = runs * 128;
-  if (threadIdx.x < 8 && hint_slot != nullptr) hint_slot[threadIdx.x] = threadIdx.x == 4 ? runs * 128 : 0;
+__global__ __launch_bounds__(64) void light_prefix_init_kernel(int32_t *result, int32_t *hint_slot, int n) {
+  if (threadIdx.x == 0 && result != nullptr) *result = (n / 128) * 128;
+  if (threadIdx.x < 8 && hint_slot != nullptr)
+    hint_slot[threadIdx.x] = threadIdx.x == 4 ? (n / 128) * 128 : (threadIdx.x == 5 ? ((n + 63) / 64) * 64 : 0);
 }
 
-// Names the array a hint slot describes (the prefix word has been counted down by then or is
-// being counted down by the same kernel: a launch that reads the slot comes later on the stream).
+// Names the array a hint slot describes (the counts have been lowered by then or are being lowered
+// by the same kernel: a launch that reads the slot comes later on the stream).
 __device__ __forceinline__ void name_hint_slot(int32_t *slot, const uint32_t *sorted, int n, uint32_t filter) {
   const uint64_t a = (uint64_t)sorted;
   slot[0] = (int32_t)(uint32_t)a;
@@ -318,21 +343,32 @@ __device__ __forceinline__ void name_hint_slot(int32_t *slot, const uint32_t *so
   slot[3] = (int32_t)filter;
 }
 
-__global__ __launch_bounds__(256) void light_prefix_kernel(const uint32_t *sorted, int n, int runs, uint32_t filter,
+// one wave, one run of 128 positions (the last run may be short: it only counts for the heavy end)
+__device__ __forceinline__ void count_run(const uint32_t *sorted, int n, uint32_t filter, int run, int lane, int light,
+                                          int32_t *result, int32_t *hint_slot) {
+  const int64_t p0 = (int64_t)run * 128 + lane, p1 = p0 + 64;
+  const uint32_t lo = wave_or_dpp(p0 < n ? sorted[p0] & filter : 0u);
+  const uint32_t hi = wave_or_dpp(p1 < n ? sorted[p1] & filter : 0u);
+  if (lane != 0) return;
+  const int c0 = __builtin_popcount(lo), c1 = __builtin_popcount(hi);
+  if (run < n / 128 && (c0 > light || c1 > light)) {
+    if (result != nullptr) atomicMin(result, run * 128);
+    if (hint_slot != nullptr) atomicMin(&hint_slot[4], run * 128);
+  }
+  if (hint_slot != nullptr && (c0 >= kHeavyOffsets || c1 >= kHeavyOffsets))
+    atomicMin(&hint_slot[5], run * 128 + (c0 >= kHeavyOffsets ? 0 : 64));
+}
+
+__global__ __launch_bounds__(256) void light_prefix_kernel(const uint32_t *sorted, int n, uint32_t filter,
                                                            int32_t *result, int32_t *hint_slot) {
   const int lane = threadIdx.x & 63;
   const int run = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (blockIdx.x == 0 && threadIdx.x == 0 && hint_slot != nullptr) name_hint_slot(hint_slot, sorted, n, filter);
-  if (run >= runs) return;
-  const uint32_t lo = wave_or_dpp(sorted[(size_t)run * 128 + lane] & filter);
-  const uint32_t hi = wave_or_dpp(sorted[(size_t)run * 128 + 64 + lane] & filter);
-  if (lane == 0 && (__builtin_popcount(lo) > kLightOffsets || __builtin_popcount(hi) > kLightOffsets)) {
-    if (result != nullptr) atomicMin(result, run * 128);
-    if (hint_slot != nullptr) atomicMin(&hint_slot[4], run * 128);
-  }
+  if ((int64_t)run * 128 >= n) return;
+  count_run(sorted, n, filter, run, lane, kLightOffsets, result, hint_slot);
 }
 
-// Behind the last pass of the sort: the light prefix of the result into the hint slot - or, when a
+// Behind the last pass of the sort: the counts of the result into the hint slot - or, when a
 // look-back of this device has given up since the host last looked, the identity order in place
 // of a result that cannot be trusted.  One wave per 128 positions, the last run may be short.
 __global__ __launch_bounds__(256) void sort_finish_kernel(const SortParams p) {
@@ -352,12 +388,12 @@ __global__ __launch_bounds__(256) void sort_finish_kernel(const SortParams p) {
     return;
   }
   if (p.hint_slot == nullptr) return;
-  if (blockIdx.x == 0 && threadIdx.x == 0) name_hint_slot(p.hint_slot, p.out_keys, p.n, p.filter);
-  if (run >= p.n / 128) return;
-  const uint32_t lo = wave_or_dpp(p.out_keys[(size_t)run * 128 + lane]);
-  const uint32_t hi = wave_or_dpp(p.out_keys[(size_t)run * 128 + 64 + lane]);
-  if (lane == 0 && (__builtin_popcount(lo) > kLightOffsets || __builtin_popcount(hi) > kLightOffsets))
-    atomicMin(&p.hint_slot[4], run * 128);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    name_hint_slot(p.hint_slot, p.out_keys, p.n, p.filter);
+    p.hint_slot[6] = p.count_major;
+  }
+  if ((int64_t)run * 128 >= p.n) return;
+  count_run(p.out_keys, p.n, 0xFFFFFFFFu, run, lane, p.count_major ? kLightOffsetsByCount : kLightOffsets, nullptr, p.hint_slot);
 }
 
 size_t align256s(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -378,14 +414,16 @@ size_t sort_by_mask_workspace_bytes(int n) {
 }
 
 hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uint32_t *sorted, int32_t *argsort,
-                               void *workspace, int32_t *give_ups, int32_t *hint_slot, hipStream_t s) {
+                               void *workspace, int32_t *give_ups, int32_t *hint_slot, int order, hipStream_t s) {
   if (n <= 0) return hipSuccess;
+  if (order != 0 && (filter >> kCountShift) != 0u) return hipErrorInvalidValue;   // no room for the count above the mask
   char *base = reinterpret_cast<char *>(workspace);
   const size_t words = align256s(4 * (size_t)n);
   SortParams p;
   p.mask = mask; p.filter = filter; p.n = n;
   p.chunks = (n + kChunk - 1) / kChunk;
-  p.passes = sort_passes(filter);
+  p.count_major = order != 0;
+  p.passes = p.count_major ? 4 : sort_passes(filter);
   p.out_keys = sorted; p.out_vals = argsort;
   p.tmp_keys = reinterpret_cast<uint32_t *>(base);
   p.tmp_vals = reinterpret_cast<int32_t *>(base + words);
@@ -409,9 +447,9 @@ hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uin
 
 hipError_t launch_light_prefix(const uint32_t *sorted, int n, uint32_t filter, int32_t *result, int32_t *hint_slot,
                                hipStream_t s) {
-  const int runs = n / 128;
-  hipLaunchKernelGGL(light_prefix_init_kernel, dim3(1), dim3(64), 0, s, result, hint_slot, runs);
-  hipLaunchKernelGGL(light_prefix_kernel, dim3(runs > 0 ? (runs + 3) / 4 : 1), dim3(256), 0, s, sorted, n, runs, filter, result,
+  const int runs = (n + 127) / 128;
+  hipLaunchKernelGGL(light_prefix_init_kernel, dim3(1), dim3(64), 0, s, result, hint_slot, n);
+  hipLaunchKernelGGL(light_prefix_kernel, dim3(runs > 0 ? (runs + 3) / 4 : 1), dim3(256), 0, s, sorted, n, filter, result,
                      hint_slot);
   return hipGetLastError();
 }

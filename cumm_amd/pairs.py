@@ -136,19 +136,30 @@ def sparse_conv_pairs(coords: np.ndarray, spatial_shape: Sequence[int], ksize=(3
     return PairTable(ind_f, ind_b, _masks(ind_f), _masks(ind_b), out_coords, out_shape)
 
 
-def sort_by_mask(mask: np.ndarray, mask_filter: int = 0xFFFFFFFF):
+def sort_by_mask(mask: np.ndarray, mask_filter: int = 0xFFFFFFFF, by_offset_count: bool = False):
     """(sorted mask, argsort): stable ascending sort of ``mask & mask_filter``
     (spconv's sort_1d_by_key[_split]; the kernel reads the mask by sorted position
     and the pair table by real row, cumm/conv/kernel.py:853-855,
-    cumm/conv/sparse_iters.py:349-352 of the reference)."""
+    cumm/conv/sparse_iters.py:349-352 of the reference).  ``by_offset_count``: ascending number
+    of kernel offsets first, then value (filters of at most 27 bits) - an order of this build's
+    own that keeps the many-offset positions in a short run at the end."""
     key = mask & np.uint32(mask_filter)
-    order = np.argsort(key, kind="stable").astype(np.int32)
+    if by_offset_count:
+        if int(mask_filter) >> 27:
+            raise ValueError("the order by offset count takes filters of at most 27 bits")
+        count = np.zeros(key.shape, np.uint32)
+        for b in range(27):
+            count += (key >> np.uint32(b)) & np.uint32(1)
+        order = np.argsort((count << np.uint32(27)) | key, kind="stable").astype(np.int32)
+    else:
+        order = np.argsort(key, kind="stable").astype(np.int32)
     return np.ascontiguousarray(key[order]), order
 
 
-def light_prefix(sorted_mask: np.ndarray, mask_filter: int = 0xFFFFFFFF) -> int:
+def light_prefix(sorted_mask: np.ndarray, mask_filter: int = 0xFFFFFFFF, light_offsets: int = 2) -> int:
     """How far the light end of a sorted mask array reaches: the number of leading positions (a
-    multiple of 128) in runs of 128 whose two halves of 64 each OR to at most two kernel offsets.
+    multiple of 128) in runs of 128 whose two halves of 64 each OR to at most ``light_offsets``
+    kernel offsets (two; the GPU sort counts with three for its order by offset count).
     The value of ``ConvParams.light_prefix`` (a submanifold layer's centre-only positions lead the
     ascending order); the reference has no such hint."""
     key = np.asarray(sorted_mask, np.uint32) & np.uint32(mask_filter)
@@ -159,8 +170,25 @@ def light_prefix(sorted_mask: np.ndarray, mask_filter: int = 0xFFFFFFFF) -> int:
     bits = np.zeros(runs * 2, np.int64)
     for b in range(32):
         bits += (words >> np.uint32(b)) & np.uint32(1)
-    heavy = np.nonzero(bits.reshape(runs, 2).max(axis=1) > 2)[0]
+    heavy = np.nonzero(bits.reshape(runs, 2).max(axis=1) > light_offsets)[0]
     return int(heavy[0] if heavy.size else runs) * 128
+
+
+def heavy_from(sorted_mask: np.ndarray, mask_filter: int = 0xFFFFFFFF, heavy_offsets: int = 10) -> int:
+    """Where the heavy end of a sorted mask array begins: the first position of the first tile of 64
+    positions whose masks OR to ``heavy_offsets`` or more kernel offsets; the length rounded up
+    to 64 when there is none.  What the GPU sort leaves next to the light prefix."""
+    key = np.asarray(sorted_mask, np.uint32) & np.uint32(mask_filter)
+    n = key.shape[0]
+    tiles = (n + 63) // 64
+    pad = np.zeros(tiles * 64, np.uint32)
+    pad[:n] = key
+    words = np.bitwise_or.reduce(pad.reshape(tiles, 64), axis=1)
+    bits = np.zeros(tiles, np.int64)
+    for b in range(32):
+        bits += (words >> np.uint32(b)) & np.uint32(1)
+    heavy = np.nonzero(bits >= heavy_offsets)[0]
+    return int(heavy[0] if heavy.size else tiles) * 64
 
 
 def masks_from_pairs(indices: np.ndarray) -> np.ndarray:
@@ -331,11 +359,13 @@ def sparse_conv_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 
     return DeviceConvPairTable(ind_f, ind_b, mask_f, mask_b, out_coords, tuple(int(v) for v in out_shape))
 
 
-def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, stream: int = 0, out=None):
+def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, stream: int = 0, out=None,
+                        by_offset_count: bool = False):
     """GPU counterpart of :func:`sort_by_mask` on a device ``tv.Tensor`` [N] uint32: returns
     (sorted mask, argsort) device tensors (spconv's sort_1d_by_key[_split], call site
     cumm/conv/main_real_spconv.py:118-145 of the reference).  With ``workspace`` and ``out`` =
-    (sorted mask, argsort) tensors of a previous call the call allocates nothing."""
+    (sorted mask, argsort) tensors of a previous call the call allocates nothing.
+    ``by_offset_count``: the order of :func:`sort_by_mask` with the same switch."""
     from . import _capi
     from . import tensorview as tv
     if mask.device < 0 or mask.dtype != tv.uint32 or mask.ndim != 1:
@@ -352,9 +382,10 @@ def sort_by_mask_device(mask, mask_filter: int = 0xFFFFFFFF, workspace=None, str
     else:
         out_mask = tv.empty([n], tv.uint32, 0)
         order = tv.empty([n], tv.int32, 0)
-    _capi.check(lib.cumm_hip_sort_by_mask(mask.byte_pointer(), n, int(mask_filter) & 0xFFFFFFFF,
-                                          out_mask.byte_pointer(), order.byte_pointer(),
-                                          workspace.byte_pointer(), workspace.nbytes, stream))
+    _capi.check(lib.cumm_hip_sort_by_mask_ordered(mask.byte_pointer(), n, int(mask_filter) & 0xFFFFFFFF,
+                                                  1 if by_offset_count else 0,
+                                                  out_mask.byte_pointer(), order.byte_pointer(),
+                                                  workspace.byte_pointer(), workspace.nbytes, stream))
     return out_mask, order
 
 
@@ -377,12 +408,19 @@ def light_hint_device(sorted_mask, mask_filter: int = 0xFFFFFFFF, stream: int = 
     """The light prefix that the library's device-side table holds for this sorted mask tensor
     (left there by :func:`sort_by_mask_device` or :func:`light_prefix_device`), -1 if none: what a
     forward / backward-input launch with ``light_prefix == 0`` on this tensor will use."""
+    return hints_device(sorted_mask, mask_filter, stream)[0]
+
+
+def hints_device(sorted_mask, mask_filter: int = 0xFFFFFFFF, stream: int = 0):
+    """(light prefix, first position of the heavy end) as the library's device-side table holds
+    them for this sorted mask tensor; (-1, -1) if it holds nothing for it."""
     import ctypes
     from . import _capi
-    out = ctypes.c_int32(-1)
+    out, heavy = ctypes.c_int32(-1), ctypes.c_int32(-1)
     _capi.check(_capi.lib().cumm_hip_query_light_hint(sorted_mask.byte_pointer(), int(sorted_mask.shape[0]),
-                                                      int(mask_filter) & 0xFFFFFFFF, ctypes.byref(out), stream))
-    return int(out.value)
+                                                      int(mask_filter) & 0xFFFFFFFF, ctypes.byref(out), ctypes.byref(heavy),
+                                                      stream))
+    return int(out.value), int(heavy.value)
 
 
 def masks_from_pairs_device(indices, stream: int = 0):

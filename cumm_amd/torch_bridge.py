@@ -157,11 +157,16 @@ class SparseConvGeometry:
         # (a mask has one bit per kernel offset: a filter of that width spares the sort the passes over
         # the bits above it)
         bits = (1 << self.kv) - 1 if self.kv < 32 else 0xFFFFFFFF
-        self.mask_fwd, self.order_fwd = pairs.sort_by_mask_device(t.mask_fwd, mask_filter=bits, stream=stream)
+        # (the library's order by offset count where the masks leave room for the count: same rows,
+        # lighter tiles, and the few many-offset tiles in a short run at the end)
+        by_count = self.kv <= 27
+        self.mask_fwd, self.order_fwd = pairs.sort_by_mask_device(t.mask_fwd, mask_filter=bits, stream=stream,
+                                                                  by_offset_count=by_count)
         if self.subm:      # the forward masks serve the backward-input pass, bit-reversed in the kernel
             self.mask_bwd, self.order_bwd = self.mask_fwd, self.order_fwd
         else:
-            self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, mask_filter=bits, stream=stream)
+            self.mask_bwd, self.order_bwd = pairs.sort_by_mask_device(t.mask_bwd, mask_filter=bits, stream=stream,
+                                                                      by_offset_count=by_count)
         # (how far the light end of each sorted order reaches - the hint of the forward and
         # backward-input launches - stays on the device: the sort leaves it in the library's table
         # under the sorted array's address and the launches look it up there; 0 = not given here)

@@ -281,11 +281,23 @@ int cumm_hip_subm_pairs(const int32_t *coords, int n, const int32_t *spatial_sha
 size_t cumm_hip_sort_by_mask_workspace(int n);
 int cumm_hip_sort_by_mask(const uint32_t *mask, int n, uint32_t mask_filter, uint32_t *sorted_mask,
                           int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream);
+/* The same with a choice of order.  order 0: ascending mask value, what cumm_hip_sort_by_mask and
+ * spconv's sort_1d_by_key give.  order 1: ascending number of kernel offsets (set bits of mask &
+ * mask_filter), then ascending value; mask_filter must fit 27 bits.  Any order with its masks is valid
+ * input of the convolutions (the results are the same rows); this one puts the few positions with many
+ * offsets - the rows whose tiles decide how long a launch runs - into a short run at the end, which the
+ * forward / backward-input launches then take in half-size tiles (the sort leaves that position in the
+ * library's table next to the light prefix), and makes the tiles of the heavy end OR together masks of
+ * similar weight (fewer kernel offsets per tile).  No counterpart in the reference. */
+int cumm_hip_sort_by_mask_ordered(const uint32_t *mask, int n, uint32_t mask_filter, int order, uint32_t *sorted_mask,
+                                  int32_t *argsort, void *workspace, size_t workspace_bytes, void *stream);
 int cumm_hip_light_prefix(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream);
 /* What the library's table holds for this array, length and filter: *prefix (host) = the light prefix a
- * launch on it would find, or -1 if the table has nothing for it.  Waits for the stream.  For tests
- * and diagnostics; no launch needs it. */
-int cumm_hip_query_light_hint(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, void *stream);
+ * launch on it would find, *heavy_from (host, may be NULL) = the first position of its heavy end (the first
+ * tile of 64 positions whose masks OR to ten or more kernel offsets; n rounded up to 64 = none); -1 each if
+ * the table has nothing for the array.  Waits for the stream.  For tests and diagnostics; no launch needs it. */
+int cumm_hip_query_light_hint(const uint32_t *sorted_mask, int n, uint32_t mask_filter, int32_t *prefix, int32_t *heavy_from,
+                              void *stream);
 
 /* Pair tables of a regular (strided) sparse convolution, in two calls like spconv's
  * generate_conv_inds_mask_stage1 / stage2 (the reference's callers take them from there; its own

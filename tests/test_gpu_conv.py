@@ -862,3 +862,67 @@ def test_pair_table_by_position(dtype, tile, c_in, k_out, strided):
                                              reverse_mask=reverse)
     assert H.rel_err(H.as_f32(base, dtype), H.as_f32(ref_d, dtype)) < TOL
     np.testing.assert_array_equal(backward_input(True).view(np.uint16), base.view(np.uint16))
+
+
+@pytest.mark.parametrize("dtype,c_in,k_out", [("f16", 64, 64), ("bf16", 48, 40), ("f16", 32, 32)])
+@pytest.mark.parametrize("n_target", [12000, 2100])
+def test_order_by_offset_count_and_half_tiles(dtype, c_in, k_out, n_target):
+    """The launch that finds its hints on the device, on masks in the GPU sort's order by offset
+    count: the light end in 128-row tiles, the heavy end - the last few tiles, ten offsets or more -
+    in halves of 32 rows (contractions of more than 64 bytes).  Forward (bias + ReLU) and
+    backward-input give the same output bits as 64-row tiles throughout (light_prefix = -1: no
+    hints) and as the same layer on masks sorted by value, the tile masks are the oracle's, and the
+    results are within tolerance of the oracle."""
+    print("case order by count", dtype, c_in, k_out, n_target, flush=True)
+    rng = np.random.default_rng(21)
+    grid = (41, 400, 400)
+    coords = synth.clustered_voxels(rng, n_target, grid, 6, sigma=15.0, noise_frac=0.1)
+    pt = pairs.subm_pairs(coords, grid)
+    n = coords.shape[0]
+    filt = 0x07FFFFFF
+    d_mask = H.dev(pt.mask_fwd, "u32")
+    feat = H.to_storage(rng.normal(0, 1, size=(n, c_in)).astype(np.float32), dtype)
+    w = H.to_storage(rng.normal(0, 0.05, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    bias = H.to_storage(rng.normal(0, 1, size=(k_out,)).astype(np.float32), dtype)
+    dout = H.to_storage(rng.normal(0, 1, size=(n, k_out)).astype(np.float32), dtype)
+    out0 = H.to_storage(np.zeros((n, k_out), np.float32), dtype)
+    din0 = H.to_storage(np.full((n, c_in), 3.0, np.float32), dtype)
+    d_feat, d_w, d_bias, d_dout = H.dev(feat, dtype), H.dev(w, dtype), H.dev(bias, dtype), H.dev(dout, dtype)
+    d_ind, d_indb = H.dev(pt.indices_fwd, "i32"), H.dev(pt.indices_bwd, "i32")
+    tiles = (n + 63) // 64
+    results = {}
+    for by_count in (False, True):
+        ms, order = pairs.sort_by_mask_device(d_mask, filt, by_offset_count=by_count)
+        ms_h, order_h = H.host(ms), H.host(order)
+        light, heavy = pairs.hints_device(ms, filt)
+        if by_count and n_target == 12000:
+            assert light >= 256 and heavy < n and (tiles - heavy // 64) * 8 <= tiles, "the case should have pairs and halves"
+        for hint in (-1, 0):
+            p = ConvParams(3, ConvOpType.Forward)
+            p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, 64, 64)
+            p.input, p.weight, p.output, p.bias = d_feat, d_w, H.dev(out0, dtype), d_bias
+            p.beta, p.act_type = 1.0, Activation.ReLU
+            p.indices, p.mask, p.mask_argsort, p.mask_filter = d_ind, ms, order, filt
+            p.mask_output = tv.zeros([tiles], tv.uint32, 0)
+            p.light_prefix = hint
+            ConvMainUnitTest.implicit_gemm2(p)
+            pd = ConvParams(3, ConvOpType.BackwardInput)
+            pd.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardInput, 64, 64)
+            pd.input, pd.weight, pd.output = H.dev(din0, dtype), d_w, d_dout
+            pd.indices, pd.mask, pd.mask_argsort, pd.mask_filter, pd.reverse_mask = d_indb, ms, order, filt, True
+            pd.light_prefix = hint
+            ConvMainUnitTest.implicit_gemm2(pd)
+            results[(by_count, hint)] = (H.host(p.output), H.host(pd.input))
+            np.testing.assert_array_equal(H.host(p.mask_output), conv_ref.tile_masks(ms_h, 64, filt))
+        if by_count:
+            ref, _ = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms_h, order_h, tile_m=64, dtype_in=dtype,
+                                                    dtype_w=dtype, dtype_out=dtype, mask_filter=filt, beta=1.0, bias=bias,
+                                                    act=onm.ACT_RELU)
+            ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, din0, pt.indices_bwd, ms_h, order_h, tile_m=64, dtype_in=dtype,
+                                                     dtype_w=dtype, dtype_out=dtype, mask_filter=filt, reverse_mask=True)
+            assert H.rel_err(H.as_f32(results[(True, 0)][0], dtype), H.as_f32(ref, dtype)) < TOL
+            assert H.rel_err(H.as_f32(results[(True, 0)][1], dtype), H.as_f32(ref_d, dtype)) < TOL
+    base = results[(False, -1)]
+    for key, (out, din) in results.items():
+        np.testing.assert_array_equal(out.view(np.uint16), base[0].view(np.uint16), err_msg=str(key))
+        np.testing.assert_array_equal(din.view(np.uint16), base[1].view(np.uint16), err_msg=str(key))

@@ -137,6 +137,50 @@ def test_subm_f16_c64_two_tile_shapes_full_size():
     assert H.rel_err_rows(H.as_f32(dins[1], dtype), H.as_f32(ref_d, dtype)) < TOL
 
 
+def test_subm_f16_c64_order_by_offset_count_full_size():
+    """The headline voxel set with input preparation as the benchmark does it: the GPU sort in its
+    order by offset count, the hints found on the device (pairs for the light end, halves for
+    the heavy end), the pair table by row and by position.  Same output bits as the launch on
+    masks sorted by value without hints; tile masks and values against the oracle."""
+    print("case full size subm f16, order by offset count", flush=True)
+    dtype, tile_m, filt = "f16", 64, 0x07FFFFFF
+    rng, pt, feat, w, n = _subm_case(20240607, 120000, dtype, 64, 64)
+    d_mask = H.dev(pt.mask_fwd, "u32")
+    d_feat, d_w, d_ind = H.dev(feat, dtype), H.dev(w, dtype), H.dev(pt.indices_fwd, "i32")
+    out0 = np.zeros((n, 64), np.float16)
+    tiles = (n + tile_m - 1) // tile_m
+
+    def run(ms, order, hint, by_pos):
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.Forward, tile_m, 64)
+        p.input, p.weight, p.output = d_feat, d_w, H.dev(out0, dtype)
+        p.indices = pairs.pairs_by_position_device(d_ind, order) if by_pos else d_ind
+        p.indices_by_position = by_pos
+        p.mask, p.mask_argsort, p.mask_filter = ms, order, filt
+        p.mask_output = tv.zeros([tiles], tv.uint32, 0)
+        p.light_prefix = hint
+        ConvMainUnitTest.implicit_gemm2(p)
+        return H.host(p.output), H.host(p.mask_output)
+
+    ms_v, order_v = pairs.sort_by_mask_device(d_mask, filt)
+    base, _ = run(ms_v, order_v, -1, False)
+    ms_c, order_c = pairs.sort_by_mask_device(d_mask, filt, by_offset_count=True)
+    ms_h, order_h = pairs.sort_by_mask(pt.mask_fwd, filt, by_offset_count=True)
+    np.testing.assert_array_equal(H.host(ms_c), ms_h)
+    np.testing.assert_array_equal(H.host(order_c), order_h)
+    light, heavy = pairs.hints_device(ms_c, filt)
+    assert light == pairs.light_prefix(ms_h, light_offsets=3) and heavy == pairs.heavy_from(ms_h)
+    assert light >= 64 * 1000 and 0 < (n - heavy) // 64 <= tiles // 8            # hundreds of pairs, some halves
+    ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms_h, order_h, tile_m=tile_m, dtype_in=dtype,
+                                                 dtype_w=dtype, dtype_out=dtype, mask_filter=filt)
+    for by_pos in (False, True):
+        got, mo = run(ms_c, order_c, 0, by_pos)
+        np.testing.assert_array_equal(got.view(np.uint16), base.view(np.uint16))
+        np.testing.assert_array_equal(mo, ref_mo)
+    assert H.rel_err(H.as_f32(got, dtype), H.as_f32(ref, dtype)) < TOL
+    assert H.rel_err_rows(H.as_f32(got, dtype), H.as_f32(ref, dtype)) < TOL
+
+
 def test_subm_f16_c64_wgrad_full_size():
     """Backward-weight at the benchmark size with the balanced descriptor and split_k_slices = 32
     (eight fp32 images), on the reduced masks that the forward pass writes."""

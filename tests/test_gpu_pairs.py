@@ -269,3 +269,42 @@ def test_sort_leaves_the_light_prefix_for_the_launch():
     for got, mo in outs:
         np.testing.assert_array_equal(got.view(np.uint16), outs[0][0].view(np.uint16))
         np.testing.assert_array_equal(mo, ref_mo)
+
+
+@pytest.mark.parametrize("n", [1, 127, 4097, 50000, 300001])
+@pytest.mark.parametrize("kind", ["cloud", "random27", "few", "all_equal"])
+def test_sort_by_offset_count_against_the_host(n, kind):
+    """cumm_hip_sort_by_mask_ordered, order 1 (ascending number of kernel offsets, then value)
+    against the host's stable argsort of the same key, and what the sort leaves in the hint table
+    for its result - the light prefix (counted with three offsets for this order) and the start
+    of the heavy end - against the host counts; a filter of more than 27 bits is refused."""
+    print("case sort by count", n, kind, flush=True)
+    rng = np.random.default_rng(n + len(kind))
+    if kind == "cloud":
+        # masks as a sparse cloud has them: most positions the centre alone, some with a few neighbours
+        mask = np.full(n, 1 << 13, np.uint32)
+        extra = rng.random(n)
+        for frac, bits in ((0.35, 1), (0.12, 2), (0.04, 4), (0.01, 7)):
+            sel = extra < frac
+            for _ in range(bits):
+                mask[sel] |= (np.uint32(1) << rng.integers(0, 27, size=int(sel.sum())).astype(np.uint32))
+    elif kind == "random27":
+        mask = rng.integers(0, 1 << 27, size=n, dtype=np.uint32)
+    elif kind == "few":
+        mask = rng.choice(np.array([0x2000, 0x6000, 0x7FFFFFF, 0x2001, 0x4002000], np.uint32), size=n)
+    else:
+        mask = np.full(n, 0x2000, np.uint32)
+    d_mask = H.dev(mask, "u32")
+    for filt in (0x07FFFFFF, 0x3FFF, 0x1FFF << 14):
+        ms_ref, order_ref = pairs.sort_by_mask(mask, filt, by_offset_count=True)
+        ms, order = pairs.sort_by_mask_device(d_mask, filt, by_offset_count=True)
+        np.testing.assert_array_equal(H.host(ms), ms_ref)
+        np.testing.assert_array_equal(H.host(order), order_ref)
+        assert pairs.hints_device(ms, filt) == (pairs.light_prefix(ms_ref, light_offsets=3), pairs.heavy_from(ms_ref))
+        ms_v, _ = pairs.sort_by_mask_device(d_mask, filt)
+        ms_vref, _ = pairs.sort_by_mask(mask, filt)
+        assert pairs.hints_device(ms_v, filt) == (pairs.light_prefix(ms_vref), pairs.heavy_from(ms_vref))
+    with pytest.raises(ValueError):
+        pairs.sort_by_mask_device(d_mask, 0xFFFFFFFF, by_offset_count=True)
+    from cumm_amd.gemm.main import GemmMainUnitTest
+    GemmMainUnitTest.device_synchronize()
