@@ -1470,7 +1470,8 @@ int cumm_hip_relu_backward(void *dst, const void *grad, const void *out, size_t 
 }
 
 size_t cumm_hip_column_sum_workspace(int64_t rows, int channels) {
-  if (rows <= 0 || channels <= 0) return 0;
+  if (rows < 0 || channels <= 0) return 0;
+  // (no rows: the sums are zeros, written through one block of partial sums all the same)
   return sizeof(float) * (size_t)column_sum_blocks(rows, channels) * (size_t)channels;
 }
 

@@ -289,6 +289,12 @@ def subm_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 3), dil
         ind_f, ind_b, mask_f, mask_b = out
         if (ind_f.shape != [kv, n] or ind_b.shape != [kv, n] or ind_f.dtype != tv.int32 or ind_b.dtype != tv.int32):
             raise ValueError("out must hold int32 tables of shape [kv, N]")
+        for m in (mask_f, mask_b):
+            if kv > 32:
+                if m is not None:
+                    raise ValueError("kernel volumes above 32 have no 32-bit masks: out must hold None for them")
+            elif m is None or m.shape != [n] or m.dtype != tv.uint32 or m.device < 0:
+                raise ValueError("out must hold uint32 device masks of shape [N]")
     else:
         ind_f = tv.empty([kv, n], tv.int32, 0)
         ind_b = tv.empty([kv, n], tv.int32, 0)
@@ -343,7 +349,9 @@ def sparse_conv_pairs_device(coords, spatial_shape: Sequence[int], ksize=(3, 3, 
                                               workspace.byte_pointer(), workspace.nbytes, stream))
     n = int(n_out.value)
     if out is not None and out.indices_fwd.shape == [kv, n] and out.indices_bwd.shape == [kv, n_in] and \
-            out.out_coords.shape == [n, 4] and (out.mask_fwd is None) == (kv > 32):
+            out.out_coords.shape == [n, 4] and (out.mask_fwd is None) == (kv > 32) and (out.mask_bwd is None) == (kv > 32) and \
+            (kv > 32 or (out.mask_fwd.shape == [n] and out.mask_bwd.shape == [n_in] and
+                         out.mask_fwd.dtype == tv.uint32 and out.mask_bwd.dtype == tv.uint32)):
         out_coords, ind_f, ind_b, mask_f, mask_b = out.out_coords, out.indices_fwd, out.indices_bwd, out.mask_fwd, out.mask_bwd
     else:
         out_coords = tv.empty([n, 4], tv.int32, 0)

@@ -117,9 +117,18 @@ class _Launch:
         self.fields = {}
         for role, t in roles.items():
             ptr = t.data_ptr()
+            if t.numel() == 0:     # an empty tensor has no address to find in the block: nothing to patch
+                self.fields[role] = []
+                continue
             self.fields[role] = [f for f in self._FIELDS if ptr and getattr(self.args, f) == ptr]
             if not self.fields[role]:
                 raise RuntimeError("the argument block does not point at the %s tensor" % role)
+        # the tensors of the first call are replaced by the caller's on every replay: only the
+        # geometry's stay referenced here (a backward-weight workspace can be tens of megabytes)
+        from .tensorview import Tensor as _T
+        for name in ("input", "weight", "output", "bias", "workspace"):
+            if name in roles:
+                params.__dict__[name] = _T()
 
     def __call__(self, stream: int, **tensors) -> None:
         for role, t in tensors.items():
@@ -171,6 +180,11 @@ class SparseConvGeometry:
         # backward-input launches - stays on the device: the sort leaves it in the library's table
         # under the sorted array's address and the launches look it up there; 0 = not given here)
         self.light_fwd = self.light_bwd = 0
+        # the pair tables once more in the order of the sorted positions: what forward and
+        # backward-input read (a tile's entries for one offset are then consecutive in memory);
+        # backward-weight keeps the table by row
+        self.indices_fwd_pos = pairs.pairs_by_position_device(self.indices_fwd, self.order_fwd, stream=stream)
+        self.indices_bwd_pos = pairs.pairs_by_position_device(self.indices_bwd, self.order_bwd, stream=stream)
         self._reduced = {}
         self._launches = {}      # validated calls of the layers on this geometry, see _Launch
 
@@ -212,7 +226,8 @@ class _SparseConvFunction(torch.autograd.Function):
         p = ConvParams(3, ConvOpType.Forward)
         p.conv_algo_desp = _desp_like(dtype, ConvOpType.Forward)
         p.input, p.weight, p.output = torch2tensor(features), torch2tensor(weight), torch2tensor(out)
-        p.indices, p.mask, p.mask_argsort = geometry.indices_fwd, geometry.mask_fwd, geometry.order_fwd
+        p.indices, p.mask, p.mask_argsort = geometry.indices_fwd_pos, geometry.mask_fwd, geometry.order_fwd
+        p.indices_by_position = True
         p.light_prefix = geometry.light_fwd
         if bias is not None:
             p.bias, p.beta = torch2tensor(bias), 1.0
@@ -257,7 +272,8 @@ class _SparseConvFunction(torch.autograd.Function):
                 p = ConvParams(3, ConvOpType.BackwardInput)
                 p.conv_algo_desp = _desp_like(dtype, ConvOpType.BackwardInput)
                 p.input, p.weight, p.output = torch2tensor(grad_in), torch2tensor(weight), torch2tensor(grad_out)
-                p.indices, p.mask, p.mask_argsort = g.indices_bwd, g.mask_bwd, g.order_bwd
+                p.indices, p.mask, p.mask_argsort = g.indices_bwd_pos, g.mask_bwd, g.order_bwd
+                p.indices_by_position = True
                 p.reverse_mask = g.subm
                 p.light_prefix = g.light_bwd
                 p.stream = stream
