@@ -1277,7 +1277,9 @@ int cumm_hip_conv_pairs_sites(const int32_t *coords, int n_in, int batch_size, c
   HIP_TRY(hipStreamSynchronize(s));
   if (counters[0] > l.bound) return fail(CUMM_HIP_ERUNTIME, "more output sites than the geometry allows (duplicate coordinates?)");
   p.n_out = (int)counters[0];
-  e = launch_conv_pairs_sort(p, counters[1], temp, l.total - l.off_temp, s);
+  int32_t *status = nullptr;
+  if (int rc = async_status_ptr(&status)) return rc;
+  e = launch_conv_pairs_sort(p, counters[1], temp, l.total - l.off_temp, status + 1, s);
   if (e != hipSuccess) return hip_fail(e, "output site sort");
   *n_out = p.n_out;
   return CUMM_HIP_OK;

@@ -109,7 +109,7 @@ struct ConvPairsParams {
 hipError_t launch_conv_pairs_sites(const ConvPairsParams &p, hipStream_t s);
 size_t conv_pairs_sort_temp_bytes(size_t max_sites);
 hipError_t launch_conv_pairs_sort(const ConvPairsParams &p, unsigned long long max_key, void *temp, size_t temp_bytes,
-                                  hipStream_t s);
+                                  int32_t *give_ups, hipStream_t s);
 hipError_t launch_conv_pairs_fill(const ConvPairsParams &p, hipStream_t s);
 size_t conv_pairs_scan_temp_bytes(size_t n_words);
 hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t temp_bytes, hipStream_t s);

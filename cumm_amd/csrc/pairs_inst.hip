@@ -22,9 +22,6 @@
 
 #include <cstring>
 
-#include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_scan.hpp>
-#include <rocprim/iterator/transform_iterator.hpp>
 
 #include "launch.h"
 
@@ -328,14 +325,102 @@ __global__ __launch_bounds__(256) void conv_bits_sites_kernel(const ConvPairsPar
   if (!(__atomic_load_n(&p.bits[key >> 5], __ATOMIC_RELAXED) & bit)) atomicOr(&p.bits[key >> 5], bit);
 }
 
-// number of active sites, behind the prefix sums (one 4-byte copy to the host instead of two)
-__global__ void conv_bits_total_kernel(const ConvPairsParams p) {
-  p.prefix[p.n_words] = p.prefix[p.n_words - 1] + (uint32_t)__popc(p.bits[p.n_words - 1]);
+// ---- prefix[w] = number of set bits in the words before w (exclusive scan of the words' bit counts),
+// prefix[n_words] = their total.  Three small kernels: bit counts per block of kScanBlock words, one
+// workgroup that turns the block counts into offsets (carrying its running sum from one batch of
+// 256 blocks to the next), and the scan inside every block again, now with its offset.
+constexpr int kScanPerThread = 16;
+constexpr int kScanBlock = 256 * kScanPerThread;   // words per workgroup
+
+// a workgroup-wide exclusive scan of one value per thread (256 threads); returns the total in *total
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t *lds_waves, uint32_t *total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t incl = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+  __syncthreads();   // (lds_waves may still be read from a previous call)
+  if (lane == 63) lds_waves[wave] = incl;
+  __syncthreads();
+  uint32_t before = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const uint32_t c = lds_waves[w];
+    before += w < wave ? c : 0u;
+    all += c;
+  }
+  *total = all;
+  return before + incl - v;
 }
 
-struct BitCount {
-  __host__ __device__ uint32_t operator()(uint32_t w) const { return (uint32_t)__builtin_popcount(w); }
-};
+__global__ __launch_bounds__(256) void bit_scan_block_sums_kernel(const uint32_t *__restrict__ bits, unsigned long long n_words,
+                                                                  uint32_t *__restrict__ block_sums) {
+  __shared__ uint32_t lds_waves[4];
+  const unsigned long long base = (unsigned long long)blockIdx.x * kScanBlock;
+  uint32_t c = 0;
+#pragma unroll
+  for (int u = 0; u < kScanPerThread; ++u) {
+    const unsigned long long w = base + (unsigned long long)u * 256 + threadIdx.x;
+    c += w < n_words ? (uint32_t)__popc(bits[w]) : 0u;
+  }
+  uint32_t total;
+  (void)block_exclusive_scan(c, lds_waves, &total);
+  if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(256) void bit_scan_block_offsets_kernel(uint32_t *__restrict__ block_sums, unsigned long long n_blocks,
+                                                                     uint32_t *__restrict__ total_out) {
+  __shared__ uint32_t lds_waves[4];
+  uint32_t carry = 0;
+  for (unsigned long long b0 = 0; b0 < n_blocks; b0 += 256) {
+    const unsigned long long b = b0 + threadIdx.x;
+    const uint32_t v = b < n_blocks ? block_sums[b] : 0u;
+    uint32_t total;
+    const uint32_t excl = block_exclusive_scan(v, lds_waves, &total);
+    if (b < n_blocks) block_sums[b] = carry + excl;
+    carry += total;
+  }
+  if (threadIdx.x == 0) *total_out = carry;
+}
+
+__global__ __launch_bounds__(256) void bit_scan_write_kernel(const uint32_t *__restrict__ bits, unsigned long long n_words,
+                                                             const uint32_t *__restrict__ block_sums, uint32_t *__restrict__ prefix) {
+  __shared__ uint32_t lds_waves[4];
+  // thread t owns kScanPerThread consecutive words (so that its own scan is a running sum)
+  const unsigned long long first = (unsigned long long)blockIdx.x * kScanBlock + (unsigned long long)threadIdx.x * kScanPerThread;
+  uint32_t cnt[kScanPerThread], mine = 0;
+#pragma unroll
+  for (int u = 0; u < kScanPerThread; ++u) {
+    cnt[u] = first + u < n_words ? (uint32_t)__popc(bits[first + u]) : 0u;
+    mine += cnt[u];
+  }
+  uint32_t total;
+  uint32_t run = block_sums[blockIdx.x] + block_exclusive_scan(mine, lds_waves, &total);
+#pragma unroll
+  for (int u = 0; u < kScanPerThread; ++u) {
+    if (first + u < n_words) prefix[first + u] = run;
+    run += cnt[u];
+  }
+}
+
+// ---- the pieces of a 64-bit key sort out of two stable 32-bit sorts (sort_inst.hip)
+__global__ __launch_bounds__(256) void key_low_words_kernel(const unsigned long long *__restrict__ keys, uint32_t *__restrict__ out, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (uint32_t)keys[i];
+}
+__global__ __launch_bounds__(256) void key_high_words_kernel(const unsigned long long *__restrict__ keys, const int32_t *__restrict__ perm,
+                                                             uint32_t *__restrict__ out, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (uint32_t)(keys[perm[i]] >> 32);
+}
+// out[i] = keys[perm1[perm2[i]]] (perm2 NULL: keys[perm1[i]])
+__global__ __launch_bounds__(256) void key_gather_kernel(const unsigned long long *__restrict__ keys, const int32_t *__restrict__ perm1,
+                                                         const int32_t *__restrict__ perm2, unsigned long long *__restrict__ out, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = keys[perm1[perm2 ? perm2[i] : i]];
+}
 
 // table prefill, masks, and the coordinates of the active sites, word by word
 __global__ __launch_bounds__(256) void conv_bits_rows_kernel(const ConvPairsParams p) {
@@ -557,20 +642,41 @@ hipError_t launch_conv_pairs_sites(const ConvPairsParams &p, hipStream_t s) {
   return hipGetLastError();
 }
 
+// 64-bit keys, ascending: a stable sort by the low words, then a stable sort of that order by the
+// high words (skipped when no key has any), each the radix sort of the mask sort.
+// temp: six arrays of n words (low words, their sorted copy, the first order, high words in that
+// order, their sorted copy, the second order) and the sort's own workspace.
+static size_t key_sort_part(size_t n) { return (4 * (n > 0 ? n : 1) + 255) & ~(size_t)255; }
 size_t conv_pairs_sort_temp_bytes(size_t max_sites) {
-  size_t bytes = 0;
-  (void)rocprim::radix_sort_keys(nullptr, bytes, (const unsigned long long *)nullptr, (unsigned long long *)nullptr,
-                                 max_sites > 0 ? max_sites : 1, 0, 64);
-  return bytes;
+  return 6 * key_sort_part(max_sites) + sort_by_mask_workspace_bytes((int)(max_sites > 0 ? max_sites : 1));
 }
 
 hipError_t launch_conv_pairs_sort(const ConvPairsParams &p, unsigned long long max_key, void *temp, size_t temp_bytes,
-                                  hipStream_t s) {
+                                  int32_t *give_ups, hipStream_t s) {
   if (p.n_out <= 0) return hipSuccess;
-  int end_bit = 1;
-  while (end_bit < 64 && (max_key >> end_bit) != 0ull) ++end_bit;
-  return rocprim::radix_sort_keys(temp, temp_bytes, (const unsigned long long *)p.uniq, p.sorted, (size_t)p.n_out, 0,
-                                  end_bit, s);
+  const int n = p.n_out;
+  if (temp_bytes < conv_pairs_sort_temp_bytes((size_t)n)) return hipErrorInvalidValue;
+  const size_t part = key_sort_part((size_t)n);
+  char *base = reinterpret_cast<char *>(temp);
+  uint32_t *lo = reinterpret_cast<uint32_t *>(base), *lo_sorted = reinterpret_cast<uint32_t *>(base + part);
+  int32_t *perm1 = reinterpret_cast<int32_t *>(base + 2 * part);
+  uint32_t *hi = reinterpret_cast<uint32_t *>(base + 3 * part), *hi_sorted = reinterpret_cast<uint32_t *>(base + 4 * part);
+  int32_t *perm2 = reinterpret_cast<int32_t *>(base + 5 * part);
+  void *sort_ws = base + 6 * part;
+  const dim3 grid((n + 255) / 256);
+  hipLaunchKernelGGL(key_low_words_kernel, grid, dim3(256), 0, s, p.uniq, lo, n);
+  hipError_t e = launch_sort_by_mask(lo, n, 0xFFFFFFFFu, lo_sorted, perm1, sort_ws, give_ups, nullptr, 0, s);
+  if (e != hipSuccess) return e;
+  const bool two = (max_key >> 32) != 0ull;
+  if (two) {
+    hipLaunchKernelGGL(key_high_words_kernel, grid, dim3(256), 0, s, p.uniq, perm1, hi, n);
+    uint32_t filter = 1;
+    while (filter != 0xFFFFFFFFu && (max_key >> 32) > filter) filter = (filter << 1) | 1u;   // the bits the high words use
+    e = launch_sort_by_mask(hi, n, filter, hi_sorted, perm2, sort_ws, give_ups, nullptr, 0, s);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(key_gather_kernel, grid, dim3(256), 0, s, p.uniq, perm1, two ? perm2 : nullptr, p.sorted, n);
+  return hipGetLastError();
 }
 
 hipError_t launch_conv_pairs_fill(const ConvPairsParams &p, hipStream_t s) {
@@ -591,11 +697,9 @@ hipError_t launch_conv_pairs_fill(const ConvPairsParams &p, hipStream_t s) {
   return hipGetLastError();
 }
 
+// block counts of the bit scan
 size_t conv_pairs_scan_temp_bytes(size_t n_words) {
-  size_t bytes = 0;
-  (void)rocprim::exclusive_scan(nullptr, bytes, rocprim::make_transform_iterator((const uint32_t *)nullptr, BitCount()),
-                                (uint32_t *)nullptr, 0u, n_words > 0 ? n_words : 1, rocprim::plus<uint32_t>());
-  return bytes;
+  return 4 * ((n_words + kScanBlock - 1) / kScanBlock + 1);
 }
 
 // bitmap of the active output sites and its prefix sums
@@ -608,10 +712,12 @@ hipError_t launch_conv_pairs_bits(const ConvPairsParams &p, void *temp, size_t t
     hipLaunchKernelGGL(conv_bits_sites_kernel, dim3((p.n_in + 255) / 256, p.kv), dim3(256), 0, s, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  e = rocprim::exclusive_scan(temp, temp_bytes, rocprim::make_transform_iterator((const uint32_t *)p.bits, BitCount()),
-                              p.prefix, 0u, (size_t)p.n_words, rocprim::plus<uint32_t>(), s);
-  if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(conv_bits_total_kernel, dim3(1), dim3(1), 0, s, p);
+  const unsigned long long n_blocks = (p.n_words + kScanBlock - 1) / kScanBlock;
+  if (n_blocks == 0ull || n_blocks > 0x7fffffffull || temp_bytes < conv_pairs_scan_temp_bytes((size_t)p.n_words)) return hipErrorInvalidValue;
+  uint32_t *block_sums = reinterpret_cast<uint32_t *>(temp);
+  hipLaunchKernelGGL(bit_scan_block_sums_kernel, dim3((unsigned)n_blocks), dim3(256), 0, s, p.bits, p.n_words, block_sums);
+  hipLaunchKernelGGL(bit_scan_block_offsets_kernel, dim3(1), dim3(256), 0, s, block_sums, n_blocks, p.prefix + p.n_words);
+  hipLaunchKernelGGL(bit_scan_write_kernel, dim3((unsigned)n_blocks), dim3(256), 0, s, p.bits, p.n_words, block_sums, p.prefix);
   return hipGetLastError();
 }
 

@@ -818,7 +818,7 @@ __global__ __launch_bounds__(256) void rowgemm_lds_mixed_kernel(const RowGemmPar
                      (slot[2] == p.n_pos) & ((((uint32_t)slot[3] ^ p.mask_filter) & live_bits) == 0u);
   // (a count from the caller comes with a slot that names nothing: one of the two is zero, and the
   // OR keeps the slot's load out of a branch, where it would wait for the pointer first)
-  const int hinted = p.pair_tiles | (named & (slot[4] > 0) ? slot[4] >> 7 : 0);
+  const int hinted = p.pair_tiles | ((named & (slot[4] > 0)) ? slot[4] >> 7 : 0);
   const int pairs = hinted < (tiles >> 1) ? hinted : (tiles >> 1);
   // The heavy end: the 64-row tiles from slot word 5 on are taken as two halves of 32 rows each,
   // which halves the life of the launch's longest tiles - when they are few (an eighth of the
