@@ -226,10 +226,13 @@ def bench_stack(args):
         return tv.from_numpy(np.ascontiguousarray(synth.f32_to_bf16_bits(v))).type_view(tv.bfloat16).cuda()
 
     t0 = time.perf_counter()
+    # input preparation as the library offers it: positions ordered by offset count, and the pair
+    # tables once more in that order for the forward / backward-input launches
+    filt = (1 << 27) - 1
     table = pairs.subm_pairs_device(d_coords, grid)
-    ms_tv, order_tv = pairs.sort_by_mask_device(table.mask_fwd)
+    ms_tv, order_tv = pairs.sort_by_mask_device(table.mask_fwd, filt, by_offset_count=True)
     table2 = pairs.sparse_conv_pairs_device(d_coords, grid, batch_size=1)
-    ms2_tv, order2_tv = pairs.sort_by_mask_device(table2.mask_fwd)
+    ms2_tv, order2_tv = pairs.sort_by_mask_device(table2.mask_fwd, filt, by_offset_count=True)
     ConvMainUnitTest_sync()
     prep_ms = (time.perf_counter() - t0) * 1e3          # first call, allocations included
     n_out2 = int(table2.indices_fwd.dim(1))
@@ -245,9 +248,9 @@ def bench_stack(args):
     ws_c = tv.empty([int(lib.cumm_hip_conv_pairs_workspace(n, 1, arr3(*grid), arr3(3, 3, 3), arr3(2, 2, 2), arr3(1, 1, 1),
                                                            arr3(1, 1, 1)))], tv.uint8, 0)
     for name, fn in (("subm_pairs", lambda: pairs.subm_pairs_device(d_coords, grid, workspace=ws_p, out=table)),
-                     ("sort_by_mask", lambda: pairs.sort_by_mask_device(table.mask_fwd, workspace=ws_s, out=sorted1)),
+                     ("sort_by_mask", lambda: pairs.sort_by_mask_device(table.mask_fwd, filt, workspace=ws_s, out=sorted1, by_offset_count=True)),
                      ("sparse_conv_pairs_stride2", lambda: pairs.sparse_conv_pairs_device(d_coords, grid, batch_size=1, workspace=ws_c, out=table2)),
-                     ("sort_by_mask_stride2", lambda: pairs.sort_by_mask_device(table2.mask_fwd, workspace=ws_s, out=sorted2))):
+                     ("sort_by_mask_stride2", lambda: pairs.sort_by_mask_device(table2.mask_fwd, filt, workspace=ws_s, out=sorted2, by_offset_count=True))):
         wms, ems = timed(fn, 5, 2)
         prep[name] = {"wall_ms": round(wms, 4), "events_ms": round(ems, 4)}
     pairs1 = int((table.indices_fwd.cpu().numpy() >= 0).sum())
@@ -260,27 +263,35 @@ def bench_stack(args):
     res = {"voxels": n, "pairs": pairs1, "voxels_out_stride2": n_out2, "pairs_stride2": pairs2,
            "input_preparation_first_call_ms": round(prep_ms, 3), "input_preparation_ms": prep}
 
-    def leg(name, p, flops):
+    def leg(name, p, flops, alg_bytes):
         r = tn.tune_conv(p)
         wms, ems = timed(lambda: ConvMainUnitTest.implicit_gemm2(p), steps, warm)
         res[name] = {"tile": list(r.desp.tile_shape[:2]),
                      "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
                                     for nm, ms in r.tried},
-                     "ms_per_step": round(wms, 5),
-                     "tflops": round(flops / (wms * 1e-3) / 1e12, 2)}
+                     "ms_per_step": round(wms, 5), "kernel_ms_events": round(ems, 5),
+                     "tflops": round(flops / (wms * 1e-3) / 1e12, 2),
+                     "hbm_frac": round(alg_bytes / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+
+    # algorithmic bytes: rows in and out once, weights, the pair table, masks and order
+    def conv_bytes(n_a, c_a, n_c, c_c, n_pos, k_w):
+        return n_a * c_a * 2 + n_c * c_c * 2 + 27 * k_w * 2 + 27 * n_pos * 4 + n_pos * 8
+    pos1 = pairs.pairs_by_position_device(table.indices_fwd, order_tv)
+    pos1b = pairs.pairs_by_position_device(table.indices_bwd, order_tv)
+    pos2 = pairs.pairs_by_position_device(table2.indices_fwd, order2_tv)
 
     pf = ConvParams(3, ConvOpType.Forward)
     pf.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 128, 128)
     pf.input, pf.weight, pf.bias, pf.output = x, w, b, tv.zeros([n, c], tv.bfloat16, 0)
-    pf.indices, pf.mask, pf.mask_argsort = table.indices_fwd, ms_tv, order_tv
+    pf.indices, pf.mask, pf.mask_argsort, pf.indices_by_position = pos1, ms_tv, order_tv, True
     pf.beta, pf.act_type = 1.0, Activation.ReLU
-    leg("subm_c128_forward", pf, 2.0 * pairs1 * c * c)
+    leg("subm_c128_forward", pf, 2.0 * pairs1 * c * c, conv_bytes(n, c, n, c, n, c * c))
     pd = ConvParams(3, ConvOpType.BackwardInput)
     pd.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.BackwardInput, 128, 128)
     pd.input, pd.weight, pd.output = tv.zeros([n, c], tv.bfloat16, 0), w, dout
-    pd.indices, pd.mask, pd.mask_argsort = table.indices_bwd, ms_tv, order_tv
+    pd.indices, pd.mask, pd.mask_argsort, pd.indices_by_position = pos1b, ms_tv, order_tv, True
     pd.reverse_mask = True
-    leg("subm_c128_backward_input", pd, 2.0 * pairs1 * c * c)
+    leg("subm_c128_backward_input", pd, 2.0 * pairs1 * c * c, conv_bytes(n, c, n, c, n, c * c))
     red = tv.zeros([(n + 63) // 64], tv.uint32, 0)
     pm = ConvParams(3, ConvOpType.Forward)        # a forward call with 64-row tiles writes the reduced masks
     pm.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 64, 128)
@@ -292,29 +303,33 @@ def bench_stack(args):
     pw.input, pw.weight, pw.output = x, tv.zeros([c, 27, c], tv.bfloat16, 0), dout
     pw.indices, pw.mask, pw.mask_argsort = table.indices_fwd, red, order_tv
     pw.mask_width, pw.split_k_slices = 64, 32
-    wms, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), steps, warm)
+    wms, ems = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), steps, warm)
     pw.deterministic, pw.workspace = True, tv.Tensor()
-    wms_fixed, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), steps, warm)
+    wms_fixed, ems_fixed = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw), steps, warm)
     pw.deterministic, pw.workspace = False, tv.Tensor()
-    res["subm_c128_backward_weight_fixed_order"] = {"ms_per_step": round(wms_fixed, 5)}
+    wbytes = n * c * 2 * 2 + 27 * n * 4 + n * 4 + 4 * ((n + 63) // 64) + 27 * c * c * 2
+    res["subm_c128_backward_weight_fixed_order"] = {"ms_per_step": round(wms_fixed, 5),
+                                                    "hbm_frac": round(wbytes / (ems_fixed * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     res["subm_c128_backward_weight_balanced"] = {"ms_per_step": round(wms, 5),
-                                                 "tflops": round(2.0 * pairs1 * c * c / (wms * 1e-3) / 1e12, 2)}
+                                                 "tflops": round(2.0 * pairs1 * c * c / (wms * 1e-3) / 1e12, 2),
+                                                 "hbm_frac": round(wbytes / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     p2 = ConvParams(3, ConvOpType.Forward)
     p2.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 128, 128)
     p2.input, p2.weight, p2.bias, p2.output = x, w2, b2, tv.zeros([n_out2, 256], tv.bfloat16, 0)
-    p2.indices, p2.mask, p2.mask_argsort = table2.indices_fwd, ms2_tv, order2_tv
+    p2.indices, p2.mask, p2.mask_argsort, p2.indices_by_position = pos2, ms2_tv, order2_tv, True
     p2.beta, p2.act_type = 1.0, Activation.ReLU
     red2 = tv.zeros([(n_out2 + 63) // 64], tv.uint32, 0)
-    leg("stride2_c128_c256_forward", p2, 2.0 * pairs2 * c * 256)
+    leg("stride2_c128_c256_forward", p2, 2.0 * pairs2 * c * 256, conv_bytes(n, c, n_out2, 256, n_out2, c * 256))
     # the stride-2 layer's backward passes: input gradient on the input-side masks, weight gradient
     # on the reduced masks of a 64-row forward
     dout2 = bf16((n_out2, 256), 1 / 64)
-    msb2_tv, orderb2_tv = pairs.sort_by_mask_device(table2.mask_bwd)
+    msb2_tv, orderb2_tv = pairs.sort_by_mask_device(table2.mask_bwd, filt, by_offset_count=True)
+    pos2b = pairs.pairs_by_position_device(table2.indices_bwd, orderb2_tv)
     pd2 = ConvParams(3, ConvOpType.BackwardInput)
     pd2.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.BackwardInput, 128, 128)
     pd2.input, pd2.weight, pd2.output = tv.zeros([n, c], tv.bfloat16, 0), w2, dout2
-    pd2.indices, pd2.mask, pd2.mask_argsort = table2.indices_bwd, msb2_tv, orderb2_tv
-    leg("stride2_c128_c256_backward_input", pd2, 2.0 * pairs2 * c * 256)
+    pd2.indices, pd2.mask, pd2.mask_argsort, pd2.indices_by_position = pos2b, msb2_tv, orderb2_tv, True
+    leg("stride2_c128_c256_backward_input", pd2, 2.0 * pairs2 * c * 256, conv_bytes(n_out2, 256, n, c, n, c * 256))
     pm2 = ConvParams(3, ConvOpType.Forward)
     pm2.conv_algo_desp = find_desp(tv.bfloat16, ConvOpType.Forward, 64, 128)
     pm2.input, pm2.weight, pm2.output = x, w2, tv.zeros([n_out2, 256], tv.bfloat16, 0)
@@ -325,13 +340,16 @@ def bench_stack(args):
     pw2.input, pw2.weight, pw2.output = x, tv.zeros([256, 27, c], tv.bfloat16, 0), dout2
     pw2.indices, pw2.mask, pw2.mask_argsort = table2.indices_fwd, red2, order2_tv
     pw2.mask_width, pw2.split_k_slices = 64, 32
-    wms, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw2), steps, warm)
+    wms, ems = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw2), steps, warm)
     pw2.deterministic, pw2.workspace = True, tv.Tensor()
-    wms_fixed, _ = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw2), steps, warm)
+    wms_fixed, ems_fixed = timed(lambda: ConvMainUnitTest.implicit_gemm2(pw2), steps, warm)
     pw2.deterministic, pw2.workspace = False, tv.Tensor()
-    res["stride2_c128_c256_backward_weight_fixed_order"] = {"ms_per_step": round(wms_fixed, 5)}
+    wbytes2 = n * c * 2 + n_out2 * 256 * 2 + 27 * n_out2 * 4 + n_out2 * 4 + 4 * ((n_out2 + 63) // 64) + 27 * c * 256 * 2
+    res["stride2_c128_c256_backward_weight_fixed_order"] = {"ms_per_step": round(wms_fixed, 5),
+                                                            "hbm_frac": round(wbytes2 / (ems_fixed * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     res["stride2_c128_c256_backward_weight_balanced"] = {
-        "ms_per_step": round(wms, 5), "tflops": round(2.0 * pairs2 * c * 256 / (wms * 1e-3) / 1e12, 2)}
+        "ms_per_step": round(wms, 5), "tflops": round(2.0 * pairs2 * c * 256 / (wms * 1e-3) / 1e12, 2),
+        "hbm_frac": round(wbytes2 / (ems * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
 
     # ---- the whole stack: 4 SubM C = 128 layers (bias + ReLU) + the stride-2 128 -> 256 layer,
     # forward then full backward (input and weight gradients of every layer), every launch through
@@ -343,13 +361,13 @@ def bench_stack(args):
         q = ConvParams(3, ConvOpType.Forward)
         q.conv_algo_desp = pf.conv_algo_desp
         q.input, q.weight, q.bias, q.output = acts[i], w, b, acts[i + 1]
-        q.indices, q.mask, q.mask_argsort = table.indices_fwd, ms_tv, order_tv
+        q.indices, q.mask, q.mask_argsort, q.indices_by_position = pos1, ms_tv, order_tv, True
         q.beta, q.act_type = 1.0, Activation.ReLU
         fwd.append(q)
         g = ConvParams(3, ConvOpType.BackwardInput)
         g.conv_algo_desp = pd.conv_algo_desp
         g.input, g.weight, g.output = grads[i], w, grads[i + 1]
-        g.indices, g.mask, g.mask_argsort = table.indices_bwd, ms_tv, order_tv
+        g.indices, g.mask, g.mask_argsort, g.indices_by_position = pos1b, ms_tv, order_tv, True
         g.reverse_mask = True
         bwd_in.append(g)
         u = ConvParams(3, ConvOpType.BackwardWeight)
@@ -361,12 +379,12 @@ def bench_stack(args):
     q5 = ConvParams(3, ConvOpType.Forward)
     q5.conv_algo_desp = p2.conv_algo_desp
     q5.input, q5.weight, q5.bias, q5.output = acts[4], w2, b2, p2.output
-    q5.indices, q5.mask, q5.mask_argsort = table2.indices_fwd, ms2_tv, order2_tv
+    q5.indices, q5.mask, q5.mask_argsort, q5.indices_by_position = pos2, ms2_tv, order2_tv, True
     q5.beta, q5.act_type = 1.0, Activation.ReLU
     g5 = ConvParams(3, ConvOpType.BackwardInput)
     g5.conv_algo_desp = pd2.conv_algo_desp
     g5.input, g5.weight, g5.output = grads[4], w2, dout2
-    g5.indices, g5.mask, g5.mask_argsort = table2.indices_bwd, msb2_tv, orderb2_tv
+    g5.indices, g5.mask, g5.mask_argsort, g5.indices_by_position = pos2b, msb2_tv, orderb2_tv, True
     u5 = ConvParams(3, ConvOpType.BackwardWeight)
     u5.conv_algo_desp = pw2.conv_algo_desp
     u5.input, u5.weight, u5.output = acts[4], pw2.weight, dout2
