@@ -74,6 +74,7 @@ SYMBOLS = {
     "cumm_hip_gemm_supported": (C.c_int, [C.POINTER(GemmDesc)]),
     "cumm_hip_conv_supported": (C.c_int, [C.POINTER(ConvDesc)]),
     "cumm_hip_last_error": (C.c_char_p, []),
+    "cumm_hip_last_wgrad_path": (C.c_int, []),
     "cumm_hip_device_count": (C.c_int, [C.POINTER(C.c_int)]),
     "cumm_hip_malloc": (C.c_int, [_PVP, C.c_size_t]),
     "cumm_hip_free": (C.c_int, [_VP]),

@@ -51,6 +51,13 @@ __device__ __forceinline__ void dma_b32(v4i rsrc, uint32_t lds, uint32_t voff, u
                :: "s"(lds), "v"(voff), "s"(rsrc), "s"(soff) : "memory", "m0");
 }
 
+// The compiler's hazard recognizer does not look into asm statements.  A vector-memory instruction
+// that reads a scalar register within four instructions of the vector instruction that wrote it
+// (v_readlane restoring a spilled descriptor, v_readfirstlane, a compare into a register pair)
+// gets the old value: a descriptor restored just before a hidden load made that load return
+// zeros.  The register loads below therefore start with five wait states of their own; the
+// direct-to-LDS loads above, which sit in the step loops, have two (s_mov m0 + s_nop 0) and are
+// covered by the check of the generated code in cumm_amd/build.py (check_asm_hazards).
 // A 4-byte buffer load into a register that the compiler does not see as a load: it cannot sink it
 // into a branch (a plain load that feeds only a select is moved behind the select's condition and
 // then waited for there, one round trip per conditional value).  To the compiler the result exists
@@ -58,7 +65,7 @@ __device__ __forceinline__ void dma_b32(v4i rsrc, uint32_t lds, uint32_t voff, u
 // the first use, which also keeps the register allocated while the load is in flight.
 __device__ __forceinline__ int load_b32_hidden(v4i rsrc, uint32_t voff) {
   int r;
-  asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
   return r;
 }
 __device__ __forceinline__ void keep_after_wait(int &r) { asm volatile("" : "+v"(r)); }
@@ -66,12 +73,12 @@ __device__ __forceinline__ void keep_after_wait(int &r) { asm volatile("" : "+v"
 typedef int v2i_hidden __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ v2i_hidden load_b64_hidden(v4i rsrc, uint32_t voff) {
   v2i_hidden r;
-  asm volatile("buffer_load_dwordx2 %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  asm volatile("s_nop 4\n\tbuffer_load_dwordx2 %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
   return r;
 }
 __device__ __forceinline__ v4i load_b128_hidden(v4i rsrc, uint32_t voff) {
   v4i r;
-  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, 0 offen" : "=&v"(r) : "v"(voff), "s"(rsrc) : "memory");
   return r;
 }
 __device__ __forceinline__ void keep_after_wait(v2i_hidden &r) { asm volatile("" : "+v"(r)); }
@@ -86,10 +93,10 @@ __device__ __forceinline__ auto load_hidden_words(v4i rsrc, uint32_t voff) {
 // value on the other path).  The register is read-write to the compiler, so both paths end in
 // the same register and no copy - which would copy too early - is needed where they meet.
 __device__ __forceinline__ void load_hidden_into(v2i_hidden &r, v4i rsrc, uint32_t voff) {
-  asm volatile("buffer_load_dwordx2 %0, %1, %2, 0 offen" : "+v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  asm volatile("s_nop 4\n\tbuffer_load_dwordx2 %0, %1, %2, 0 offen" : "+v"(r) : "v"(voff), "s"(rsrc) : "memory");
 }
 __device__ __forceinline__ void load_hidden_into(v4i &r, v4i rsrc, uint32_t voff) {
-  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "+v"(r) : "v"(voff), "s"(rsrc) : "memory");
+  asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, 0 offen" : "+v"(r) : "v"(voff), "s"(rsrc) : "memory");
 }
 
 // Workgroup barrier without the fence of __syncthreads(): the fence would wait for every

@@ -20,13 +20,17 @@ def clustered_voxels(rng: np.random.Generator, n_target: int, grid: Sequence[int
     pts = []
     have = 0
     # oversample: rejection at the grid border and de-duplication both lose points
-    while have < n_clu:
+    # (clusters too small for the count asked for saturate: stop when two rounds in a row add
+    # less than a hundredth of what is missing, and return what there is)
+    stalled = 0
+    while have < n_clu and stalled < 2:
         want = int((n_clu - have) * 1.5) + 1024
         cid = rng.integers(0, n_clusters, size=want)
         p = np.rint(centers[cid] + rng.normal(0.0, sigma, size=(want, 3))).astype(np.int64)
         ok = np.all((p >= 0) & (p < grid), axis=1)
-        pts.append(p[ok])
-        have = np.unique(np.concatenate(pts), axis=0).shape[0]
+        pts = [np.unique(np.concatenate(pts + [p[ok]]), axis=0)]
+        stalled = stalled + 1 if pts[0].shape[0] - have < (n_clu - have) // 100 + 1 else 0
+        have = pts[0].shape[0]
     clu = np.unique(np.concatenate(pts), axis=0)
     if clu.shape[0] > n_clu:
         clu = clu[np.sort(rng.choice(clu.shape[0], n_clu, replace=False))]

@@ -23,9 +23,9 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def _case(seed, n, c_in, k_out, dtype, grid=(12, 40, 36), strided=False):
+def _case(seed, n, c_in, k_out, dtype, grid=(12, 40, 36), strided=False, clusters=6, sigma=3.0):
     rng = np.random.default_rng(seed)
-    coords = synth.clustered_voxels(rng, n, grid, 6, sigma=3.0)
+    coords = synth.clustered_voxels(rng, n, grid, clusters, sigma=sigma)
     if strided:
         pt = pairs.sparse_conv_pairs(coords, grid)
     else:
@@ -390,6 +390,81 @@ def test_backward_weight_fixed_order(dtype, shape, strided):
         assert "workspace at least" in str(e)
     with pytest.raises(RuntimeError, match="workspace at least"):
         run(tv.empty([4096], tv.uint8, 0))
+
+
+def _wgrad_problem(seed, n, c_in, k_out, mask_width, dtype, grid=(12, 40, 36), strided=False, filt=0xFFFFFFFF,
+                   alpha=1.0, beta=0.0, clusters=6, sigma=3.0):
+    rng, coords, pt, feat, w, n_in, n_out = _case(seed, n, c_in, k_out, dtype, grid=grid, strided=strided,
+                                                  clusters=clusters, sigma=sigma)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    red = conv_ref.tile_masks(ms, mask_width)
+    dw0 = H.to_storage(rng.normal(0, 1, size=(k_out, 27, c_in)).astype(np.float32), dtype)
+    ref = conv_ref.implicit_gemm_wgrad_ref(
+        dout, feat, dw0, pt.indices_fwd, red, order, mask_width=mask_width, dtype_dout=dtype,
+        dtype_in=dtype, dtype_w=dtype, mask_filter=filt, alpha=alpha, beta=beta, split_k_slices=1)
+    p = ConvParams(3, ConvOpType.BackwardWeight)
+    p.conv_algo_desp = H.find_conv_desp(dtype, ConvOpType.BackwardWeight, 64, 64, split_k_parallel=True)
+    p.input, p.output = H.dev(feat, dtype), H.dev(dout, dtype)
+    p.indices = H.dev(pt.indices_fwd, "i32")
+    p.mask, p.mask_argsort = H.dev(red, "u32"), H.dev(order, "i32")
+    p.mask_width, p.split_k_slices = mask_width, 4
+    p.mask_filter, p.alpha, p.beta = filt, alpha, beta
+    return p, dw0, H.as_f32(ref, dtype), red
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_backward_weight_one_launch_keeps_its_memory_clean(dtype):
+    """The balanced backward-weight in ONE launch sums into fp32 images that the library owns and
+    that must be zero, tickets included, when a launch starts; the launch itself puts the zeros
+    back.  So: problems of different channel counts, mask widths, filters (offsets switched off,
+    offsets without a live tile: a handful of voxels), alpha and beta, one after the other on one
+    stream, twice over, then the same on a second stream of its own - every result against the
+    oracle.  A leftover of an earlier problem in the images or a ticket would show in a later one."""
+    print("case backward_weight_one_launch", dtype, flush=True)
+    lib = _capi.lib()
+    problems = [
+        _wgrad_problem(21, 3000, 64, 64, 64, dtype),
+        _wgrad_problem(22, 2500, 24, 40, 32, dtype, alpha=0.5, beta=1.0),
+        _wgrad_problem(23, 3000, 128, 128, 64, dtype, strided=True),
+        _wgrad_problem(24, 40, 64, 64, 32, dtype, grid=(30, 60, 60), beta=1.0),      # most offsets have no pair
+        _wgrad_problem(25, 3000, 72, 136, 64, dtype, filt=0x2AAAAAA, alpha=2.0, beta=0.5),
+        _wgrad_problem(26, 9000, 64, 64, 32, dtype, grid=(20, 80, 80)),
+    ]
+    assert (problems[3][3] != 0).any() and bin(int(np.bitwise_or.reduce(problems[3][3]))).count("1") < 27
+    other = tv.Context().create_cuda_stream()
+    for stream in (0, other.cuda_stream_int()):
+        for trip in range(2):
+            for i, (p, dw0, ref, _) in enumerate(problems):
+                p.stream = stream
+                p.weight = H.dev(dw0, dtype)
+                ConvMainUnitTest.implicit_gemm2(p)
+                assert lib.cumm_hip_last_wgrad_path() == 1, "problem %d did not take the one-launch path" % i
+                if stream:
+                    other.synchronize_stream()
+                got = H.as_f32(H.host(p.weight), dtype)
+                assert H.rel_err(got, ref) < TOL, "stream %d trip %d problem %d" % (stream, trip, i)
+
+
+@pytest.mark.parametrize("dtype", ["f16"])
+def test_backward_weight_paths_by_size(dtype):
+    """Which kernels serve a balanced backward-weight call: one launch while a workgroup can hold
+    the reduced masks (4096 words), the three-launch path beyond, the fixed-order variant when
+    asked for; all three against the oracle on the same problem size class."""
+    print("case backward_weight_paths", dtype, flush=True)
+    lib = _capi.lib()
+    p, dw0, ref, red = _wgrad_problem(27, 150000, 64, 64, 32, dtype, grid=(40, 300, 300), clusters=60, sigma=15.0)
+    assert red.shape[0] > 4096
+    p.weight = H.dev(dw0, dtype)
+    ConvMainUnitTest.implicit_gemm2(p)
+    assert lib.cumm_hip_last_wgrad_path() in (2, 4)
+    assert H.rel_err(H.as_f32(H.host(p.weight), dtype), ref) < TOL
+    p, dw0, ref, red = _wgrad_problem(28, 3000, 64, 64, 64, dtype)
+    p.deterministic = True
+    p.weight = H.dev(dw0, dtype)
+    ConvMainUnitTest.implicit_gemm2(p)
+    assert lib.cumm_hip_last_wgrad_path() == 4
+    assert H.rel_err(H.as_f32(H.host(p.weight), dtype), ref) < TOL
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
