@@ -308,74 +308,6 @@ const int32_t *light_hint_no_slot() {
   return first ? first - 8 * light_hint_slot(nullptr) + 8 * kLightHintSlots : nullptr;
 }
 
-// ---- memory of the one-launch backward-weight (wgrad_units_kernel<..., FUSED>): fp32 images of
-// dW and ticket words that must be zero when a launch starts.  The kernel puts the zeros back
-// itself, so the memory has to be the library's own - a caller's workspace may hold anything.
-// One array per GPU, cut into slots; a stream gets a slot at its first call and keeps it (launches
-// of one stream follow one another, so they can share; launches of different streams may overlap,
-// so they cannot).  A stream that finds no slot left, or that is being captured into a graph - a
-// replay could overlap the capturing stream's own launches -, takes the three-launch path.
-constexpr int kWgradOwnSlots = 8;
-constexpr size_t kWgradOwnTicketBytes = 4096;
-constexpr size_t kWgradOwnImageBytes = (size_t)4 << 20;
-constexpr size_t kWgradOwnSlotBytes = kWgradOwnTicketBytes + kWgradOwnImageBytes;
-static __device__ __align__(256) unsigned char wgrad_own[kWgradOwnSlots * kWgradOwnSlotBytes];
-unsigned char *g_wgrad_own_ptr[kMaxDevices] = {};
-hipStream_t g_wgrad_own_stream[kMaxDevices][kWgradOwnSlots] = {};
-int g_wgrad_own_used[kMaxDevices] = {};
-
-unsigned char *wgrad_own_slot(hipStream_t stream) {
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return nullptr;
-  }
-  int dev = -1;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
-  std::lock_guard<std::mutex> guard(g_scratch_lock);
-  if (g_wgrad_own_ptr[dev] == nullptr) {
-    void *ptr = nullptr;
-    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(wgrad_own)) != hipSuccess || ptr == nullptr) {
-      (void)hipGetLastError();
-      return nullptr;
-    }
-    g_wgrad_own_ptr[dev] = reinterpret_cast<unsigned char *>(ptr);
-  }
-  const hipStream_t released = reinterpret_cast<hipStream_t>(~(uintptr_t)0);
-  int slot = 0, spare = -1;
-  for (; slot < g_wgrad_own_used[dev] && g_wgrad_own_stream[dev][slot] != stream; ++slot)
-    if (g_wgrad_own_stream[dev][slot] == released && spare < 0) spare = slot;
-  if (slot == g_wgrad_own_used[dev]) {
-    if (spare >= 0) {
-      slot = spare;
-    } else {
-      if (slot == kWgradOwnSlots) return nullptr;
-      ++g_wgrad_own_used[dev];
-    }
-    g_wgrad_own_stream[dev][slot] = stream;
-  }
-  return g_wgrad_own_ptr[dev] + (size_t)slot * kWgradOwnSlotBytes;
-}
-
-// A stream that goes away gives its slot back - after its work has finished, since the next owner's
-// launches may start at once.  (Streams destroyed by other means keep their slot: eight of those
-// and later streams take the three-launch path.)
-void wgrad_own_release(hipStream_t stream) {
-  int dev = -1;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return;
-  std::lock_guard<std::mutex> guard(g_scratch_lock);
-  for (int slot = 0; slot < g_wgrad_own_used[dev]; ++slot) {
-    if (g_wgrad_own_stream[dev][slot] != stream) continue;
-    if (hipStreamSynchronize(stream) != hipSuccess) {
-      (void)hipGetLastError();
-      return;
-    }
-    // (slots keep their place: another stream may be using a later one)
-    g_wgrad_own_stream[dev][slot] = reinterpret_cast<hipStream_t>(~(uintptr_t)0);
-    return;
-  }
-}
-
 int report_async_errors() {
   int32_t timeouts = 0, sort_give_ups = 0;
   if (int rc = take_async_errors(&timeouts, &sort_give_ups)) return rc;
@@ -920,32 +852,6 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
     w.image_floats = f.image_floats = (int64_t)(image_bytes / sizeof(float));
     // (the unit-walking kernel divides unit numbers with a float reciprocal: exact below 2^22)
     const int64_t unit_bound = ((int64_t)(w.num_red + qt - 1) / qt + 1) * kv * (((int64_t)a->K + 63) / 64) * (((int64_t)a->C + 63) / 64);
-    // One launch where the reduced masks are few enough for a workgroup to count them itself and
-    // the library has memory of its own for this stream (not for the entry point that promises to
-    // use the static workspace only, not for the fixed-order variant: the sums are atomic)
-    {
-      const int kblocks = (a->K + 63) / 64, cblocks = (a->C + 63) / 64;
-      const int64_t keys = (int64_t)kv * kblocks * cblocks;
-      if (!workspace_cap && fits32 && unit_bound < ((int64_t)1 << 22) && w.num_red <= 256 * kWgradFusedWords &&
-          keys * 4 <= (int64_t)kWgradOwnTicketBytes && keys * 16384 <= (int64_t)kWgradOwnImageBytes) {
-        if (unsigned char *own = wgrad_own_slot(stream)) {
-          WgradParams u = w;
-          u.live_cnt = nullptr; u.live_list = nullptr; u.merge_blocks = 0;
-          u.tickets = reinterpret_cast<int32_t *>(own);
-          u.scratch = reinterpret_cast<float *>(own + kWgradOwnTicketBytes);
-          u.image_floats = keys * 4096;
-          int copies = (int)((int64_t)kWgradOwnImageBytes / (keys * 16384));
-          u.images = copies > 8 ? 8 : copies;
-          u.dw = a->ptr_C; u.src = ptr_D; u.alpha = a->alpha; u.beta = a->beta;
-          const hipError_t eu = dt == CUMM_HIP_F16 ? launch_wgrad_fused_f16(u, stream) : launch_wgrad_fused_bf16(u, stream);
-          if (eu == hipSuccess) {
-            g_wgrad_path = CUMM_HIP_WGRAD_ONE_LAUNCH;
-            return CUMM_HIP_OK;
-          }
-          if (eu != hipErrorNotSupported) return hip_fail(eu, "sparse conv wgrad launch");
-        }
-      }
-    }
     if (images && fits32 && unit_bound < ((int64_t)1 << 22) && w.num_red < (1 << 22)) {
       char *base = reinterpret_cast<char *>(workspace);
       const size_t lists_at = images * image_bytes;
@@ -1072,7 +978,6 @@ int cumm_hip_stream_create(void **stream) {
   return CUMM_HIP_OK;
 }
 int cumm_hip_stream_destroy(void *stream) {
-  wgrad_own_release(reinterpret_cast<hipStream_t>(stream));
   HIP_TRY(hipStreamDestroy(reinterpret_cast<hipStream_t>(stream)));
   return CUMM_HIP_OK;
 }

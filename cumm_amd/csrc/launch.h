@@ -56,8 +56,6 @@ hipError_t launch_wgrad_atomic_f16(const WgradParams &p, const WgradPrepareParam
 hipError_t launch_wgrad_atomic_bf16(const WgradParams &p, const WgradPrepareParams &pre, const WgradFinalizeParams &f, hipStream_t s);
 int wgrad_ordered_resident_f16(bool wide);
 int wgrad_ordered_resident_bf16(bool wide);
-hipError_t launch_wgrad_fused_f16(const WgradParams &p, hipStream_t s);
-hipError_t launch_wgrad_fused_bf16(const WgradParams &p, hipStream_t s);
 hipError_t launch_wgrad_ordered_f16(const WgradParams &p, const WgradPrepareParams &pre, const WgradOrderedParams &f, bool wide, int wgs, hipStream_t s);
 hipError_t launch_wgrad_ordered_bf16(const WgradParams &p, const WgradPrepareParams &pre, const WgradOrderedParams &f, bool wide, int wgs, hipStream_t s);
 

@@ -132,39 +132,6 @@ hipError_t CUMM_CAT(launch_wgrad_atomic_, CUMM_NAME)(const WgradParams &p, const
   return hipGetLastError();
 }
 
-// One launch: wgrad_units_kernel<T, 1, 1, 2, false, true> on images and tickets the library owns
-// (p.scratch, p.tickets: zero on entry, zero again on exit).  hipErrorNotSupported when the build's
-// kernel cannot keep its counted waits or the problem is not one for it.
-hipError_t CUMM_CAT(launch_wgrad_fused_, CUMM_NAME)(const WgradParams &p, hipStream_t s) {
-  using T = CUMM_ELEM;
-  const int groups = (p.num_red + p.tiles_per_wg - 1) / p.tiles_per_wg;
-  if (groups == 0 || p.kv == 0) return hipErrorNotSupported;
-  if (p.num_red > 256 * kWgradFusedWords) return hipErrorNotSupported;
-  if (!counted_waits_hold<wgrad_units_kernel<T, 1, 1, 2, false, true>>()) return hipErrorNotSupported;
-  static int resident_of[16] = {};
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  int &resident = resident_of[dev & 15];
-  if (resident == 0) {
-    int cus = 0, per_cu = 0;
-    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e == hipSuccess)
-      e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, wgrad_units_kernel<T, 1, 1, 2, false, true>, 256, 0);
-    if (e != hipSuccess) return e;
-    resident = cus * per_cu > 0 ? cus * per_cu : 1;
-  }
-  const int kblocks = (p.K + 63) / 64, cblocks = (p.C + 63) / 64;
-  const int keys = p.kv * kblocks * cblocks;
-  // never more workgroups than units can exist, never fewer than keys (workgroup `key` writes the
-  // block of a key that has no unit)
-  long long wgs = ((long long)groups * p.kv + p.kv) * kblocks * cblocks;
-  if (wgs > resident) wgs = resident;
-  if (wgs < keys) wgs = keys;
-  hipLaunchKernelGGL((wgrad_units_kernel<T, 1, 1, 2, false, true>), dim3((unsigned)wgs), dim3(256), 0, s, p);
-  return hipGetLastError();
-}
-
 // Fixed-order variant: the same units, a contiguous run per workgroup, partial sums stored into
 // slots and added up in workgroup order.  `max_wgs` = workgroups the caller's slots allow.
 int CUMM_CAT(wgrad_ordered_resident_, CUMM_NAME)(bool wide) {

@@ -60,16 +60,6 @@ struct WgradParams {
   // b + key (key = offset * channel blocks + channel block) of `scratch`; key_range[key] = {first
   // workgroup, number of workgroups} tells wgrad_finalize_ordered_kernel which slots to sum.
   int32_t *key_range;
-  // one-launch variant (wgrad_units_kernel<..., FUSED = true>): no lists, no prepare or finalize kernel.
-  // Every workgroup counts the live tiles per offset from the reduced masks itself and finds its
-  // unit's tiles there; `scratch` is memory the LIBRARY owns - `images` copies of [keys][64 * 64]
-  // floats - and `tickets` [keys] words of the same memory, all of it zero between calls: the
-  // workgroup that draws the last ticket of an (offset, channel block) key sums the copies of its
-  // block, writes dW, and puts zeros and a zero ticket back.
-  int32_t *tickets;
-  void *dw;
-  const void *src;
-  float alpha, beta;
 };
 
 constexpr int kWgradMaxPos = 1024;  // positions one workgroup handles at most (QT * mask_width)
@@ -319,11 +309,8 @@ __device__ __forceinline__ int wave_prefix_sum_dpp(int v) {
 // 64 x 64 block (four gathers of each pair at C = K = 128, where the launch is bound by that
 // traffic once dOut and In no longer fit the last-level cache); its stage holds 32 pairs (16 KB,
 // four stages, still two workgroups per CU) and a wave accumulates 64 x 64.
-constexpr int kWgradFusedWords = 16;   // reduced-mask words a thread holds in the one-launch variant
-
-template <class T, int KB, int CB, int H, bool DET = false, bool FUSED = false>
+template <class T, int KB, int CB, int H, bool DET = false>
 __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
-  static_assert(!FUSED || (KB == 1 && CB == 1 && !DET), "the one-launch variant has 64 x 64 units and atomic sums");
   using E = Elem<T>;
   constexpr int TK = 32 * H;          // pairs per step
   constexpr int NS = 4, L = NS - 1;   // ring stages, steps the loads run ahead
@@ -344,65 +331,13 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   const int l16 = lane & 15, q = lane >> 4;
 
   const int kblocks = (p.K + 64 * KB - 1) / (64 * KB), cblocks = (p.C + 64 * CB - 1) / (64 * CB);
-  const bool merge = !DET && !FUSED && p.merge_blocks;   // (a key of the one-launch variant is one channel block)
-  const int per_r = merge ? 1 : kblocks * cblocks;
-  const int combos = merge ? kblocks * cblocks : 1;
+  const int per_r = (!DET && p.merge_blocks) ? 1 : kblocks * cblocks;
+  const int combos = (!DET && p.merge_blocks) ? kblocks * cblocks : 1;
   // units of offset r: its workgroups (ceil(live / QT)) times the channel blocks.  Lane r of every
   // wave holds offset r's numbers (kv <= 32: one mask bit per offset); a prefix sum over the
   // lanes and a ballot locate a unit without a loop over memory.
-  constexpr int MAXW = FUSED ? kWgradFusedWords : 1;
-  uint32_t words[MAXW];   // FUSED: reduced mask of tile k * 256 + tid, filtered
-  __shared__ int wave_live[FUSED ? 4 : 1][16];
-  __shared__ int tile_cnt[FUSED ? 64 : 1];
-  __shared__ int lds_tiles[FUSED ? 64 : 1];
-  __shared__ int last_flag;
-  int my_live;
-  if constexpr (FUSED) {
-    // ---- live tiles per offset, counted by every workgroup for itself: num_red <= 256 * MAXW
-    // words, MAXW per thread in one round trip.  A thread adds its words bit-sliced (five planes:
-    // bit r of plane j = bit j of the number of its words that have bit r), takes the counts of
-    // two offsets per register out of the planes, a DPP prefix sum adds them over the wave, LDS
-    // over the four waves; lane r ends up with the count of offset r, as the list variant reads it.
-    const v4i rs_red = rsrc_words(p.red_mask, (uint32_t)p.num_red * 4u);
-    int raw[MAXW];
-#pragma unroll
-    for (int k = 0; k < MAXW; ++k)
-      raw[k] = load_b32_hidden(rs_red, k * 256 + tid < p.num_red ? (uint32_t)(k * 256 + tid) * 4u : 0x80000000u);
-    wait_vmcnt<0>();
-#pragma unroll
-    for (int k = 0; k < MAXW; ++k) keep_after_wait(raw[k]);
-    uint32_t b0 = 0, b1 = 0, b2 = 0, b3 = 0, b4 = 0;
-#pragma unroll
-    for (int k = 0; k < MAXW; ++k) {
-      const uint32_t w = (uint32_t)raw[k] & p.mask_filter;
-      words[k] = w;
-      const uint32_t c0 = b0 & w;  b0 ^= w;
-      const uint32_t c1 = b1 & c0; b1 ^= c0;
-      const uint32_t c2 = b2 & c1; b2 ^= c1;
-      const uint32_t c3 = b3 & c2; b3 ^= c2;
-      b4 ^= c3;
-    }
-    int mine = 0;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      // offsets 2j (low half) and 2j + 1 (high half): a thread counts at most 16, a wave 1024
-      const uint32_t x0 = (b0 >> (2 * j)) & 3u, x1 = (b1 >> (2 * j)) & 3u, x2 = (b2 >> (2 * j)) & 3u,
-                     x3 = (b3 >> (2 * j)) & 3u, x4 = (b4 >> (2 * j)) & 3u;
-      const uint32_t lo2 = (x0 & 1u) + 2u * (x1 & 1u) + 4u * (x2 & 1u) + 8u * (x3 & 1u) + 16u * (x4 & 1u);
-      const uint32_t hi2 = (x0 >> 1) + 2u * (x1 >> 1) + 4u * (x2 >> 1) + 8u * (x3 >> 1) + 16u * (x4 >> 1);
-      const int total = __builtin_amdgcn_readlane(wave_prefix_sum_dpp((int)(lo2 | (hi2 << 16))), 63);
-      mine = lane == j ? total : mine;
-    }
-    if (lane < 16) wave_live[wave][lane] = mine;
-    __syncthreads();
-    int sum = 0;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) sum += (wave_live[w][(lane >> 1) & 15] >> (16 * (lane & 1))) & 0xffff;
-    my_live = lane < p.kv ? sum : 0;
-  } else {
-    my_live = lane < p.kv ? p.live_cnt[lane] : 0;
-  }
-  const v4i rs_list = rsrc_words(p.live_list, FUSED ? 0u : (uint32_t)p.kv * (uint32_t)p.num_red * 4u);
+  const int my_live = lane < p.kv ? p.live_cnt[lane] : 0;
+  const v4i rs_list = rsrc_words(p.live_list, (uint32_t)p.kv * (uint32_t)p.num_red * 4u);
   const v4i rs_sort = rsrc_words(p.argsort, (uint32_t)p.n_pos * 4u);
   const v4i rs_idx = rsrc_words(p.indices, (uint32_t)p.kv * (uint32_t)p.n_idx * 4u);
   const v4i y_rsrc = rsrc_words(p.dout, (uint32_t)p.rows_y * (uint32_t)p.K * 2u);
@@ -450,34 +385,6 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
   const int my_units = my_wgs * per_r;
   const int incl = wave_prefix_sum_dpp(my_units);
   const int total_units = __builtin_amdgcn_readlane(incl, 31);
-  if constexpr (FUSED) {
-    // an (offset, channel block) key without a live tile has no unit to write its block of dW:
-    // workgroup `key` does it here (alpha * 0 + beta * source); keys whose offset is filtered out
-    // are left alone, as by the finalize kernel of the list variant
-    const int key = (int)blockIdx.x;
-    if (key < p.kv * per_r) {
-      const int r = key / per_r, combo = key - r * per_r;
-      const int kb = combo / cblocks, cb = combo - kb * cblocks;
-      if (((p.mask_filter >> r) & 1u) && __builtin_amdgcn_readlane(my_live, r) == 0) {
-        typedef uint16_t v4h __attribute__((ext_vector_type(4)));
-        const int row = tid >> 2, mm = kb * 64 + row;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int nn = cb * 64 + (tid & 3) * 16 + c * 4;
-          if (mm < p.K && nn < p.C) {
-            const int64_t at = ((int64_t)mm * p.kv + r) * p.C + nn;
-            v4h out = v4h{0, 0, 0, 0};
-            if (p.beta != 0.0f) {
-              const v4h src = *reinterpret_cast<const v4h *>(reinterpret_cast<const uint16_t *>(p.src) + at);
-#pragma unroll
-              for (int x = 0; x < 4; ++x) out[x] = E::from_float(p.beta * E::to_float(src[x]));
-            }
-            *reinterpret_cast<v4h *>(reinterpret_cast<uint16_t *>(p.dw) + at) = out;
-          }
-        }
-      }
-    }
-  }
 
   // fixed-order variant: a contiguous run of units per workgroup, and the table of the workgroups
   // that hold a partial sum of each (offset, channel block)
@@ -554,36 +461,6 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     // through the descriptor and is sorted out with a select) and waited for once: as
     // conditional C++ loads every one of the twelve got a branch and a wait of its own.
     int t_[MAXIT], o_[MAXIT], i_[MAXIT], within[MAXIT];
-    if constexpr (FUSED) {
-      // the live tiles lo .. lo + n_list - 1 of offset r, in tile order = (k, wave, lane): ballots
-      // per word index, their counts through LDS, one prefix sum over the 64 (k, wave) counts
-      uint64_t lb[MAXW];
-      int cnt = 0;
-#pragma unroll
-      for (int k = 0; k < MAXW; ++k) {
-        lb[k] = __ballot((words[k] >> r) & 1u);
-        cnt = lane == k ? __builtin_popcountll(lb[k]) : cnt;
-      }
-      if (lane < MAXW) tile_cnt[lane * 4 + wave] = cnt;
-      __syncthreads();
-      const int v = tile_cnt[lane];
-      const int before = wave_prefix_sum_dpp(v) - v;
-#pragma unroll
-      for (int k = 0; k < MAXW; ++k) {
-        const int rank = __builtin_amdgcn_readlane(before, k * 4 + wave) +
-                         __builtin_popcountll(lb[k] & ((1ull << lane) - 1ull)) - lo;
-        if (((words[k] >> r) & 1u) && rank >= 0 && rank < n_list) lds_tiles[rank] = k * 256 + tid;
-      }
-      __syncthreads();
-#pragma unroll
-      for (int k = 0; k < MAXIT; ++k) {
-        const int s = k * 256 + tid;
-        const int ti = fast_div(s, mw);
-        within[k] = s - ti * mw;
-        t_[k] = s < n_slots ? lds_tiles[ti] : 0;
-      }
-      wait_vmcnt<0>();   // the previous unit's atomics
-    } else {
 #pragma unroll
     for (int k = 0; k < MAXIT; ++k) {
       const int s = k * 256 + tid;
@@ -594,7 +471,6 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     wait_vmcnt<0>();   // (also the previous unit's atomics)
 #pragma unroll
     for (int k = 0; k < MAXIT; ++k) keep_after_wait(t_[k]);
-    }
     bool have[MAXIT];
 #pragma unroll
     for (int k = 0; k < MAXIT; ++k) {
@@ -664,7 +540,7 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     // landed, everybody is done with step s-1), reads its operands, refills the stage of step
     // s-1 with step s+NS-1, computes.
     for (int combo = 0; combo < combos; ++combo) {
-    if (merge) {
+    if (p.merge_blocks) {
       kb = fast_div(combo, cblocks);
       cb = combo - kb * cblocks;
     }
@@ -753,77 +629,7 @@ __global__ __launch_bounds__(256) void wgrad_units_kernel(const WgradParams p) {
     // consecutive floats (one 64-byte segment per quarter).  Units that follow each other go to
     // different images, so that the many units of one offset do not all queue on the same
     // addresses.
-    if (FUSED && n_steps > 0) {
-      // the library's own images: [copy][key][64 x 64]
-      float *block = p.scratch + (int64_t)(unit % p.images) * p.image_floats + (int64_t)(r * per_r + kb * cblocks + cb) * 4096;
-#pragma unroll
-      for (int i = 0; i < NJ; ++i) {
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-          const int nl = (wn * NI + j) * 16 + l16;
-          if (cb * 64 + nl >= p.C) continue;
-#pragma unroll
-          for (int x = 0; x < 4; ++x) {
-            const int ml = (wm * NJ + i) * 16 + 4 * q + x;
-            if (kb * 64 + ml < p.K)
-              __hip_atomic_fetch_add(block + ml * 64 + nl, acc[i][j][x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-        }
-      }
-    }
-    if constexpr (FUSED) {
-      // ---- ticket of the key: who draws the last one of its n_wg finds every unit's sums in
-      // the images (each workgroup waits for its atomics before it draws), adds the copies,
-      // writes dW and leaves zeros and a zero ticket behind for the next call
-      const int key = r * per_r + kb * cblocks + cb;
-      wait_vmcnt<0>();
-      __syncthreads();
-      if (tid == 0) {
-        const int t = __hip_atomic_fetch_add(p.tickets + key, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        last_flag = t == n_wg - 1;
-      }
-      __syncthreads();
-      if (last_flag) {
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // (every wave: the images were written by other workgroups)
-        typedef uint16_t v4h __attribute__((ext_vector_type(4)));
-        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            p.scratch, 0, (int)((uint32_t)p.images * (uint32_t)p.image_floats * 4u), 0x00020000);
-        const int row = tid >> 2, mm = kb * 64 + row;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int nl = (tid & 3) * 16 + c * 4, nn = cb * 64 + nl;
-          const uint32_t at = (uint32_t)(key * 4096 + row * 64 + nl) * 4u;
-          v4f part[8];
-#pragma unroll
-          for (int g = 0; g < 8; ++g)
-            part[g] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
-                rs, g < p.images ? (uint32_t)((int64_t)g * p.image_floats * 4) + at : 0x80000000u, 0, 0));
-          v4f sum = part[0];
-#pragma unroll
-          for (int g = 1; g < 8; ++g) sum += part[g];
-#pragma unroll
-          for (int g = 0; g < 8; ++g)
-            if (g < p.images)
-              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v4f{0, 0, 0, 0}), rs,
-                                                     (uint32_t)((int64_t)g * p.image_floats * 4) + at, 0, 0);
-          if (mm < p.K && nn < p.C) {
-            const int64_t dst = ((int64_t)mm * p.kv + r) * p.C + nn;
-            v4h out;
-            if (p.beta != 0.0f) {
-              const v4h src = *reinterpret_cast<const v4h *>(reinterpret_cast<const uint16_t *>(p.src) + dst);
-#pragma unroll
-              for (int x = 0; x < 4; ++x) out[x] = E::from_float(__builtin_fmaf(p.alpha, sum[x], p.beta * E::to_float(src[x])));
-            } else {
-#pragma unroll
-              for (int x = 0; x < 4; ++x) out[x] = E::from_float(p.alpha * sum[x]);
-            }
-            *reinterpret_cast<v4h *>(reinterpret_cast<uint16_t *>(p.dw) + dst) = out;
-          }
-        }
-        if (tid == 0) __hip_atomic_store(p.tickets + key, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    if (!FUSED && !DET && n_steps > 0) {
+    if (!DET && n_steps > 0) {
       const int64_t ldn = (int64_t)p.kv * p.C;
       float *image = p.scratch + (int64_t)(unit % p.images) * p.image_floats;
 #pragma unroll

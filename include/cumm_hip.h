@@ -210,11 +210,9 @@ const char *cumm_hip_last_error(void);
 
 /* Which kernels served the calling thread's last successful backward-weight call (a diagnostic for
  * tests, benchmarks and the tuner; no counterpart in the reference, whose descriptor names its one
- * kernel).  ONE_LAUNCH: balanced units on fp32 images the library owns, sums and conversion in the
- * same launch; LISTS: live-tile lists + balanced units + conversion, three launches on the caller's
+ * kernel).  LISTS: live-tile lists + balanced units + conversion, three launches on the caller's
  * workspace; SCAN: the (groups, offsets) grid that reads the reduced masks itself + conversion;
  * FIXED_ORDER: the reproducible variant; TILED: the tile GEMM (one slice or serial split-K). */
-#define CUMM_HIP_WGRAD_ONE_LAUNCH 1
 #define CUMM_HIP_WGRAD_LISTS 2
 #define CUMM_HIP_WGRAD_SCAN 3
 #define CUMM_HIP_WGRAD_FIXED_ORDER 4
