@@ -37,8 +37,13 @@ constexpr int kRadixBits = 9;
 constexpr int kBins = 1 << kRadixBits;            // 512
 constexpr int kSortThreads = 512;                 // one bin per thread
 constexpr int kSortWaves = kSortThreads / 64;     // 8
-constexpr int kItems = 8;                         // keys per lane
-constexpr int kChunk = kSortThreads * kItems;     // 4096 keys per workgroup
+constexpr int kItems = 8;                         // keys per lane: 4096 keys per workgroup of a pass ...
+// ... and half of that for inputs of up to kSmallInput keys, where the chunks are few and a pass is
+// as long as one chunk's chain of round trips (120 k keys: 62.7 us with 59 chunks of 2048 against
+// 70.8 us with 30 of 4096; at 1 M keys the larger chunks win, 131 against 152 us)
+constexpr int kSmallItems = 4;
+constexpr int kSmallInput = 1 << 18;
+inline int pass_items(int n) { return n <= kSmallInput ? kSmallItems : kItems; }
 constexpr uint32_t kFlagAggregate = 1u << 30, kFlagInclusive = 2u << 30, kValueMask = (1u << 30) - 1u;
 constexpr int kLookbackSpins = 1 << 20;   // (about a second)
 
@@ -136,7 +141,9 @@ __global__ __launch_bounds__(256) void sort_clear_hist_kernel(uint32_t *hist, in
   if (i < words) hist[i] = 0u;
 }
 
+template <int ITEMS>
 __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParams p) {
+  constexpr int kChunk = kSortThreads * ITEMS;
   __shared__ uint32_t wave_hist[kSortWaves][kBins];   // per wave: keys per digit, then the prefix over waves
   __shared__ uint32_t bin_base[kBins];                // where this chunk's keys of a digit go
   __shared__ uint32_t scan_tmp[kBins];
@@ -196,7 +203,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
 
   if (copy_through) {
 #pragma unroll
-    for (int u = 0; u < kItems; ++u) {
+    for (int u = 0; u < ITEMS; ++u) {
       const int64_t pos = (int64_t)chunk * kChunk + u * kSortThreads + t;
       if (pos < p.n) {
         dst_keys[pos] = p.mask[pos] & p.filter;      // (nothing moves: the masks themselves)
@@ -206,14 +213,14 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
     return;
   }
 
-  // ---- keys of this chunk, wave-striped: wave w owns positions [base_w, base_w + 64 * kItems),
+  // ---- keys of this chunk, wave-striped: wave w owns positions [base_w, base_w + 64 * ITEMS),
   // item u of lane l is position base_w + u * 64 + l, i.e. position order = (u, l)
-  const int64_t base_w = (int64_t)chunk * kChunk + (int64_t)wave * (64 * kItems);
-  uint32_t key[kItems];
-  int32_t val[kItems];
-  uint32_t rank[kItems];   // offset among this wave's keys of the same digit
+  const int64_t base_w = (int64_t)chunk * kChunk + (int64_t)wave * (64 * ITEMS);
+  uint32_t key[ITEMS];
+  int32_t val[ITEMS];
+  uint32_t rank[ITEMS];   // offset among this wave's keys of the same digit
 #pragma unroll
-  for (int u = 0; u < kItems; ++u) {
+  for (int u = 0; u < ITEMS; ++u) {
     const int64_t pos = base_w + u * 64 + lane;
     const bool valid = pos < p.n;
     if (first) {
@@ -225,7 +232,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
     }
   }
 #pragma unroll
-  for (int u = 0; u < kItems; ++u) {
+  for (int u = 0; u < ITEMS; ++u) {
     const int64_t pos = base_w + u * 64 + lane;
     const bool valid = pos < p.n;
     const uint32_t d = (key[u] >> shift) & (kBins - 1);
@@ -304,7 +311,7 @@ __global__ __launch_bounds__(kSortThreads) void sort_pass_kernel(const SortParam
 
   // ---- scatter
 #pragma unroll
-  for (int u = 0; u < kItems; ++u) {
+  for (int u = 0; u < ITEMS; ++u) {
     const int64_t pos = base_w + u * 64 + lane;
     if (pos < p.n) {
       const uint32_t d = (key[u] >> shift) & (kBins - 1);
@@ -409,7 +416,11 @@ int sort_passes(uint32_t filter) {
 // keys + values of the intermediate order, histograms, tickets, look-back state
 size_t sort_by_mask_workspace_bytes(int n) {
   const size_t nn = (size_t)(n > 0 ? n : 1);
-  const size_t chunks = (nn + kChunk - 1) / kChunk;
+  const size_t chunk = (size_t)kSortThreads * pass_items((int)nn);
+  size_t chunks = (nn + chunk - 1) / chunk;
+  // (never less than a smaller input asks for: a workspace sized for a larger one must do)
+  const size_t small_most = ((size_t)kSmallInput + kSortThreads * kSmallItems - 1) / (kSortThreads * kSmallItems);
+  if (nn > (size_t)kSmallInput && chunks < small_most) chunks = small_most;
   return 2 * align256s(4 * nn) + align256s(4 * 4 * kBins) + 256 + align256s(4 * 4 * chunks * kBins);
 }
 
@@ -421,7 +432,8 @@ hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uin
   const size_t words = align256s(4 * (size_t)n);
   SortParams p;
   p.mask = mask; p.filter = filter; p.n = n;
-  p.chunks = (n + kChunk - 1) / kChunk;
+  const int items = pass_items(n), chunk = kSortThreads * items;
+  p.chunks = (n + chunk - 1) / chunk;
   p.count_major = order != 0;
   p.passes = p.count_major ? 4 : sort_passes(filter);
   p.out_keys = sorted; p.out_vals = argsort;
@@ -434,12 +446,16 @@ hipError_t launch_sort_by_mask(const uint32_t *mask, int n, uint32_t filter, uin
   p.hint_slot = hint_slot;
   p.pass = 0;
   hipLaunchKernelGGL(sort_clear_hist_kernel, dim3((4 * kBins + 255) / 256), dim3(256), 0, s, p.hist, 4 * kBins);
-  int setup_blocks = p.chunks < 512 ? p.chunks : 512;
+  // (two keys per lane where that still leaves fewer workgroups than the device holds: with one
+  // workgroup per chunk the 120 k keys of a small input sat on 30 or 59 of the 256 CUs)
+  int setup_blocks = (n + 2 * kSortThreads - 1) / (2 * kSortThreads);
+  if (setup_blocks > 512) setup_blocks = 512;
   hipLaunchKernelGGL(sort_setup_kernel, dim3(setup_blocks), dim3(kSortThreads), 0, s, p);
   for (int q = 0; q < p.passes; ++q) {
     SortParams r = p;
     r.pass = q;
-    hipLaunchKernelGGL(sort_pass_kernel, dim3(p.chunks), dim3(kSortThreads), 0, s, r);
+    if (items == kSmallItems) hipLaunchKernelGGL(sort_pass_kernel<kSmallItems>, dim3(p.chunks), dim3(kSortThreads), 0, s, r);
+    else hipLaunchKernelGGL(sort_pass_kernel<kItems>, dim3(p.chunks), dim3(kSortThreads), 0, s, r);
   }
   hipLaunchKernelGGL(sort_finish_kernel, dim3((n + 511) / 512), dim3(256), 0, s, p);
   return hipGetLastError();
