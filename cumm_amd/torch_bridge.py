@@ -84,14 +84,15 @@ _TUNER = tuner.Tuner(steps=3, warmup=1)
 _DESP_LIKE = {}
 
 
-def _desp_like(dtype, op, parallel=False):
+def _desp_like(dtype, op, parallel=False, dynamic=False):
     """A descriptor of the wanted kind (the tuner then picks the tile); looked up once per kind:
-    building the table of all descriptors costs more than a forward launch."""
-    key = (dtype, op, parallel)
+    building the table of all descriptors costs more than a forward launch.  ``dynamic``: several
+    mask words per position (kernel volumes above 32)."""
+    key = (dtype, op, parallel, dynamic)
     if key not in _DESP_LIKE:
         for d in ConvMainUnitTest.get_all_conv_algo_desp():
             if (d.dtype_a == dtype and d.dtype_c == dtype and ConvOpType(d.op_type) == op and not d.is_int8_inference and
-                    bool(d.split_k_parallel) == parallel and d.mask_sparse and not d.dynamic_mask):
+                    bool(d.split_k_parallel) == parallel and d.mask_sparse and bool(d.dynamic_mask) == dynamic):
                 _DESP_LIKE[key] = d
                 break
         else:
@@ -142,7 +143,10 @@ class _Launch:
 
 class SparseConvGeometry:
     """Pair tables, masks and sorts of one convolution geometry, built on the GPU once and shared by
-    every layer (and every pass) that uses it."""
+    every layer (and every pass) that uses it.  Kernel volumes up to 32 have one mask word per
+    position; above that (up to 128, e.g. 5 x 5 x 5) the masks have ``ceil(kv / 32)`` words, forward
+    and backward-input run on the ``dynamic_mask`` descriptors, and backward-weight - which has no
+    such kernel, in the reference neither - goes offset by offset over the pair lists."""
 
     def __init__(self, coords: torch.Tensor, spatial_shape: Sequence[int], ksize=(3, 3, 3), stride=None,
                  padding=(1, 1, 1), dilation=(1, 1, 1), batch_size: int = 1):
@@ -163,6 +167,25 @@ class SparseConvGeometry:
             self.out_coords, self.out_shape = tensor2torch(t.out_coords, clone=False), t.out_shape
         self.indices_fwd, self.indices_bwd = t.indices_fwd, t.indices_bwd
         self.n_out = int(t.indices_fwd.dim(1))
+        self.words = (self.kv + 31) // 32
+        self.lists = None
+        if self.kv > 32:
+            # the builders give no masks for these volumes: made from the tables, sorted by offset
+            # count and word pattern; the per-offset lists serve backward-weight
+            mf = pairs.masks_from_pairs_device(t.indices_fwd, stream=stream)
+            self.mask_fwd, self.order_fwd = pairs.sort_by_mask_words_device(mf, stream=stream)
+            if self.subm:
+                self.mask_bwd, self.order_bwd = self.mask_fwd, self.order_fwd
+            else:
+                mb = pairs.masks_from_pairs_device(t.indices_bwd, stream=stream)
+                self.mask_bwd, self.order_bwd = pairs.sort_by_mask_words_device(mb, stream=stream)
+            self.lists = pairs.pair_lists_device(t.indices_fwd, stream=stream)
+            self.light_fwd = self.light_bwd = 0
+            self.indices_fwd_pos = pairs.pairs_by_position_device(self.indices_fwd, self.order_fwd, stream=stream)
+            self.indices_bwd_pos = pairs.pairs_by_position_device(self.indices_bwd, self.order_bwd, stream=stream)
+            self._reduced = {}
+            self._launches = {}
+            return
         # (a mask has one bit per kernel offset: a filter of that width spares the sort the passes over
         # the bits above it)
         bits = (1 << self.kv) - 1 if self.kv < 32 else 0xFFFFFFFF
@@ -224,10 +247,11 @@ class _SparseConvFunction(torch.autograd.Function):
             ctx.save_for_backward(features, weight, out if relu else None)
             return out
         p = ConvParams(3, ConvOpType.Forward)
-        p.conv_algo_desp = _desp_like(dtype, ConvOpType.Forward)
+        p.conv_algo_desp = _desp_like(dtype, ConvOpType.Forward, dynamic=geometry.words > 1)
         p.input, p.weight, p.output = torch2tensor(features), torch2tensor(weight), torch2tensor(out)
         p.indices, p.mask, p.mask_argsort = geometry.indices_fwd_pos, geometry.mask_fwd, geometry.order_fwd
         p.indices_by_position = True
+        p.mask_int_count = geometry.words
         p.light_prefix = geometry.light_fwd
         if bias is not None:
             p.bias, p.beta = torch2tensor(bias), 1.0
@@ -236,8 +260,10 @@ class _SparseConvFunction(torch.autograd.Function):
         p.stream = current_stream()
         _TUNER.tune_conv(p)
         # the tile masks the forward launch computes anyway are what backward-weight needs
+        # (not for several mask words: that backward-weight walks the pair lists)
         tile_m = int(p.conv_algo_desp.tile_shape[0])
-        p.mask_output = geometry.reduced_mask_buffer(tile_m)
+        if geometry.words == 1:
+            p.mask_output = geometry.reduced_mask_buffer(tile_m)
         ConvMainUnitTest.implicit_gemm2(p)
         roles = {"input": features, "weight": weight, "output": out}
         if bias is not None:
@@ -270,17 +296,25 @@ class _SparseConvFunction(torch.autograd.Function):
                 launch(stream, input=grad_in, weight=weight, output=grad_out)
             else:
                 p = ConvParams(3, ConvOpType.BackwardInput)
-                p.conv_algo_desp = _desp_like(dtype, ConvOpType.BackwardInput)
+                p.conv_algo_desp = _desp_like(dtype, ConvOpType.BackwardInput, dynamic=g.words > 1)
                 p.input, p.weight, p.output = torch2tensor(grad_in), torch2tensor(weight), torch2tensor(grad_out)
                 p.indices, p.mask, p.mask_argsort = g.indices_bwd_pos, g.mask_bwd, g.order_bwd
                 p.indices_by_position = True
+                p.mask_int_count = g.words
                 p.reverse_mask = g.subm
                 p.light_prefix = g.light_bwd
                 p.stream = stream
                 _TUNER.tune_conv(p)
                 ConvMainUnitTest.implicit_gemm2(p)
                 g._launches[key] = _Launch(p, {"input": grad_in, "weight": weight, "output": grad_out})
-        if ctx.needs_input_grad[1]:
+        if ctx.needs_input_grad[1] and g.words > 1:
+            # no mask kernel for this pass: one gathered GEMM per kernel offset, straight into its
+            # slice of the gradient (an offset without pairs writes zeros)
+            from .conv import native
+            grad_w = torch.empty_like(weight)
+            native.backward_weight(torch2tensor(grad_out), torch2tensor(features), torch2tensor(grad_w), g.lists,
+                                   stream=stream)
+        elif ctx.needs_input_grad[1]:
             grad_w = torch.empty_like(weight)
             # torch's switch for reproducible results selects the fixed-order sum of the partial blocks
             deterministic = bool(torch.are_deterministic_algorithms_enabled())

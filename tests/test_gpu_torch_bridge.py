@@ -113,6 +113,52 @@ def test_autograd_matches_torch_indexing(dtype, strided):
         tb.sparse_conv(f_d, w_d[:, :26], b_d, geo, relu=True)
 
 
+@pytest.mark.parametrize("case", ["subm555", "strided335"])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_autograd_with_kernel_volumes_above_32(dtype, case):
+    """5 x 5 x 5 submanifold and strided 3 x 3 x 5 layers through the bridge: masks of several words
+    made and sorted on the GPU, forward and backward-input on the dynamic_mask descriptors (one
+    launch each), backward-weight offset by offset over the pair lists; outputs and all three
+    gradients against the convolution written with torch indexing in fp32."""
+    from cumm_amd import torch_bridge as tb
+    print("case torch bridge large kernel", dtype, case, flush=True)
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    coords, grid = H.small_cloud(31, 1500, grid=(12, 30, 28))
+    if case == "subm555":
+        ksize, stride, padding = (5, 5, 5), None, (2, 2, 2)
+        host = pairs.subm_pairs(coords, grid, ksize)
+    else:
+        ksize, stride, padding = (3, 3, 5), (2, 2, 2), (1, 1, 2)
+        host = pairs.sparse_conv_pairs(coords, grid, ksize, stride, padding)
+    kv = ksize[0] * ksize[1] * ksize[2]
+    geo = tb.SparseConvGeometry(torch.as_tensor(coords, device="cuda"), grid, ksize=ksize, stride=stride, padding=padding)
+    assert geo.words == (kv + 31) // 32 and geo.kv == kv
+    np.testing.assert_array_equal(H.host(geo.indices_fwd), host.indices_fwd)
+    c_in, k_out = 64, 64
+    torch.manual_seed(5)
+
+    def rel(a, b):
+        return float((a.float().cpu() - b).abs().max() / b.abs().max().clamp_min(1e-6))
+
+    for trip in range(2):
+        feat = torch.randn(coords.shape[0], c_in).to(tdt)
+        weight = (torch.randn(k_out, kv, c_in) * 0.03).to(tdt)
+        bias = (torch.randn(k_out) * 0.1).to(tdt)
+        gout = torch.randn(geo.n_out, k_out).to(tdt)
+        f_d, w_d, b_d = (t.cuda().requires_grad_(True) for t in (feat, weight, bias))
+        out = tb.sparse_conv(f_d, w_d, b_d, geo, relu=True)
+        out.backward(gout.cuda())
+        f_r, w_r, b_r = (t.float().requires_grad_(True) for t in (feat, weight, bias))
+        ref = _reference(f_r, w_r, b_r, host.indices_fwd, relu=True)
+        gate = (out.detach().float().cpu() > 0).float()
+        pre = _reference(f_r, w_r, b_r, host.indices_fwd, relu=False)
+        (pre * gate * gout.float()).sum().backward()
+        assert rel(out.detach(), ref.detach()) < 1e-2, trip
+        assert rel(f_d.grad, f_r.grad) < 1e-2, trip
+        assert rel(w_d.grad, w_r.grad) < 1e-2, trip
+        assert rel(b_d.grad, b_r.grad) < 1e-2, trip
+
+
 def test_module_stack_runs_and_trains_a_step():
     from cumm_amd import torch_bridge as tb
     coords, grid = H.small_cloud(22, 3000)
