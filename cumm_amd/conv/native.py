@@ -167,6 +167,80 @@ def backward_input(dout: tv.Tensor, weight: tv.Tensor, dinp: tv.Tensor, lists, *
 _NO_PAIR = {}
 
 
+class _WeightPlan:
+    """The per-offset launches of backward-weight, validated once (the first run goes through the
+    operator's prelude, a hundred microseconds of Python per offset) and then replayed straight at
+    the C entry point - on the same tensors, or on others of the same shapes and types whose
+    addresses ``rebind`` writes into the argument blocks."""
+
+    def __init__(self, steps, dout, inp, dweight):
+        self.steps = steps
+        self._tensors = (dout, inp, dweight)     # kept alive with the blocks that point at them
+        self._blocks = None
+
+    def __call__(self) -> None:
+        for p in self.steps:
+            GemmMainUnitTest.matmul2(p)
+        if self._blocks is None:
+            base = self._tensors[2].byte_pointer()
+            self._blocks = []
+            for p in self.steps:
+                prep = p.__dict__.get("_prepared")
+                if prep is None:
+                    raise RuntimeError("the operator call left no validated argument block")
+                args = prep[5]
+                self._blocks.append((prep[1], prep[2], prep[3], args, int(args.ptr_C) - base, int(args.ptr_D or 0) - base))
+
+    def rebind(self, dout_ptr: int, inp_ptr: int, dweight_ptr: int, stream: int) -> None:
+        """Run on other tensors of the same shapes (device addresses), on ``stream``."""
+        if self._blocks is None:
+            raise RuntimeError("the plan has not run yet")
+        for fn, cdesc_ref, args_ref, args, c_delta, d_delta in self._blocks:
+            args.ptr_A, args.ptr_B = dout_ptr, inp_ptr
+            args.ptr_C = dweight_ptr + c_delta
+            if args.ptr_D:
+                args.ptr_D = dweight_ptr + d_delta
+            status = fn(cdesc_ref, args_ref, stream)
+            if status:
+                _capi.check(status)
+
+    def release(self) -> None:
+        """Forget the tensors of the first run (a caller that goes on through ``rebind`` with its
+        own): the argument blocks hold addresses only, the pair lists belong to their owner."""
+        if self._blocks is None:
+            raise RuntimeError("the plan has not run yet")
+        self.steps, self._tensors = [], None
+
+    @property
+    def launches(self) -> int:
+        return len(self._blocks) if self._blocks is not None else len(self.steps)
+
+
+def plan_backward_weight(dout: tv.Tensor, inp: tv.Tensor, dweight: tv.Tensor, lists, *, stream: int = 0) -> _WeightPlan:
+    """Backward-weight as a reusable plan: one gathered GEMM per kernel offset into its slice of
+    ``dweight`` [K, kv, C] (an offset without pairs writes zeros)."""
+    kv = _check(inp, dweight, lists, dout.dim(0))
+    if dout.dim(1) != dweight.dim(0) or dout.dtype != inp.dtype:
+        raise RuntimeError("error")
+    steps = []
+    for k in range(kv):
+        cnt = int(lists.counts[k])
+        p = GemmParams()
+        p.algo_desp = _find(inp.dtype, inp.dtype, ShuffleStrideType.ShuffleAB, 64, 64, True, False).copy()
+        p.a, p.b, p.c = dout, inp, dweight.select(1, k)
+        if cnt > 0:
+            p.a_inds = lists.pair_out.select(0, k).slice_first_axis(0, cnt)
+            p.b_inds = lists.pair_in.select(0, k).slice_first_axis(0, cnt)
+        else:
+            dev = inp.device
+            if dev not in _NO_PAIR:
+                _NO_PAIR[dev] = tv.from_numpy(np.full(32, -1, np.int32)).cuda()
+            p.a_inds = p.b_inds = _NO_PAIR[dev]
+        p.stream = stream
+        steps.append(p)
+    return _WeightPlan(steps, dout, inp, dweight)
+
+
 def backward_weight(dout: tv.Tensor, inp: tv.Tensor, dweight: tv.Tensor, lists, *, split_k_slices: int = 1,
                     stream: int = 0, workspace: Optional[tv.Tensor] = None) -> None:
     """dweight[:, k, :] = dout[pair_out[k]].T @ inp[pair_in[k]] for every offset (zero without pairs)."""

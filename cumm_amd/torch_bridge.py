@@ -312,8 +312,16 @@ class _SparseConvFunction(torch.autograd.Function):
             # slice of the gradient (an offset without pairs writes zeros)
             from .conv import native
             grad_w = torch.empty_like(weight)
-            native.backward_weight(torch2tensor(grad_out), torch2tensor(features), torch2tensor(grad_w), g.lists,
-                                   stream=stream)
+            key = ("wgrad_per_offset", dtype, tuple(weight.shape), tuple(features.shape), tuple(grad_out.shape))
+            plan = g._launches.get(key)
+            if plan is None:      # validated once (the prelude costs 0.1 ms of Python per offset), replayed after
+                plan = native.plan_backward_weight(torch2tensor(grad_out), torch2tensor(features), torch2tensor(grad_w),
+                                                   g.lists, stream=stream)
+                plan()
+                plan.release()      # (later calls bring their own tensors)
+                g._launches[key] = plan
+            else:
+                plan.rebind(grad_out.data_ptr(), features.data_ptr(), grad_w.data_ptr(), stream)
         elif ctx.needs_input_grad[1]:
             grad_w = torch.empty_like(weight)
             # torch's switch for reproducible results selects the fixed-order sum of the partial blocks

@@ -266,3 +266,36 @@ def test_plan_runs_again_on_new_contents():
         plan()
         ref = native_ref.native_fwd_ref(feat, weight, lists_h.pair_in, lists_h.pair_out, lists_h.counts, n, dtype="f16")
         assert H.rel_err(H.host(out).astype(np.float32), ref.astype(np.float32)) < TOL
+
+
+def test_backward_weight_plan_replays_on_other_tensors():
+    """The backward-weight plan validates its per-offset launches once; ``rebind`` then runs them
+    on other tensors of the same shapes by address (what the torch bridge does every iteration),
+    also after the plan has let go of the first run's tensors."""
+    rng = np.random.default_rng(66)
+    grid = (8, 10, 10)
+    coords = synth.clustered_voxels(rng, 300, grid, 3, sigma=2.5)
+    c_in, k_out = 16, 24
+    host = pairs.subm_pairs(coords, grid, ksize=(5, 5, 5))
+    devt = pairs.subm_pairs_device(H.dev(coords, "i32"), grid, ksize=(5, 5, 5))
+    lists_h, lists_d = pairs.pair_lists(host.indices_fwd), pairs.pair_lists_device(devt.indices_fwd)
+    n = coords.shape[0]
+
+    def data(seed):
+        r = np.random.default_rng(seed)
+        return (r.normal(0, 1, size=(n, k_out)).astype(np.float16), r.normal(0, 1, size=(n, c_in)).astype(np.float16))
+
+    dout, feat = data(1)
+    d_dout, d_feat, d_dw = H.dev(dout, "f16"), H.dev(feat, "f16"), tv.zeros([k_out, 125, c_in], tv.float16, 0)
+    plan = native.plan_backward_weight(d_dout, d_feat, d_dw, lists_d)
+    plan()
+    assert plan.launches == 125
+    ref = native_ref.native_wgrad_ref(dout, feat, lists_h.pair_in, lists_h.pair_out, lists_h.counts, 125, dtype="f16")
+    assert H.rel_err(H.host(d_dw).astype(np.float32), ref.astype(np.float32)) < TOL
+    plan.release()
+    dout2, feat2 = data(2)
+    e_dout, e_feat = H.dev(dout2, "f16"), H.dev(feat2, "f16")
+    e_dw = H.dev(np.full((k_out, 125, c_in), 7.0, np.float16), "f16")     # every slice is written, also those without pairs
+    plan.rebind(e_dout.byte_pointer(), e_feat.byte_pointer(), e_dw.byte_pointer(), 0)
+    ref2 = native_ref.native_wgrad_ref(dout2, feat2, lists_h.pair_in, lists_h.pair_out, lists_h.counts, 125, dtype="f16")
+    assert H.rel_err(H.host(e_dw).astype(np.float32), ref2.astype(np.float32)) < TOL
