@@ -730,6 +730,7 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
         (int64_t)kv * a->N * 4 >= (int64_t)1 << 31)
       return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
     p.gather_bytes = (uint32_t)((int64_t)kv * a->N * 4);
+    p.stream_stores = p.c_bytes <= kStreamStoreMaxBytes;
     hipError_t e = launch_rowgemm(dt, wide, d.tile_shape[0], d.tile_shape[1], pick_ks(p.c_in, dt), !fwd, p, stream);
     if (e != hipSuccess) return hip_fail(e, "sparse conv launch");
     return CUMM_HIP_OK;

@@ -75,11 +75,36 @@ struct RowGemmParams {
   // rows are gated by their pair-table entry alone, cumm/conv/sparse_iters.py:629-631), instead of
   // only in the offsets whose bit its own mask word has
   int32_t ungated_rows;
+  // non-zero: the output rows are stored with the non-temporal hint (see kStreamStore)
+  int32_t stream_stores;
 };
 
 // An offset no buffer contains: every operand is smaller than 2 GiB (checked on the host), and
 // adding a scalar offset below 2 GiB to it cannot wrap back into range.
 constexpr uint32_t kOob = 0x80000000u;
+
+// Cache policy of the output stores when RowGemmParams::stream_stores is set: non-temporal.  A
+// launch writes every output row once and never reads it back, and what the L2s still hold dirty
+// when the last workgroup leaves is written back before the launch counts as finished; streamed
+// stores are on their way to memory while the launch still runs (headline forward, 15 MB of
+// output: 13.2 -> 12.4 us; write-through with sc1 instead: 13.2 us on a box where the plain stores
+// gave 13.8).  The tail is at most the 32 MB the L2s hold, so larger launches gain little and
+// lose the L2's merging of a row's pieces (84 MB of one-byte rows: 57.0 -> 59.2 us; 256 MB: 2 - 3 %
+// slower): the host sets the flag for outputs up to kStreamStoreMaxBytes.  The same hint on the
+// gathered row loads made the headline launch slower (16.4 us), and on the stores of the
+// gather-GEMM-scatter kernel that keeps its weights in registers too (13.4 -> 14.5 us).
+constexpr int kStreamStore = 2;   // aux bit 1 = nt
+constexpr uint32_t kStreamStoreMaxBytes = 32u << 20;
+template <class V>
+__device__ __forceinline__ void store_out_b128(V v, __amdgpu_buffer_rsrc_t rs, uint32_t off, bool stream) {
+  if (stream) __builtin_amdgcn_raw_buffer_store_b128(v, rs, off, 0, kStreamStore);
+  else __builtin_amdgcn_raw_buffer_store_b128(v, rs, off, 0, 0);
+}
+template <class V>
+__device__ __forceinline__ void store_out_b64(V v, __amdgpu_buffer_rsrc_t rs, uint32_t off, bool stream) {
+  if (stream) __builtin_amdgcn_raw_buffer_store_b64(v, rs, off, 0, kStreamStore);
+  else __builtin_amdgcn_raw_buffer_store_b64(v, rs, off, 0, 0);
+}
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
@@ -121,7 +146,7 @@ __device__ __forceinline__ void store_wide_piece(const AccV &a, const RowGemmPar
     }
     outv = __builtin_bit_cast(v4i, of);
   }
-  __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
+  store_out_b128(outv, rs_c, coff, p.stream_stores != 0);
 }
 
 // T: element tag; NW: waves per workgroup; RB: 16-row blocks per wave; TN: output channels per

@@ -680,7 +680,7 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
             t = apply_act(t, ACT, p.act_alpha);
             oh[x] = E::from_float(t);
           }
-          __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
+          store_out_b128(outv, rs_c, coff, p.stream_stores != 0);
         }
       }
     } else {
@@ -715,8 +715,8 @@ __device__ __forceinline__ void rowgemm_lds_tile(const RowGemmParams &p, const i
         }
 #pragma unroll
         for (int g = 0; g < ND; ++g) outv[g] = pack4_bytes(ob[4 * g], ob[4 * g + 1], ob[4 * g + 2], ob[4 * g + 3]);
-        if constexpr (ND == 4) __builtin_amdgcn_raw_buffer_store_b128(outv, rs_c, coff, 0, 0);
-        else __builtin_amdgcn_raw_buffer_store_b64(outv, rs_c, coff, 0, 0);
+        if constexpr (ND == 4) store_out_b128(outv, rs_c, coff, p.stream_stores != 0);
+        else store_out_b64(outv, rs_c, coff, p.stream_stores != 0);
       }
     }
   };
