@@ -81,10 +81,29 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
     }
     return hipErrorInvalidValue;
   }
-  // A contraction longer than 128 bytes: the LDS-streaming kernel with 128-byte stage rows (three
-  // stages fit, three workgroups per CU) walking the contraction in chunks, rather than
-  // 256-byte rows with two stages or the register-gather kernels.
+  // A contraction longer than 128 bytes: the LDS-streaming kernel walking the contraction in
+  // chunks of one stage row, rather than 256-byte rows with two stages or the register-gather
+  // kernels.  Stage rows of 128 bytes where three stages of them fit; for the 128 x 128 tile, whose
+  // 128-byte stages are 32 KB (two stages, two workgroups per CU), rows of 64 bytes: three stages
+  // of 16 KB and three workgroups per CU keep half as much again in flight per CU (C = K = 128
+  // bf16 at 1 M voxels: forward 0.229 -> 0.220 ms, backward-input 0.218 -> 0.194 ms, stride-2
+  // 128 -> 256 forward 0.838 -> 0.751 ms; four stages at two workgroups per CU: no gain; the other
+  // tiles are slower with 64-byte rows).
   if constexpr (KS == 4) {
+    if constexpr (TM == 128 && TN == 128 && lds_stages(TM, TN, 1) == 3 && (!WT || Elem<T>::kBytes == 2)) {
+      constexpr int chunk1 = 4 * 1 * Elem<T>::kPerVec;
+      const int nch = (p.c_in + chunk1 - 1) / chunk1;
+      int shift = 0;
+      while ((1 << shift) < nch) ++shift;
+      if (shift <= 3 && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
+        if (counted_waits_hold<rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 1, 3, WT, kWide>>()) {
+          RowGemmParams q = p;
+          q.chunk_shift = shift;
+          hipLaunchKernelGGL((rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 1, 3, WT, kWide>), grid, dim3(256), 0, s, q);
+          return hipGetLastError();
+        }
+      }
+    }
     constexpr int NS2 = lds_stages(TM, TN, 2);
     if constexpr (NS2 > 0 && (!WT || Elem<T>::kBytes == 2)) {
       constexpr int chunk2 = 4 * 2 * Elem<T>::kPerVec;
