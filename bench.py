@@ -79,6 +79,13 @@ def find_desp(tv_dtype, op, tile_m, tile_n, int8=False, parallel=False, dynamic_
     raise KeyError((tv_dtype, op, tile_m, tile_n, int8, parallel))
 
 
+def tile_key(name):
+    """'128x128' from a descriptor's name, with ' (3 stages)' for the three-stage twin of a tile."""
+    key = "%sx%s" % re.search(r"_m(\d+)n(\d+)k", name).groups()
+    stages = re.search(r"_(\d+)[01][01](?:_|$)", name[name.index("_m"):])
+    return key + (" (3 stages)" if stages and stages.group(1) == "3" else "")
+
+
 def dev(arr):
     return tv.from_numpy(np.ascontiguousarray(arr)).cuda()
 
@@ -179,7 +186,7 @@ def bench_gather_gemm(args):
     w_ms, e_ms = timed(lambda: GemmMainUnitTest.matmul2(pg), args.steps, args.warmup)
     nbytes = m * k * 2 + 2 * m * n * 2 + k * n * 2 + 2 * m * 4
     return {"tile": list(best.desp.tile_shape[:2]),
-            "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
+            "ms_by_tile": {tile_key(nm): round(ms, 5)
                            for nm, ms in best.tried},
             "ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
             "tflops": round(2.0 * m * n * k / (w_ms * 1e-3) / 1e12, 3),
@@ -267,7 +274,7 @@ def bench_stack(args):
         r = tn.tune_conv(p)
         wms, ems = timed(lambda: ConvMainUnitTest.implicit_gemm2(p), steps, warm)
         res[name] = {"tile": list(r.desp.tile_shape[:2]),
-                     "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
+                     "ms_by_tile": {tile_key(nm): round(ms, 5)
                                     for nm, ms in r.tried},
                      "ms_per_step": round(wms, 5), "kernel_ms_events": round(ems, 5),
                      "tflops": round(flops / (wms * 1e-3) / 1e12, 2),
@@ -594,7 +601,7 @@ def bench_s8(args, tile_m):
             "by_value_order_and_row_table": {"tile_m": tile_m, "kernel_ms_events": round(e0_ms, 5),
                                              "hbm_frac": round(bytes4 / (e0_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
             "tile": list(best.desp.tile_shape[:2]),
-            "ms_by_tile": {"%sx%s" % re.search(r"_m(\d+)n(\d+)k", nm).groups(): round(ms, 5)
+            "ms_by_tile": {tile_key(nm): round(ms, 5)
                            for nm, ms in best.tried},
             "ms_per_step": round(w_ms, 5), "kernel_ms_events": round(e_ms, 5),
             "tops": round(ops4 / (w_ms * 1e-3) / 1e12, 3),

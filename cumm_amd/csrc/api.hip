@@ -156,7 +156,7 @@ int conv_family(const CummHipConvDesc &c) {
 }
 
 void fill_gemm_desc(CummHipGemmDesc &d, int dt, int ta, int tb, int tc, int tm, int tn, int shuffle,
-                    int splitk, bool wide = false) {
+                    int splitk, bool wide = false, int num_stage = 2) {
   std::memset(&d, 0, sizeof(d));
   d.dtype_a = d.dtype_b = d.dtype_c = dt;
   d.dacc = dt == CUMM_HIP_S8 ? CUMM_HIP_S32 : CUMM_HIP_F32;
@@ -168,7 +168,7 @@ void fill_gemm_desc(CummHipGemmDesc &d, int dt, int ta, int tb, int tc, int tm, 
   d.trans_a = ta; d.trans_b = tb; d.trans_c = tc;
   const int tk = dt == CUMM_HIP_S8 ? 64 : 32;
   d.tile_shape[0] = tm; d.tile_shape[1] = tn; d.tile_shape[2] = tk;
-  d.num_stage = 2;
+  d.num_stage = num_stage;
   d.shuffle_type = shuffle;
   d.split_k_serial = splitk;
   d.split_k_parallel = 0;
@@ -438,15 +438,21 @@ int cumm_hip_list_conv_algos(CummHipConvDesc *out, int cap) {
   const int fdts[2] = {CUMM_HIP_F16, CUMM_HIP_BF16};
   for (int dt : fdts) {
     for (int wide = 0; wide < 2; ++wide)   // output in the operands' type, then in f32
-    for (auto &t : row_tiles) {
+    for (auto &t : row_tiles)
+    // The 128 x 128 tile comes twice: num_stage 3 walks a contraction of more than 128 bytes in
+    // 64-byte chunks through three stages of 16 KB (three workgroups per CU: faster where most
+    // tiles have few kernel offsets, as in sparse clouds), num_stage 2 in 128-byte chunks through
+    // two stages of 32 KB (half as many steps per offset: faster where tiles have many).  Shorter
+    // contractions fit one chunk either way.  The three-stage one is listed first.
+    for (int stages = (t[0] == 128 && t[1] == 128 ? 3 : 2); stages >= 2; --stages) {
       // forward: A = input [N,C] row major, B = weight [K, kv*C] ("tn"), C = output
       CummHipConvDesc c;
-      fill_gemm_desc(c.gemm, dt, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, wide != 0);
+      fill_gemm_desc(c.gemm, dt, 0, 1, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, wide != 0, stages);
       c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
       base(c, CUMM_HIP_OP_FORWARD);
       v.push_back(c);
       // backward input: A = dOut [N,K], B = weight viewed [kv*K, C] ("tt")
-      fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, wide != 0);
+      fill_gemm_desc(c.gemm, dt, 0, 0, 0, t[0], t[1], CUMM_HIP_NO_SHUFFLE, 0, wide != 0, stages);
       c.gemm.warp_tile_shape[0] = t[0] / 4; c.gemm.warp_tile_shape[1] = t[1]; c.gemm.warp_tile_shape[2] = 32;
       base(c, CUMM_HIP_OP_BACKWARD_INPUT);
       v.push_back(c);
@@ -731,6 +737,7 @@ int sparse_conv_impl(const CummHipConvDesc *desc, const CummHipSparseConvArgs *a
       return fail(CUMM_HIP_ERUNTIME, "your data exceed int32 range.");
     p.gather_bytes = (uint32_t)((int64_t)kv * a->N * 4);
     p.stream_stores = p.c_bytes <= kStreamStoreMaxBytes;
+    p.small_stages = d.num_stage >= 3;
     hipError_t e = launch_rowgemm(dt, wide, d.tile_shape[0], d.tile_shape[1], pick_ks(p.c_in, dt), !fwd, p, stream);
     if (e != hipSuccess) return hip_fail(e, "sparse conv launch");
     return CUMM_HIP_OK;

@@ -77,6 +77,9 @@ struct RowGemmParams {
   int32_t ungated_rows;
   // non-zero: the output rows are stored with the non-temporal hint (see kStreamStore)
   int32_t stream_stores;
+  // non-zero (descriptors with num_stage 3): a contraction of more than 128 bytes is walked in
+  // 64-byte chunks through three stages where the tile has such a kernel (128 x 128)
+  int32_t small_stages;
 };
 
 // An offset no buffer contains: every operand is smaller than 2 GiB (checked on the host), and

@@ -83,19 +83,22 @@ static hipError_t launch_one(const RowGemmParams &p, hipStream_t s) {
   }
   // A contraction longer than 128 bytes: the LDS-streaming kernel walking the contraction in
   // chunks of one stage row, rather than 256-byte rows with two stages or the register-gather
-  // kernels.  Stage rows of 128 bytes where three stages of them fit; for the 128 x 128 tile, whose
-  // 128-byte stages are 32 KB (two stages, two workgroups per CU), rows of 64 bytes: three stages
-  // of 16 KB and three workgroups per CU keep half as much again in flight per CU (C = K = 128
-  // bf16 at 1 M voxels: forward 0.229 -> 0.220 ms, backward-input 0.218 -> 0.194 ms, stride-2
-  // 128 -> 256 forward 0.838 -> 0.751 ms; four stages at two workgroups per CU: no gain; the other
-  // tiles are slower with 64-byte rows).
+  // kernels.  Stage rows of 128 bytes; for the 128 x 128 tile, whose 128-byte stages are 32 KB
+  // (two stages, two workgroups per CU), also rows of 64 bytes when the descriptor asks for three
+  // stages: 16 KB each, three workgroups per CU, half as much again in flight per CU.  Launches
+  // whose tiles have few kernel offsets are bound by the latency of their round trips and gain
+  // (C = K = 128 bf16 at 1 M voxels, 2 pairs per voxel: forward 0.229 -> 0.220 ms, backward-input
+  // 0.218 -> 0.194 ms, stride-2 128 -> 256 forward 0.838 -> 0.751 ms; four stages at two
+  // workgroups per CU: no gain); tiles with many offsets are bound by their steps, and twice the
+  // steps per offset cost them (125 offsets, C = K = 128: 0.239 -> 0.300 ms), as they do the
+  // smaller tiles (64 x 128 at 1 M voxels: 0.258 -> 0.281 ms).
   if constexpr (KS == 4) {
     if constexpr (TM == 128 && TN == 128 && lds_stages(TM, TN, 1) == 3 && (!WT || Elem<T>::kBytes == 2)) {
       constexpr int chunk1 = 4 * 1 * Elem<T>::kPerVec;
       const int nch = (p.c_in + chunk1 - 1) / chunk1;
       int shift = 0;
       while ((1 << shift) < nch) ++shift;
-      if (shift <= 3 && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
+      if (p.small_stages && shift <= 3 && (WT ? p.w_stride_n == 1 : p.w_stride_c == 1)) {
         if (counted_waits_hold<rowgemm_lds_kernel<T, 2, 2, TM / 32, TN / 32, 1, 3, WT, kWide>>()) {
           RowGemmParams q = p;
           q.chunk_shift = shift;

@@ -71,6 +71,11 @@ def conv_candidates(params: ConvParams, desps: Optional[List[ConvAlgoDesp]] = No
             continue
         if not d.supported(mnk[0], mnk[1], mnk[2], C, K, params.mask_width):
             continue
+        # the three-stage twin of a tile differs from it only where the contraction is walked in
+        # chunks (more than 128 bytes per row): elsewhere it would be timed twice
+        contraction = K if op == ConvOpType.BackwardInput else C
+        if d.num_stage >= 3 and contraction * params.input.itemsize <= 128:
+            continue
         res.append(d)
     return res
 

@@ -51,7 +51,10 @@ extern "C" {
 #define CUMM_HIP_ACT_LEAKY_RELU 3
 
 /* The fields of tv::gemm::GemmAlgoDesp that select a kernel
- * (include/tensorview/gemm/core/params.h:24-54). */
+ * (include/tensorview/gemm/core/params.h:24-54).  num_stage is 2 except for the second descriptor of
+ * the 128 x 128 forward / backward-input tile (f16, bf16), where 3 selects three small stages for
+ * contractions of more than 128 bytes per row: same results to the bit, faster where tiles have
+ * few kernel offsets, slower where they have many - a choice for the caller's tuner. */
 typedef struct CummHipGemmDesc {
   int32_t dtype_a, dtype_b, dtype_c, dacc, dcomp;
   int32_t trans_a, trans_b, trans_c;

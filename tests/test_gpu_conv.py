@@ -788,6 +788,63 @@ def test_long_contraction_forward_and_backward_input(dtype):
     assert H.rel_err(H.as_f32(H.host(q.input), dtype), H.as_f32(ref_d, dtype)) < TOL
 
 
+def _desps_128(dtype, op):
+    """Both descriptors of the 128 x 128 tile: three stages of 64-byte chunks, two of 128-byte chunks."""
+    found = {}
+    for d in ConvMainUnitTest.get_all_conv_algo_desp():
+        if (d.dtype_a == H.TV_DTYPE[dtype] and d.dtype_output == H.TV_DTYPE[dtype] and
+                d.dtype_input == H.TV_DTYPE[dtype] and ConvOpType(d.op_type) == op and
+                tuple(d.tile_shape[:2]) == (128, 128) and not d.dynamic_mask and not d.is_int8_inference):
+            found[d.num_stage] = d
+    assert sorted(found) == [2, 3]
+    return found
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("c_in,k_out", [(128, 128), (96, 256), (160, 72), (256, 128)])
+def test_both_stage_counts_of_the_128_tile(dtype, c_in, k_out):
+    """Contractions of more than 128 bytes through both descriptors of the 128 x 128 tile, forward
+    and backward-input (strided table, so the two passes differ): each against the oracle, and
+    the same bits from both (the products are added in the same order, chunk by chunk)."""
+    print("case both stage counts", dtype, c_in, k_out, flush=True)
+    rng, coords, pt, feat, w, n_in, n_out = _case(31, 2500, c_in, k_out, dtype, strided=True)
+    ms, order = pairs.sort_by_mask(pt.mask_fwd)
+    out0 = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    ref, ref_mo = conv_ref.implicit_gemm_fwd_ref(feat, w, out0, pt.indices_fwd, ms, order, tile_m=128, dtype_in=dtype,
+                                                 dtype_w=dtype, dtype_out=dtype, beta=1.0)
+    got = {}
+    for stages, desp in _desps_128(dtype, ConvOpType.Forward).items():
+        p = ConvParams(3, ConvOpType.Forward)
+        p.conv_algo_desp = desp
+        p.input, p.weight, p.output = H.dev(feat, dtype), H.dev(w, dtype), H.dev(out0, dtype)
+        p.indices = H.dev(pt.indices_fwd, "i32")
+        p.mask, p.mask_argsort = H.dev(ms, "u32"), H.dev(order, "i32")
+        p.mask_output = tv.zeros([(n_out + 127) // 128], tv.uint32, 0)
+        p.mask_width = 128
+        p.beta = 1.0
+        ConvMainUnitTest.implicit_gemm2(p)
+        got[stages] = H.host(p.output)
+        assert H.rel_err_rows(H.as_f32(got[stages], dtype), H.as_f32(ref, dtype)) < TOL, stages
+        np.testing.assert_array_equal(H.host(p.mask_output), ref_mo)
+    np.testing.assert_array_equal(got[2], got[3])
+    msb, orderb = pairs.sort_by_mask(pt.mask_bwd)
+    dout = H.to_storage(rng.normal(0, 1, size=(n_out, k_out)).astype(np.float32), dtype)
+    din0 = H.to_storage(np.zeros((n_in, c_in), np.float32), dtype)
+    ref_d = conv_ref.implicit_gemm_dgrad_ref(dout, w, din0, pt.indices_bwd, msb, orderb, tile_m=128, dtype_in=dtype,
+                                             dtype_w=dtype, dtype_out=dtype)
+    got = {}
+    for stages, desp in _desps_128(dtype, ConvOpType.BackwardInput).items():
+        q = ConvParams(3, ConvOpType.BackwardInput)
+        q.conv_algo_desp = desp
+        q.input, q.weight, q.output = H.dev(din0, dtype), H.dev(w, dtype), H.dev(dout, dtype)
+        q.indices = H.dev(pt.indices_bwd, "i32")
+        q.mask, q.mask_argsort = H.dev(msb, "u32"), H.dev(orderb, "i32")
+        ConvMainUnitTest.implicit_gemm2(q)
+        got[stages] = H.host(q.input)
+        assert H.rel_err_rows(H.as_f32(got[stages], dtype), H.as_f32(ref_d, dtype)) < TOL, stages
+    np.testing.assert_array_equal(got[2], got[3])
+
+
 @pytest.mark.parametrize("dtype,tile", [("f16", (64, 64)), ("bf16", (128, 128)), ("s8", (64, 128))])
 def test_mask_bit_clear_over_a_valid_entry(dtype, tile):
     """Where this library narrows the reference's mask contract, as a tested fact.  The reference

@@ -31,6 +31,13 @@ def test_conv_candidates_share_the_kind_and_accept_the_problem():
                not d.is_int8_inference for d in cands)
     # channels that are not a multiple of the access width: nothing supports them
     assert tuner.conv_candidates(_host_conv_params(ConvOpType.Forward, "f16", 60, 64)) == []
+    # a contraction of more than 128 bytes: the 128 x 128 tile is a candidate with two and with three stages
+    long_c = tuner.conv_candidates(_host_conv_params(ConvOpType.Forward, "f16", 128, 64))
+    assert sorted(d.num_stage for d in long_c if tuple(d.tile_shape[:2]) == (128, 128)) == [2, 3]
+    assert all(d.num_stage == 2 for d in long_c if tuple(d.tile_shape[:2]) != (128, 128))
+    # (backward-input contracts over the output channels)
+    long_k = tuner.conv_candidates(_host_conv_params(ConvOpType.BackwardInput, "f16", 64, 128))
+    assert sorted(d.num_stage for d in long_k if tuple(d.tile_shape[:2]) == (128, 128)) == [2, 3]
     # int8 inference descriptors stay among themselves
     s8 = tuner.conv_candidates(_host_conv_params(ConvOpType.Forward, "s8", 64, 128))
     assert s8 and all(d.is_int8_inference and d.dtype_a == tv.int8 for d in s8)
